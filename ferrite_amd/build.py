@@ -1,0 +1,55 @@
+"""Builds libferrite_amd.so in-tree: the gfx950 code objects (hipcc --genco), linked into the host library as data.
+
+    python -m ferrite_amd.build        # compile everything
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+KERN = os.path.join(CSRC, "kernels")
+OUT = os.path.join(HERE, "_build")
+LIB = os.path.join(HERE, "libferrite_amd.so")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.path.join(ROCM, "bin", "hipcc")
+
+# -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from the float code in these kernels
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-mcode-object-version=5",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+KERNELS = ["k_exl3", "k_fp4"]
+HOST = ["fe_hip.cpp", "fe_exl3.cpp", "fe_fp4.cpp"]
+
+
+def _run(cmd, **kw):
+    r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, **kw)
+    if r.returncode:
+        sys.stderr.write(" ".join(cmd) + "\n" + r.stdout)
+        raise RuntimeError(f"build step failed: {cmd[0]} ... {cmd[-1]}")
+    return r.stdout
+
+
+def build(verbose: bool = False) -> str:
+    os.makedirs(OUT, exist_ok=True)
+    for k in KERNELS:
+        _run([HIPCC, "--genco", "--no-gpu-bundle-output", *DEVICE_FLAGS, "-I", KERN, os.path.join(KERN, k + ".hip"), "-o", os.path.join(OUT, k + ".hsaco")])
+    # the code objects become .rodata of the library (.incbin resolves against the working directory)
+    _run(["gcc", "-c", os.path.join(CSRC, "fe_embed.S"), "-o", os.path.join(OUT, "fe_embed.o")], cwd=OUT)
+    objs = [os.path.join(OUT, "fe_embed.o")]
+    inc = ["-I", os.path.join(os.path.dirname(HERE), "include"), "-I", CSRC, "-I", os.path.join(ROCM, "include")]
+    for src in HOST:
+        o = os.path.join(OUT, src.replace(".cpp", ".o"))
+        _run(["g++", "-c", "-O2", "-fPIC", "-std=c++17", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", *inc,
+              os.path.join(CSRC, src), "-o", o])
+        objs.append(o)
+    _run(["g++", "-shared", "-o", LIB, *objs, "-L", os.path.join(ROCM, "lib"), "-lamdhip64",
+          "-Wl,-rpath," + os.path.join(ROCM, "lib"), "-Wl,--no-undefined"])
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(verbose=True)

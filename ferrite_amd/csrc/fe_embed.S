@@ -1,0 +1,16 @@
+/* The gfx950 code objects, linked into the library as read-only data (the reference embeds its cubins with
+ * include_bytes!, crates/fe-exl3/src/gpu/mod.rs:12-13). Paths are relative to the build directory. */
+    .section .rodata
+    .balign 4096
+    .global fe_k_exl3_hsaco
+fe_k_exl3_hsaco:
+    .incbin "k_exl3.hsaco"
+    .global fe_k_exl3_hsaco_end
+fe_k_exl3_hsaco_end:
+    .balign 4096
+    .global fe_k_fp4_hsaco
+fe_k_fp4_hsaco:
+    .incbin "k_fp4.hsaco"
+    .global fe_k_fp4_hsaco_end
+fe_k_fp4_hsaco_end:
+    .section .note.GNU-stack,"",@progbits

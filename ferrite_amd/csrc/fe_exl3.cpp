@@ -1,0 +1,439 @@
+// fe_exl3: host side of the EXL3 linear (see include/fe_exl3.h). Launch geometry, workspaces and argument checks
+// follow crates/fe-exl3/src/linear.rs and crates/fe-exl3/src/gpu/mod.rs; the kernels are ferrite_amd/csrc/kernels/k_exl3.hip.
+#include "fe_exl3.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "fe_internal.h"
+
+namespace {
+
+constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
+constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
+constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
+constexpr uint32_t kGemmLds = 128 * 132 * 4;  // epilogue tile of the prefill GEMM (covers the A/B tiles too)
+
+bool env_is(const char *name, const char *v) {
+    const char *e = getenv(name);
+    return e && strcmp(e, v) == 0;
+}
+
+const int kBits[] = {2, 3, 4, 5, 6, 8};
+
+int bits_slot(uint32_t bits) {
+    for (int i = 0; i < 6; i++)
+        if ((uint32_t)kBits[i] == bits) return i;
+    return -1;
+}
+
+}  // namespace
+
+struct fe_exl3_kernels {
+    fe_module_t module = nullptr;
+    fe_function_t recon_hat_f32 = nullptr, recon_hat_f16 = nullptr, had_rows = nullptr, had_cols_bf16 = nullptr;
+    fe_function_t rot_in = nullptr, probe_v4 = nullptr;
+    fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
+    fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
+    fe_function_t gemm[6] = {};
+    uint32_t group_m = 8;
+};
+
+struct fe_exl3_linear {
+    std::string name;
+    uint32_t k = 0, n = 0, bits = 0;
+    fe_exl3_plan plan{};
+    fe_exl3_view view{};
+    FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
+    const fe_exl3_kernels *kern = nullptr;
+};
+
+struct fe_exl3_workspace {
+    uint32_t max_rows = 0, max_k = 0;
+    FeBuf xh, z, counters;
+    size_t z_len = 0, counters_len = 0;
+};
+
+int fe_load_module(fe_module_t *out, const char *env, const unsigned char *begin, const unsigned char *end) {
+    const char *path = getenv(env);
+    if (path && *path) return fe_hip_module_load_file(out, path);
+    return fe_hip_module_load(out, begin, (size_t)(end - begin));
+}
+
+// (words between k steps, words between 128-column blocks), crates/fe-exl3/src/gpu/mod.rs:28-33
+static void view_strides(const fe_exl3_view &v, uint32_t *stride_k, uint32_t *stride_nb) {
+    uint32_t tw = 8 * v.bits;
+    if (v.strips) {
+        *stride_k = 8 * tw;
+        *stride_nb = v.k / 16 * 8 * tw;
+    } else {
+        *stride_k = v.n / 16 * tw;
+        *stride_nb = 8 * tw;
+    }
+}
+
+extern "C" {
+
+int fe_exl3_kernels_load(fe_exl3_kernels **out) {
+    if (!out) return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_load", "null out");
+    auto *k = new fe_exl3_kernels;
+    int c = fe_load_module(&k->module, "FE_EXL3_HSACO", fe_k_exl3_hsaco, fe_k_exl3_hsaco_end);
+    auto get = [&](fe_function_t *f, const char *name) {
+        if (!c) c = fe_hip_module_get_function(f, k->module, name);
+    };
+    get(&k->recon_hat_f32, "exl3_recon_hat_f32");
+    get(&k->recon_hat_f16, "exl3_recon_hat_f16");
+    get(&k->had_rows, "exl3_had_rows");
+    get(&k->had_cols_bf16, "exl3_had_cols_bf16");
+    get(&k->rot_in, "exl3_rot_in");
+    get(&k->probe_v4, "exl3_probe_v4");
+    for (int b = 3; b <= 5; b++) {
+        char nm[64];
+        snprintf(nm, sizeof nm, "exl3_probe_decode_b%d", b);
+        get(&k->probe_decode[b - 3], nm);
+    }
+    for (int i = 0; i < 6; i++) {
+        char nm[64];
+        for (int rg = 1; rg <= 4; rg++) {
+            snprintf(nm, sizeof nm, "exl3_gemv_b%d_r%d", kBits[i], rg);
+            get(&k->gemv[i][rg - 1], nm);
+            if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv[i][rg - 1], 64 * 1024);
+        }
+        snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
+        get(&k->gemm[i], nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
+    }
+    if (const char *g = getenv("FE_EXL3_GROUP")) k->group_m = (uint32_t)atoi(g);
+    if (c) {
+        fe_exl3_kernels_destroy(k);
+        return c;
+    }
+    *out = k;
+    return 0;
+}
+
+int fe_exl3_kernels_destroy(fe_exl3_kernels *k) {
+    if (!k) return 0;
+    if (k->module) fe_hip_module_unload(k->module);
+    delete k;
+    return 0;
+}
+
+// K splits for `blocks` programs: the smallest divisor of the load-step count that reaches the target, backing off
+// while a program would get fewer than min_steps load steps (the role of tf_plan, crates/fe-exl3/src/linear.rs:100-129;
+// one load step = 4 k steps = 64 input channels).
+int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_exl3_plan *out) {
+    (void)bits;
+    if (!out || !k || !n || k % 128 || n % 128) return fe_set_error(FE_ERR_SHAPE, "fe_exl3_plan_for", "k, n must be multiples of 128");
+    const uint32_t steps = k / 64, nb = n / 128, min_steps = 2;
+    uint32_t sk = 1;
+    for (uint32_t d = 1; d <= steps; d++) {
+        if (steps % d) continue;
+        if (steps / d < min_steps) break;
+        sk = d;
+        if (nb * d >= blocks) break;
+    }
+    if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) sk = 1;
+    *out = fe_exl3_plan{sk, 4, 1, 0};
+    return 0;
+}
+
+int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out) {
+    if (!s || !out) return fe_set_error(FE_ERR_ARG, "fe_exl3_plan_parse", "null");
+    unsigned v[4] = {0, 0, 1, 0};
+    int got = sscanf(s, " %u , %u , %u , %u", &v[0], &v[1], &v[2], &v[3]);
+    if (got < 2) return fe_set_error(FE_ERR_ARG, "fe_exl3_plan_parse", s);
+    *out = fe_exl3_plan{v[0], v[1], v[2], v[3]};
+    return 0;
+}
+
+static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, const fe_exl3_plan &p) {
+    char msg[160];
+    if (bits_slot(bits) < 0) {
+        snprintf(msg, sizeof msg, "%s: %u bits (kernels exist for 2, 3, 4, 5, 6, 8)", name, bits);
+        return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear", msg);
+    }
+    // linear.rs:244: k, n multiples of 128 and the K range divides into the plan's pieces (here: load steps of 64)
+    if (!k || !n || k % 128 || n % 128 || p.sk == 0 || (k / 64) % p.sk) {
+        snprintf(msg, sizeof msg, "%s: %ux%u does not fit plan sk %u", name, k, n, p.sk);
+        return fe_set_error(FE_ERR_SHAPE, "fe_exl3_linear", msg);
+    }
+    return 0;
+}
+
+int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, const char *name, const fe_exl3_view *view,
+                             const fe_exl3_plan *plan) {
+    if (!out || !kern || !view || !plan) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_from_view", "null argument");
+    FE_TRY(check_fit(name ? name : "?", view->k, view->n, view->bits, *plan));
+    auto *l = new fe_exl3_linear;
+    l->name = name ? name : "";
+    l->k = view->k, l->n = view->n, l->bits = view->bits;
+    l->plan = *plan;
+    l->view = *view;
+    l->kern = kern;
+    *out = l;
+    return 0;
+}
+
+int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, const char *name, uint32_t k, uint32_t n,
+                          uint32_t bits, const uint32_t *trellis, const uint16_t *suh, const uint16_t *svh, int strips,
+                          const fe_exl3_plan *plan, uint32_t blocks) {
+    if (!out || !kern || !trellis || !suh || !svh) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_upload", "null argument");
+    fe_exl3_plan p;
+    if (plan)
+        p = *plan;
+    else
+        FE_TRY(fe_exl3_plan_for(k, n, bits, blocks, &p));
+    FE_TRY(check_fit(name ? name : "?", k, n, bits, p));
+    auto *l = new fe_exl3_linear;
+    l->name = name ? name : "";
+    l->k = k, l->n = n, l->bits = bits, l->plan = p, l->kern = kern;
+    const size_t tw = 8 * (size_t)bits, kt = k / 16, nt = n / 16, words = kt * nt * tw;
+    int c = 0;
+    if (strips) {
+        // [n/128][k/16][8][tw] (Exl3Tensor::strips, crates/fe-exl3/src/format.rs:70-84)
+        std::vector<uint32_t> st(words);
+        for (size_t b = 0; b < nt / 8; b++)
+            for (size_t t = 0; t < kt; t++)
+                memcpy(&st[(b * kt + t) * 8 * tw], &trellis[(t * nt + b * 8) * tw], 8 * tw * sizeof(uint32_t));
+        c = l->trellis.from_host(st.data(), words * 4);
+    } else {
+        c = l->trellis.from_host(trellis, words * 4);
+    }
+    if (!c) c = l->suh.from_host(suh, (size_t)k * 2);
+    if (!c) c = l->svh.from_host(svh, (size_t)n * 2);
+    if (c) {
+        delete l;
+        return c;
+    }
+    l->view = fe_exl3_view{k, n, bits, l->trellis.p, l->suh.p, l->svh.p, strips ? 1u : 0u};
+    *out = l;
+    return 0;
+}
+
+int fe_exl3_linear_destroy(fe_exl3_linear *l) {
+    delete l;
+    return 0;
+}
+
+int fe_exl3_linear_view(const fe_exl3_linear *l, fe_exl3_view *view, fe_exl3_plan *plan) {
+    if (!l) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_view", "null linear");
+    if (view) *view = l->view;
+    if (plan) *plan = l->plan;
+    return 0;
+}
+
+size_t fe_exl3_linear_weight_bytes(const fe_exl3_linear *l) { return l ? (size_t)l->k * l->n * l->bits / 8 : 0; }
+
+int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows) {
+    if (!out || (count && !linears) || !max_rows) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_create", "bad argument");
+    size_t max_k = 128, max_z = 0, max_nb = 1;
+    for (size_t i = 0; i < count; i++) {
+        const fe_exl3_linear *l = linears[i];
+        max_k = std::max<size_t>(max_k, l->k);
+        if (l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
+        max_nb = std::max<size_t>(max_nb, l->n / 128);
+    }
+    auto *ws = new fe_exl3_workspace;
+    ws->max_rows = max_rows, ws->max_k = (uint32_t)max_k;
+    ws->z_len = std::max<size_t>(max_z * std::min(max_rows, kMaxRowsPerPass), 4);
+    ws->counters_len = (size_t)((max_rows + 7) / 8) * max_nb;
+    int c = ws->xh.alloc((size_t)max_rows * max_k * 2);
+    if (!c) c = ws->z.alloc(ws->z_len * 4);
+    if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
+    if (c) {
+        delete ws;
+        return c;
+    }
+    *out = ws;
+    return 0;
+}
+
+int fe_exl3_workspace_destroy(fe_exl3_workspace *ws) {
+    delete ws;
+    return 0;
+}
+
+int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t *max_rows, uint32_t *max_k) {
+    if (!ws) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_xh", "null workspace");
+    if (xh) *xh = ws->xh.p;
+    if (max_rows) *max_rows = ws->max_rows;
+    if (max_k) *max_k = ws->max_k;
+    return 0;
+}
+
+int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
+                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "null argument");
+    if (rows == 0 || rows > ws->max_rows || l->k > ws->max_k) {
+        char msg[160];
+        snprintf(msg, sizeof msg, "%s: rows %u (workspace %u x %u)", l->name.c_str(), rows, ws->max_rows, ws->max_k);
+        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_rotate_input", msg);
+    }
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "x is bf16 or f32");
+    uint32_t x_f32 = (uint32_t)x_dtype & 1, k = l->k;
+    fe_devptr_t suh = l->view.suh, xh = ws->xh.p;
+    void *args[] = {&x, &x_f32, &suh, &xh, &k};
+    return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
+}
+
+static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows) {
+    const fe_exl3_kernels *kern = l->kern;
+    uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb, group = kern->group_m;
+    view_strides(l->view, &stride_k, &stride_nb);
+    uint32_t tiles_m = (rows + 127) / 128;
+    if (group == 0 || group > tiles_m) group = tiles_m;
+    fe_devptr_t tr = l->view.trellis, svh = l->view.svh;
+    void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group};
+    return fe_hip_launch(kern->gemm[bits_slot(l->bits)], tiles_m * (n / 128), 1, 1, 256, 1, 1, kGemmLds, s, args);
+}
+
+int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
+                                uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "null argument");
+    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "bad y dtype");
+    const fe_exl3_plan &p = l->plan;
+    char msg[200];
+    if (rows > kMaxRowsPerPass) {
+        if (rows > ws->max_rows) {
+            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
+            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
+        }
+        return launch_gemm(l, s, xh, y, y_dtype, rows);
+    }
+    // linear.rs:302-307
+    if (rows == 0 || rows > ws->max_rows || (p.sk > 1 && ws->z_len < (size_t)p.sk * rows * l->n)) {
+        snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u, z %zu)", l->name.c_str(), rows, ws->max_rows,
+                 ws->z_len);
+        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
+    }
+    if (ws->counters_len < (size_t)((rows + 7) / 8) * (l->n / 128)) {
+        snprintf(msg, sizeof msg, "%s: workspace counters too small for %u rows", l->name.c_str(), rows);
+        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
+    }
+    const uint32_t rg = (rows + 15) / 16;
+    const uint32_t steps = l->k / 64 / p.sk;
+    // staged input chunk: as many load steps as the LDS budget holds for `rows` rows, a multiple of 4
+    uint32_t chunk = (kLdsBudget / rows - 16) / 128 / 4 * 4;
+    chunk = std::max(chunk, 4u);
+    chunk = std::min(chunk, (steps + 3) / 4 * 4);
+    const uint32_t lds = std::max(rows * (chunk * 128 + 16), rows * kRedPitch * 4);
+    uint32_t n = l->n, k = l->k, sk = p.sk, mode = (uint32_t)y_dtype, stride_k, stride_nb;
+    view_strides(l->view, &stride_k, &stride_nb);
+    fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
+    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk};
+    return fe_hip_launch(l->kern->gemv[bits_slot(l->bits)][rg - 1], n / 128 * sk, 1, 1, 256, 1, 1, lds, s, args);
+}
+
+int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    FE_TRY(fe_exl3_linear_rotate_input(l, kern, s, x, x_dtype, rows, ws));
+    return fe_exl3_linear_gemv_rotated(l, s, ws->xh.p, y, y_dtype, rows, ws);
+}
+
+int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out) {
+    if (!kern || !w || !out) return fe_set_error(FE_ERR_ARG, "fe_exl3_reconstruct_hat_f16", "null argument");
+    if (w->strips || w->k % 16 || w->n % 128 || w->bits < 1 || w->bits > 8)
+        return fe_set_error(FE_ERR_SHAPE, "fe_exl3_reconstruct_hat_f16", "needs the stored layout, n % 128 == 0, 1..8 bits");
+    uint32_t n_tiles = w->n / 16, nt0 = 0, ns = w->n, bits = w->bits;
+    fe_devptr_t tr = w->trellis;
+    void *args[] = {&out, &tr, &n_tiles, &nt0, &ns, &bits};
+    return fe_hip_launch(kern->recon_hat_f16, w->n / 128, w->k / 16, 1, 256, 1, 1, 0, s, args);
+}
+
+int fe_exl3_reconstruct_bf16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out, int layout,
+                             fe_devptr_t scratch, size_t scratch_bytes) {
+    if (!kern || !w || !out || !scratch) return fe_set_error(FE_ERR_ARG, "fe_exl3_reconstruct_bf16", "null argument");
+    const size_t k = w->k, n = w->n;
+    if (k % 128 || n % 128 || w->strips || w->bits < 1 || w->bits > 8)
+        return fe_set_error(FE_ERR_SHAPE, "fe_exl3_reconstruct_bf16", "not 128-aligned, or strips layout");
+    const size_t max_ns = (scratch_bytes / (k * 4)) / 128 * 128;
+    if (max_ns == 0) return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_reconstruct_bf16", "scratch smaller than k * 128 * 4 bytes");
+    uint32_t ld = layout ? (uint32_t)k : (uint32_t)n, nk = layout ? 1u : 0u;
+    for (size_t n0 = 0; n0 < n;) {
+        uint32_t ns = (uint32_t)std::min(max_ns, n - n0), n032 = (uint32_t)n0, nt0 = n032 / 16, n_tiles = (uint32_t)n / 16;
+        uint32_t bits = w->bits;
+        fe_devptr_t tr = w->trellis, svh = w->svh, suh = w->suh;
+        {
+            void *args[] = {&scratch, &tr, &n_tiles, &nt0, &ns, &bits};
+            FE_TRY(fe_hip_launch(kern->recon_hat_f32, ns / 128, (uint32_t)k / 16, 1, 256, 1, 1, 0, s, args));
+        }
+        {
+            void *args[] = {&scratch, &ns, &svh, &n032};
+            FE_TRY(fe_hip_launch(kern->had_rows, (ns / 128 + 1) / 2, (uint32_t)k, 1, 64, 1, 1, 0, s, args));
+        }
+        {
+            void *args[] = {&scratch, &out, &ns, &suh, &n032, &ld, &nk};
+            FE_TRY(fe_hip_launch(kern->had_cols_bf16, ns / 32, (uint32_t)k / 128, 1, 128, 1, 1, 0, s, args));
+        }
+        n0 += ns;
+    }
+    return 0;
+}
+
+static int time_launches(fe_stream_t s, uint32_t launches, float *ms, int (*launch)(void *), void *ctx) {
+    fe_event_t a = nullptr, b = nullptr;
+    FE_TRY(fe_hip_event_create(&a));
+    int c = fe_hip_event_create(&b);
+    if (!c) c = launch(ctx);  // warm-up
+    if (!c) c = fe_hip_event_record(a, s);
+    for (uint32_t i = 0; !c && i < launches; i++) c = launch(ctx);
+    if (!c) c = fe_hip_event_record(b, s);
+    if (!c) c = fe_hip_event_sync(b);
+    float t = 0;
+    if (!c) c = fe_hip_event_elapsed_ms(&t, a, b);
+    fe_hip_event_destroy(a);
+    fe_hip_event_destroy(b);
+    if (!c && ms) *ms = t / (float)launches;
+    return c;
+}
+
+int fe_exl3_probe_stream_read(const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t buf, size_t bytes, uint32_t grid,
+                              uint32_t launches, float *ms) {
+    if (!kern || !buf || !grid || !launches || bytes < 16) return fe_set_error(FE_ERR_ARG, "fe_exl3_probe_stream_read", "bad argument");
+    struct Ctx {
+        const fe_exl3_kernels *k;
+        fe_stream_t s;
+        fe_devptr_t buf, out;
+        uint64_t vecs;
+        uint32_t grid;
+    } ctx{kern, s, buf, 0, bytes / 16, grid};
+    FeBuf out;
+    FE_TRY(out.zeroed(64));
+    ctx.out = out.p;
+    return time_launches(s, launches, ms,
+                         [](void *p) {
+                             Ctx *c = (Ctx *)p;
+                             void *args[] = {&c->buf, &c->out, &c->vecs};
+                             return fe_hip_launch(c->k->probe_v4, c->grid, 1, 1, 256, 1, 1, 0, c->s, args);
+                         },
+                         &ctx);
+}
+
+int fe_exl3_probe_decode(const fe_exl3_kernels *kern, fe_stream_t s, uint32_t bits, uint32_t grid, uint32_t iters,
+                         uint32_t launches, float *ms) {
+    if (!kern || bits < 3 || bits > 5 || !grid || !launches) return fe_set_error(FE_ERR_ARG, "fe_exl3_probe_decode", "bits 3..5");
+    struct Ctx {
+        const fe_exl3_kernels *k;
+        fe_stream_t s;
+        fe_devptr_t out;
+        uint32_t bits, grid, iters, seed;
+    } ctx{kern, s, 0, bits, grid, iters, 12345u};
+    FeBuf out;
+    FE_TRY(out.zeroed((size_t)grid * 256 * 4));
+    ctx.out = out.p;
+    return time_launches(s, launches, ms,
+                         [](void *p) {
+                             Ctx *c = (Ctx *)p;
+                             void *args[] = {&c->out, &c->iters, &c->seed};
+                             return fe_hip_launch(c->k->probe_decode[c->bits - 3], c->grid, 1, 1, 256, 1, 1, 0, c->s, args);
+                         },
+                         &ctx);
+}
+
+}  // extern "C"

@@ -1,0 +1,64 @@
+// Shared by the host-side sources of libferrite_amd: error plumbing, device buffers, embedded code objects.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+
+#include "fe_hip.h"
+
+int fe_set_error(int code, const char *call, const char *detail);
+int fe_check_hip(int code, const char *call);
+
+#define FE_TRY(x)            \
+    do {                     \
+        int _c = (x);        \
+        if (_c) return _c;   \
+    } while (0)
+
+// gfx950 code objects linked into the library (fe_embed.S)
+extern "C" const unsigned char fe_k_exl3_hsaco[];
+extern "C" const unsigned char fe_k_exl3_hsaco_end[];
+extern "C" const unsigned char fe_k_fp4_hsaco[];
+extern "C" const unsigned char fe_k_fp4_hsaco_end[];
+
+// The embedded image, or the file the environment variable names.
+int fe_load_module(fe_module_t *out, const char *env, const unsigned char *begin, const unsigned char *end);
+
+// Device memory owned until destruction, or a borrowed view (DeviceBuffer / DeviceBuffer::view,
+// crates/fe-cuda/src/lib.rs:201-297).
+struct FeBuf {
+    fe_devptr_t p = 0;
+    size_t bytes = 0;
+    bool owned = false;
+    FeBuf() = default;
+    FeBuf(const FeBuf &) = delete;
+    FeBuf &operator=(const FeBuf &) = delete;
+    ~FeBuf() { release(); }
+    int alloc(size_t n) {
+        release();
+        FE_TRY(fe_hip_malloc(&p, n));
+        bytes = n;
+        owned = true;
+        return 0;
+    }
+    int zeroed(size_t n) {
+        FE_TRY(alloc(n));
+        FE_TRY(fe_hip_memset_d8(p, 0, n, nullptr));
+        return fe_hip_synchronize();
+    }
+    int from_host(const void *src, size_t n) {
+        FE_TRY(alloc(n));
+        return fe_hip_memcpy_htod(p, src, n);
+    }
+    void view(fe_devptr_t q, size_t n) {
+        release();
+        p = q;
+        bytes = n;
+        owned = false;
+    }
+    void release() {
+        if (owned && p) fe_hip_free(p);
+        p = 0;
+        bytes = 0;
+        owned = false;
+    }
+};

@@ -1,0 +1,600 @@
+// EXL3 (trellis-coded, Hadamard-rotated) linear for gfx950: input rotation, the decode GEMV for 1..64 rows,
+// whole-tensor reconstruct, and probes.
+//
+// The trellis of a 16x16 tile is a cyclic stream of 256 * BITS bits, most significant bit of each u32 first; position t
+// owns the 16-bit state ending at stream bit (t + 1) * BITS (crates/fe-exl3/src/cpu.rs:12-23). Position
+// t = 8 * f + i sits at row k = 2 (f & 3) + (i & 1) + 8 ((i >> 1) & 1), column n = (f >> 2) + 8 (i >> 2) of the tile
+// (crates/fe-exl3/src/format.rs:146-156). A state decodes to fp16 by the mul1 codebook
+// (crates/fe-exl3/src/cpu.rs:25-43, kernels/k-exl3/src/util.rs:76-85).
+#include "gemm_core.h"
+
+// ---- the mul1 codebook ------------------------------------------------------------------------------------------
+
+#define MUL1_LO 0xD12Du
+#define MUL1_HI 0x83DCu
+
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+// x = state * 0x83DCD12D mod 2^32 for the 16-bit state in the low (HI = 0) or high (HI = 1) half of r; the other half
+// of r may hold anything. Two full-rate instructions: a packed 16-bit multiply whose low lane is multiplied by zero
+// gives (state * 0x83DC) << 16, and a 16 x 16 + 32 multiply-add supplies state * 0xD12D.
+template <int HI>
+__device__ __forceinline__ uint32_t mul1_x(uint32_t r) {
+    u16x2 rv = __builtin_bit_cast(u16x2, r);
+    uint16_t s = HI ? rv.y : rv.x;
+    u16x2 ss = {s, s};
+    u16x2 kk = {0, MUL1_HI};
+    uint32_t t = __builtin_bit_cast(uint32_t, (u16x2)(ss * kk));
+    uint32_t x;
+    const uint32_t mlo = MUL1_LO;
+    if (HI)
+        asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,0,0,0]" : "=v"(x) : "v"(r), "s"(mlo), "v"(t));
+    else
+        asm("v_mad_u32_u16 %0, %1, %2, %3" : "=v"(x) : "v"(r), "s"(mlo), "v"(t));
+    return x;
+}
+
+// Two codebook values as packed fp16 (x0's in the low half): 0x6400 + byte sum is fp16(1024 + sum); one fused
+// fp16 multiply-add by 0x1eee with 0xc931 added, a single rounding per value.
+__device__ __forceinline__ uint32_t mul1_finish2(uint32_t x0, uint32_t x1) {
+    uint32_t h = __builtin_amdgcn_sad_u8(x0, 0u, 0x64006400u);
+    h = __builtin_amdgcn_sad_hi_u8(x1, 0u, h);
+    f16x2 v = __builtin_bit_cast(f16x2, h);
+    const f16x2 c1 = __builtin_bit_cast(f16x2, 0x1eee1eeeu);
+    const f16x2 c2 = __builtin_bit_cast(f16x2, 0xc931c931u);
+    f16x2 o = __builtin_elementwise_fma(v, c1, c2);
+    return __builtin_bit_cast(uint32_t, o);
+}
+
+__device__ __forceinline__ uint32_t decode2_mul1(uint32_t s0, uint32_t s1) {
+    return mul1_finish2(mul1_x<0>(s0), mul1_x<0>(s1));
+}
+
+// ---- whole-tensor reconstruct (bits at run time: load-time code) ---------------------------------------------------
+
+// 16-bit state of position p of a tile: two words and a funnel shift (kernels/k-exl3/src/recon.rs:12-22).
+__device__ __forceinline__ uint32_t tile_state_rt(const uint32_t* tile, uint32_t bits, uint32_t p) {
+    uint32_t words = 8 * bits;
+    uint32_t b1 = (p + 1) * bits + 256 * bits;
+    uint32_t b0 = b1 - 16;
+    uint32_t i0 = b0 / 32, i1 = (b1 - 1) / 32;
+    uint32_t s = (i1 + 1) * 32 - b1;
+    uint32_t a = tile[i0 % words], b = tile[i1 % words];
+    return (uint32_t)((((uint64_t)a << 32) | b) >> s) & 0xffff;
+}
+
+// W_hat (rotated basis) of columns nt0 * 16 .. + ns: grid (ns / 128, k / 16), 256 threads; half-wavefront w of the
+// block decodes tile (blockIdx.y, nt0 + 8 blockIdx.x + w), lane f of it the 8 values of fragment lane f.
+// OUT_F32 = 0: fp16 bits [k][ns]; 1: f32 [k][ns]. (kernels/k-exl3/src/recon.rs:24-51, 131-157)
+template <int OUT_F32>
+__device__ __forceinline__ void recon_hat_body(void* out, const uint32_t* trellis, uint32_t n_tiles, uint32_t nt0,
+                                               uint32_t ns, uint32_t bits) {
+    uint32_t hw = threadIdx.x / 32, f = threadIdx.x % 32;
+    uint32_t kt = blockIdx.y, ntl = blockIdx.x * 8 + hw;
+    const uint32_t* tile = trellis + (size_t)(kt * n_tiles + nt0 + ntl) * 8 * bits;
+#pragma unroll
+    for (uint32_t j = 0; j < 8; j += 2) {
+        uint32_t h = decode2_mul1(tile_state_rt(tile, bits, f * 8 + j), tile_state_rt(tile, bits, f * 8 + j + 1));
+#pragma unroll
+        for (uint32_t e = 0; e < 2; e++) {
+            uint32_t jj = j + e, v = e ? (h >> 16) : (h & 0xffff);
+            uint32_t row = 2 * (f & 3) + (jj & 1) + 8 * ((jj >> 1) & 1);
+            uint32_t col = (f >> 2) + 8 * (jj >> 2);
+            size_t at = (size_t)(kt * 16 + row) * ns + ntl * 16 + col;
+            if (OUT_F32)
+                ((float*)out)[at] = f16_bits_to_f32(v);
+            else
+                ((uint16_t*)out)[at] = (uint16_t)v;
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(256) void exl3_recon_hat_f16(uint16_t* out, const uint32_t* trellis,
+                                                                     uint32_t n_tiles, uint32_t nt0, uint32_t ns,
+                                                                     uint32_t bits) {
+    recon_hat_body<0>(out, trellis, n_tiles, nt0, ns, bits);
+}
+
+extern "C" __global__ __launch_bounds__(256) void exl3_recon_hat_f32(float* out, const uint32_t* trellis,
+                                                                     uint32_t n_tiles, uint32_t nt0, uint32_t ns,
+                                                                     uint32_t bits) {
+    recon_hat_body<1>(out, trellis, n_tiles, nt0, ns, bits);
+}
+
+// In place: H over each row's 128-column blocks, * svh[n0 + col] / sqrt(128). grid (ns / 256, k), 64 threads: each
+// half of the wavefront owns one 128-column block (ns / 128 odd: the last block's upper half idles).
+// (kernels/k-exl3/src/recon.rs:54-64)
+extern "C" __global__ __launch_bounds__(64) void exl3_had_rows(float* buf, uint32_t ns, const uint16_t* svh, uint32_t n0) {
+    uint32_t lane = threadIdx.x, l32 = lane & 31;
+    uint32_t c = (blockIdx.x * 2 + (lane >> 5)) * 128 + 4 * l32;
+    bool live = c < ns;
+    float* p = buf + (size_t)blockIdx.y * ns + (live ? c : 0);
+    float v[4] = {p[0], p[1], p[2], p[3]};
+    fwht128_half_wave(v, l32);
+    if (live) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) p[q] = v[q] * FE_HAD_SCALE * f16_bits_to_f32(svh[n0 + c + q]);
+    }
+}
+
+// H over k (128-row blocks) * suh / sqrt(128) -> bf16, [k][n] (nk = 0, ld = n) or [n][k] (nk = 1, ld = k).
+// grid (ns / 32, k / 128), 128 threads, a 128 x 32 f32 tile in LDS. (kernels/k-exl3/src/recon.rs:66-128)
+extern "C" __global__ __launch_bounds__(128) void exl3_had_cols_bf16(const float* buf, uint16_t* out, uint32_t ns,
+                                                                      const uint16_t* suh, uint32_t n0, uint32_t ld,
+                                                                      uint32_t nk) {
+    constexpr uint32_t PITCH = 33;
+    __shared__ float sm[128 * PITCH];
+    uint32_t hw = threadIdx.x / 32, l32 = threadIdx.x % 32;
+    uint32_t r0 = blockIdx.y * 128, c0 = blockIdx.x * 32;
+    for (uint32_t i = 0; i < 32; i++) {
+        uint32_t r = hw * 32 + i;
+        sm[r * PITCH + l32] = buf[(size_t)(r0 + r) * ns + c0 + l32];
+    }
+    __syncthreads();
+    for (uint32_t cc = 0; cc < 8; cc++) {
+        uint32_t c = hw * 8 + cc;
+        float v[4];
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++) v[q] = sm[(4 * l32 + q) * PITCH + c];
+        fwht128_half_wave(v, l32);
+#pragma unroll
+        for (uint32_t q = 0; q < 4; q++) {
+            uint32_t r = 4 * l32 + q;
+            sm[r * PITCH + c] = v[q] * FE_HAD_SCALE * f16_bits_to_f32(suh[r0 + r]);
+        }
+    }
+    __syncthreads();
+    if (nk) {
+        for (uint32_t cc = 0; cc < 8; cc++) {
+            uint32_t c = hw * 8 + cc;
+            float v[4];
+#pragma unroll
+            for (uint32_t q = 0; q < 4; q++) v[q] = sm[(4 * l32 + q) * PITCH + c];
+            uint32_t* p = (uint32_t*)(out + (size_t)(n0 + c0 + c) * ld + r0 + 4 * l32);
+            p[0] = pack_bf16x2(v[0], v[1]);
+            p[1] = pack_bf16x2(v[2], v[3]);
+        }
+    } else {
+        for (uint32_t i = 0; i < 32; i++) {
+            uint32_t r = hw * 32 + i;
+            out[(size_t)(r0 + r) * ld + n0 + c0 + l32] = (uint16_t)f32_to_bf16_bits(sm[r * PITCH + l32]);
+        }
+    }
+}
+
+// ---- input rotation ------------------------------------------------------------------------------------------------
+
+// xh[row][k] = fp16(H(x * suh) / sqrt(128)), x bf16 (x_f32 = 0) or f32. grid (ceil(k / 512), rows), 128 threads: each
+// half wavefront one 128-element block, 4 elements a lane. (kernels/k-exl3/src/gemv.rs:147-170)
+extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_f32, const uint16_t* suh,
+                                                               uint16_t* xh, uint32_t k) {
+    uint32_t l32 = threadIdx.x & 31;
+    uint32_t blk = blockIdx.x * 4 + threadIdx.x / 32;
+    bool live = blk * 128 < k;
+    uint32_t c = (live ? blk : 0) * 128 + 4 * l32;
+    size_t at = (size_t)blockIdx.y * k + c;
+    float v[4];
+    if (x_f32) {
+        f32x4 t = *(const f32x4*)((const float*)x + at);
+        v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
+    } else {
+        u32x2 t = *(const u32x2*)((const uint16_t*)x + at);
+        v[0] = __uint_as_float(t[0] << 16), v[1] = __uint_as_float(t[0] & 0xffff0000u);
+        v[2] = __uint_as_float(t[1] << 16), v[3] = __uint_as_float(t[1] & 0xffff0000u);
+    }
+    u32x2 s = *(const u32x2*)(suh + c);
+    v[0] *= f16_bits_to_f32(s[0] & 0xffff), v[1] *= f16_bits_to_f32(s[0] >> 16);
+    v[2] *= f16_bits_to_f32(s[1] & 0xffff), v[3] *= f16_bits_to_f32(s[1] >> 16);
+    fwht128_half_wave(v, l32);
+    if (live) {
+        u32x2 o = {pack_f16x2(v[0] * FE_HAD_SCALE, v[1] * FE_HAD_SCALE), pack_f16x2(v[2] * FE_HAD_SCALE, v[3] * FE_HAD_SCALE)};
+        *(u32x2*)(xh + at) = o;
+    }
+}
+
+// ---- decode GEMV -----------------------------------------------------------------------------------------------------
+//
+// One program = one 128-column block x one K split; 256 threads = 4 wavefronts, wavefront w owning tiles 2w, 2w + 1 of
+// the block's 8. A wavefront's load step covers 4 consecutive k steps of its two tiles: lane L = 16 g + r reads k step g,
+// tile r >> 3, the BITS words of fragment lanes 4q .. 4q + 3 (q = r & 7) plus the word before them, which is all its 32
+// states need. Those states are rows n = q and n = q + 8 of the tile over all 16 k, so after decoding the lane holds, for
+// each of the two, the 16 values as two 8-value MFMA operands (k 0..7 and k 8..15) in k order. v_mfma_f32_16x16x32_f16
+// then sums over the 4 k steps: A = decoded weights (row r), B = 16 rotated input rows (column = input row), and the
+// accumulator of lane L holds output column 4 (L >> 4) + i of the 16 rows-of-A, input row L & 15.
+
+template <int BITS>
+struct LaneWords {
+    uint32_t w[BITS + 1];  // w[0] = the word before the lane's run
+};
+
+template <int BITS>
+__device__ __forceinline__ LaneWords<BITS> load_lane_words(const uint32_t* run, const uint32_t* prev) {
+    LaneWords<BITS> r;
+    r.w[0] = __builtin_nontemporal_load(prev);
+    if constexpr (BITS == 1) {
+        r.w[1] = __builtin_nontemporal_load(run);
+    } else if constexpr (BITS == 2) {
+        u32x2_a4 t = __builtin_nontemporal_load((const u32x2_a4*)run);
+        r.w[1] = t[0], r.w[2] = t[1];
+    } else if constexpr (BITS == 3) {
+        u32x3_a4 t = __builtin_nontemporal_load((const u32x3_a4*)run);
+        r.w[1] = t[0], r.w[2] = t[1], r.w[3] = t[2];
+    } else {
+        u32x4_a4 t = __builtin_nontemporal_load((const u32x4_a4*)run);
+        r.w[1] = t[0], r.w[2] = t[1], r.w[3] = t[2], r.w[4] = t[3];
+        if constexpr (BITS == 5) {
+            r.w[5] = __builtin_nontemporal_load(run + 4);
+        } else if constexpr (BITS == 6) {
+            u32x2_a4 u = __builtin_nontemporal_load((const u32x2_a4*)(run + 4));
+            r.w[5] = u[0], r.w[6] = u[1];
+        } else if constexpr (BITS == 7) {
+            u32x3_a4 u = __builtin_nontemporal_load((const u32x3_a4*)(run + 4));
+            r.w[5] = u[0], r.w[6] = u[1], r.w[7] = u[2];
+        } else if constexpr (BITS == 8) {
+            u32x4_a4 u = __builtin_nontemporal_load((const u32x4_a4*)(run + 4));
+            r.w[5] = u[0], r.w[6] = u[1], r.w[7] = u[2], r.w[8] = u[3];
+        }
+    }
+    return r;
+}
+
+// The 32-bit window of the lane's local stream starting at bit S (bit 0 = most significant bit of w[0]).
+template <int BITS, int S>
+__device__ __forceinline__ uint32_t window32(const LaneWords<BITS>& lw) {
+    constexpr int wi = S / 32, o = S % 32;
+    if constexpr (o == 0)
+        return lw.w[wi];
+    else
+        return __builtin_amdgcn_alignbit(lw.w[wi], lw.w[wi + 1], 32 - o);
+}
+
+// x = state * MUL1 of local position U (0..31): its state ends at local stream bit (U + 1) * BITS + 32.
+template <int BITS, int U>
+__device__ __forceinline__ uint32_t lane_x(const LaneWords<BITS>& lw) {
+    constexpr int end = (U + 1) * BITS + 32;
+    if constexpr (16 % BITS == 0) {
+        // positions 16 / BITS apart share one 32-bit window: the earlier one in its high half
+        constexpr int D = 16 / BITS;
+        if constexpr ((U / D) % 2 == 0)
+            return mul1_x<1>(window32<BITS, end - 16>(lw));
+        else
+            return mul1_x<0>(window32<BITS, end - 32>(lw));
+    } else {
+        if constexpr (end % 32 == 16)
+            return mul1_x<1>(lw.w[end / 32]);
+        else if constexpr (end % 32 == 0)
+            return mul1_x<0>(lw.w[end / 32 - 1]);
+        else if constexpr (end % 32 > 16)
+            return mul1_x<0>(lw.w[end / 32] >> (32 - end % 32));
+        else
+            return mul1_x<0>(window32<BITS, end - 32>(lw));
+    }
+}
+
+// The lane's 32 values as MFMA operands op[h][kh]: rows n = q + 8 h of the tile, k = 8 kh .. 8 kh + 7 in order.
+// Local position u = 8 c + i (fragment lane 4q + c, value i) is k = 2c + (i & 1) + 8 ((i >> 1) & 1), n half i >> 2.
+template <int BITS>
+__device__ __forceinline__ void decode_lane(const LaneWords<BITS>& lw, f16x8 (&op)[2][2]) {
+#define FE_PAIR(H, KH, C) mul1_finish2(lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H)>(lw), lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H) + 1>(lw))
+#define FE_OP(H, KH)                                                                             \
+    {                                                                                            \
+        u32x4 t = {FE_PAIR(H, KH, 0), FE_PAIR(H, KH, 1), FE_PAIR(H, KH, 2), FE_PAIR(H, KH, 3)};  \
+        op[H][KH] = __builtin_bit_cast(f16x8, t);                                                \
+    }
+    FE_OP(0, 0) FE_OP(0, 1) FE_OP(1, 0) FE_OP(1, 1)
+#undef FE_OP
+#undef FE_PAIR
+}
+
+// Store 4 consecutive outputs. mode: 0 bf16, 1 f32, 2 bf16 y += v (f32 add, one rounding), 3 f32 y += v.
+// (kernels/k-exl3/src/gemv.rs:122-145)
+__device__ __forceinline__ void store4(void* y, uint32_t mode, size_t i, float (&v)[4]) {
+    if (mode & 1) {
+        float* p = (float*)y + i;
+        f32x4 o = {v[0], v[1], v[2], v[3]};
+        if (mode & 2) o += *(const f32x4*)p;
+        *(f32x4*)p = o;
+    } else {
+        uint32_t* p = (uint32_t*)((uint16_t*)y + i);
+        if (mode & 2) {
+            uint32_t a = p[0], b = p[1];
+            v[0] += __uint_as_float(a << 16), v[1] += __uint_as_float(a & 0xffff0000u);
+            v[2] += __uint_as_float(b << 16), v[3] += __uint_as_float(b & 0xffff0000u);
+        }
+        u32x2 o = {pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])};
+        *(u32x2*)p = o;
+    }
+}
+
+// H over the 128 sums of a row (4 a lane of a half wavefront), * svh / sqrt(128), stored. (gemv.rs:172-180)
+__device__ __forceinline__ void finish_row(float (&v)[4], uint32_t l32, const uint16_t* svh, uint32_t col, void* y,
+                                           uint32_t mode, size_t at) {
+    fwht128_half_wave(v, l32);
+    u32x2 s = *(const u32x2*)(svh + col);
+    v[0] = v[0] * FE_HAD_SCALE * f16_bits_to_f32(s[0] & 0xffff);
+    v[1] = v[1] * FE_HAD_SCALE * f16_bits_to_f32(s[0] >> 16);
+    v[2] = v[2] * FE_HAD_SCALE * f16_bits_to_f32(s[1] & 0xffff);
+    v[3] = v[3] * FE_HAD_SCALE * f16_bits_to_f32(s[1] >> 16);
+    store4(y, mode, at, v);
+}
+
+#define GEMV_RED_PITCH 132  // floats a row of the 128-column partial sums (16-byte aligned, banks spread)
+
+// y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for m <= 16 RG rows. grid (n / 128 * sk), 256 threads. The rotated
+// inputs of the program's K range pass through LDS in chunks of `chunk` load steps (a multiple of 4): dynamic LDS
+// max(m * (chunk * 128 + 16), m * GEMV_RED_PITCH * 4) bytes. With sk > 1 the splits leave f32 partials in
+// z[split][m][n]; the last to arrive (counters[column block]) adds them in split order, finishes the block and re-arms
+// the counter. (kernels/k-exl3/src/gemv.rs:412-587)
+template <int BITS, int RG>
+__device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
+                                          const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
+                                          uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode,
+                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ uint32_t last_flag;
+    constexpr uint32_t tw = 8 * BITS;
+    constexpr int DEPTH = 4;  // load steps in flight per lane
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
+    const uint32_t nbs = n / 128, nb = blockIdx.x % nbs, split = blockIdx.x / nbs;
+    const uint32_t per_split = (k / 16) / sk;  // k steps of this program, a multiple of 4
+    const uint32_t kt0 = split * per_split;
+    const uint32_t col0 = nb * 128;
+    const uint32_t steps = per_split / 4;
+    const uint32_t xpitch = chunk * 128 + 16;  // bytes a row of staged inputs
+
+    const uint32_t tile_word = (2 * wave + tau) * tw;
+    const uint32_t* base = trellis + (size_t)nb * stride_nb + (size_t)(kt0 + g) * stride_k + tile_word;
+    const uint32_t run_off = q * BITS, prev_off = (q * BITS + tw - 1) % tw;
+    const size_t step_words = (size_t)4 * stride_k;
+
+    uint32_t xrow[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        uint32_t row = 16 * rg + r;
+        xrow[rg] = (row < m ? row : m - 1) * xpitch + g * 32;
+    }
+
+    f32x4 acc[RG][2];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    // the ring is indexed by constants only, so it stays in registers
+    LaneWords<BITS> ring[DEPTH];
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) {
+        const uint32_t* p = base + (size_t)(j < (int)steps ? j : 0) * step_words;
+        ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
+    }
+    for (uint32_t c0 = 0; c0 < steps; c0 += chunk) {
+        const uint32_t cs = steps - c0 < chunk ? steps - c0 : chunk;
+        if (c0) __syncthreads();
+        {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
+            const uint32_t chunks16 = cs * 8;  // 16-byte pieces a row
+            for (uint32_t i = tid; i < m * chunks16; i += 256) {
+                uint32_t row = i / chunks16, c = i - row * chunks16;
+                u32x4 v = *(const u32x4*)(xh + (size_t)row * k + (size_t)(kt0 + 4 * c0) * 16 + c * 8);
+                *(u32x4*)(lds + row * xpitch + c * 16) = v;
+            }
+        }
+        __syncthreads();
+        for (uint32_t s0 = 0; s0 < cs; s0 += DEPTH) {
+#pragma unroll
+            for (int j = 0; j < DEPTH; j++) {
+                const uint32_t sl = s0 + j, s = c0 + sl;
+                if (sl < cs) {
+                    f16x8 op[2][2];
+                    decode_lane<BITS>(ring[j], op);
+                    if (s + DEPTH < steps) {
+                        const uint32_t* p = base + (size_t)(s + DEPTH) * step_words;
+                        ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
+                    }
+#pragma unroll
+                    for (int rg = 0; rg < RG; rg++) {
+                        const unsigned char* xp = lds + xrow[rg] + sl * 128;
+                        f16x8 x0 = *(const f16x8*)xp, x1 = *(const f16x8*)(xp + 16);
+                        acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[rg][0], 0, 0, 0);
+                        acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[rg][1], 0, 0, 0);
+                        acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[rg][0], 0, 0, 0);
+                        acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // the block's sums -> LDS [row][128] (the input rows are no longer needed)
+    __syncthreads();
+    float* red = (float*)lds;
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        uint32_t row = 16 * rg + r;  // accumulator column = input row
+        if (row < m) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t arow = 4 * g + i;  // row of A: tile arow >> 3 of the pair, n = (arow & 7) + 8 h
+                    uint32_t col = 32 * wave + 16 * (arow >> 3) + (arow & 7) + 8 * h;
+                    red[row * GEMV_RED_PITCH + col] = acc[rg][h][i];
+                }
+        }
+    }
+    __syncthreads();
+
+    const uint32_t hw = tid >> 5, l32 = tid & 31;
+    if (sk == 1) {
+        for (uint32_t row = hw; row < m; row += 8) {
+            f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
+            float v[4] = {t[0], t[1], t[2], t[3]};
+            finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)row * n + col0 + 4 * l32);
+        }
+        return;
+    }
+    for (uint32_t row = hw; row < m; row += 8) {
+        f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
+        *(f32x4*)(z + ((size_t)split * m + row) * n + col0 + 4 * l32) = t;
+    }
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t old = atomicAdd(&counters[nb], 1u);
+        last_flag = (old == sk - 1);
+    }
+    __syncthreads();
+    if (last_flag) {
+        __threadfence();
+        for (uint32_t row = hw; row < m; row += 8) {
+            size_t at = (size_t)row * n + col0 + 4 * l32;
+            f32x4 t = __builtin_nontemporal_load((const f32x4*)(z + at));
+            for (uint32_t sp = 1; sp < sk; sp++) t += __builtin_nontemporal_load((const f32x4*)(z + (size_t)sp * m * n + at));
+            float v[4] = {t[0], t[1], t[2], t[3]};
+            finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, at);
+        }
+        if (tid == 0) counters[nb] = 0;
+    }
+}
+
+#define GEMV_KERNEL(BITS, RG)                                                                                         \
+    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_b##BITS##_r##RG(                                      \
+        const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,       \
+        uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb,       \
+        uint32_t chunk) {                                                                                             \
+        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk);       \
+    }
+#define GEMV_FAMILY(BITS) GEMV_KERNEL(BITS, 1) GEMV_KERNEL(BITS, 2) GEMV_KERNEL(BITS, 3) GEMV_KERNEL(BITS, 4)
+GEMV_FAMILY(2)
+GEMV_FAMILY(3)
+GEMV_FAMILY(4)
+GEMV_FAMILY(5)
+GEMV_FAMILY(6)
+GEMV_FAMILY(8)
+
+// ---- prefill GEMM ----------------------------------------------------------------------------------------------------
+
+// Weight tile producer of the prefill GEMM: a 64-wide k tile of a 128-column block is 4 k steps x 8 tiles; wavefront w
+// takes k step w, lane L tile L >> 3, rows n = (L & 7) and (L & 7) + 8 of it (the same run of words as in the GEMV).
+template <int BITS>
+struct Exl3Producer {
+    const uint32_t* base;  // block's trellis + this lane's tile
+    uint32_t stride_k, run_off, prev_off, brow, ks;
+    LaneWords<BITS> lw;
+    __device__ __forceinline__ void load(uint32_t kt) {
+        const uint32_t* p = base + (size_t)(kt * 4 + ks) * stride_k;
+        lw = load_lane_words<BITS>(p + run_off, p + prev_off);
+    }
+    __device__ __forceinline__ void store(_Float16* Bs) const {
+        f16x8 op[2][2];
+        decode_lane<BITS>(lw, op);
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int kh = 0; kh < 2; kh++) *(f16x8*)(Bs + (brow + 8 * h) * GM_PITCH + 16 * ks + 8 * kh) = op[h][kh];
+    }
+};
+
+#define GEMM_EPI_PITCH 132  // floats a row of the 128 x 128 output tile in LDS
+
+// y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for prefill-sized m: xh fp16 [m][k] (rotated inputs), 128 x 128 output
+// tiles, each exactly one Hadamard block wide so the output rotation is local to the tile. grid ceil(m / 128) * n / 128
+// (grouped raster), 256 threads, dynamic LDS 128 * GEMM_EPI_PITCH * 4 bytes.
+template <int BITS>
+__device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, const uint32_t* __restrict__ trellis,
+                                               const uint16_t* __restrict__ svh, void* y, uint32_t n, uint32_t k, uint32_t m,
+                                               uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    uint32_t tm, tn;
+    gemm_raster(blockIdx.x, (m + GM_BM - 1) / GM_BM, n / GM_BN, group_m, tm, tn);
+    const uint32_t m0 = tm * GM_BM, col0 = tn * GM_BN;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    constexpr uint32_t tw = 8 * BITS;
+    Exl3Producer<BITS> prod;
+    {
+        uint32_t tj = lane >> 3, q = lane & 7;
+        prod.base = trellis + (size_t)tn * stride_nb + tj * tw;
+        prod.stride_k = stride_k;
+        prod.run_off = q * BITS;
+        prod.prev_off = (q * BITS + tw - 1) % tw;
+        prod.brow = tj * 16 + q;
+        prod.ks = wave;
+    }
+    f32x16 acc[2][2];
+    gemm_mainloop(xh, k, m, k, m0, prod, lds, acc);
+    float* tile = (float*)lds;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) {
+                uint32_t row = wm * 64 + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+                tile[row * GEMM_EPI_PITCH + wn * 64 + 32 * j + (lane & 31)] = acc[i][j][e];
+            }
+    __syncthreads();
+    const uint32_t hw = tid >> 5, l32 = tid & 31;
+    for (uint32_t row = hw; row < GM_BM; row += 8) {
+        if (m0 + row >= m) break;
+        f32x4 t = *(const f32x4*)(tile + row * GEMM_EPI_PITCH + 4 * l32);
+        float v[4] = {t[0], t[1], t[2], t[3]};
+        finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)(m0 + row) * n + col0 + 4 * l32);
+    }
+}
+
+#define GEMM_KERNEL(BITS)                                                                                              \
+    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemm_b##BITS(                                            \
+        const _Float16* xh, const uint32_t* trellis, const uint16_t* svh, void* y, uint32_t n, uint32_t k, uint32_t m,  \
+        uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m) {                                    \
+        exl3_gemm_body<BITS>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m);                      \
+    }
+GEMM_KERNEL(2)
+GEMM_KERNEL(3)
+GEMM_KERNEL(4)
+GEMM_KERNEL(5)
+GEMM_KERNEL(6)
+GEMM_KERNEL(8)
+
+// ---- probes ----------------------------------------------------------------------------------------------------------
+
+// Streaming read of `bytes` (a multiple of 16 * 256 * gridDim.x * unroll) with 16-byte loads; each thread xors what it
+// read into one word of out so the loads stay. (kernels/k-exl3/src/probe.rs:7-36)
+extern "C" __global__ __launch_bounds__(256) void exl3_probe_v4(const u32x4* in, uint32_t* out, uint64_t vec_count) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x, stride = (uint64_t)gridDim.x * 256;
+    u32x4 a = {0, 0, 0, 0};
+    for (; i + 3 * stride < vec_count; i += 4 * stride) {
+        u32x4 v0 = __builtin_nontemporal_load(in + i), v1 = __builtin_nontemporal_load(in + i + stride);
+        u32x4 v2 = __builtin_nontemporal_load(in + i + 2 * stride), v3 = __builtin_nontemporal_load(in + i + 3 * stride);
+        a ^= v0 ^ v1 ^ v2 ^ v3;
+    }
+    for (; i < vec_count; i += stride) a ^= __builtin_nontemporal_load(in + i);
+    uint32_t x = a[0] ^ a[1] ^ a[2] ^ a[3];
+    if (x == 0x9e3779b9u) out[0] = x;  // practically never: keeps the loads alive without a store stream
+}
+
+// Decode-only probe: every lane decodes `iters` load steps of synthetic words (no memory traffic, no MFMA): the ALU
+// ceiling of the trellis decode in weights per second. out receives a checksum.
+template <int BITS>
+__device__ __forceinline__ void probe_decode_body(uint32_t* out, uint32_t iters, uint32_t seed) {
+    LaneWords<BITS> lw;
+#pragma unroll
+    for (int i = 0; i <= BITS; i++) lw.w[i] = seed * (threadIdx.x + 1) + i * 0x9e3779b9u;
+    uint32_t acc = 0;
+    for (uint32_t it = 0; it < iters; it++) {
+        f16x8 op[2][2];
+        decode_lane<BITS>(lw, op);
+        u32x4 a = __builtin_bit_cast(u32x4, op[0][0]) ^ __builtin_bit_cast(u32x4, op[0][1]) ^
+                  __builtin_bit_cast(u32x4, op[1][0]) ^ __builtin_bit_cast(u32x4, op[1][1]);
+        acc ^= a[0] ^ a[1] ^ a[2] ^ a[3];
+#pragma unroll
+        for (int i = 0; i <= BITS; i++) lw.w[i] += acc | 1;
+    }
+    if (acc == seed) out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+}
+extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b3(uint32_t* out, uint32_t iters, uint32_t seed) {
+    probe_decode_body<3>(out, iters, seed);
+}
+extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b4(uint32_t* out, uint32_t iters, uint32_t seed) {
+    probe_decode_body<4>(out, iters, seed);
+}
+extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b5(uint32_t* out, uint32_t iters, uint32_t seed) {
+    probe_decode_body<5>(out, iters, seed);
+}

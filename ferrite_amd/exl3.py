@@ -1,0 +1,291 @@
+"""Python mirror of the reference's fe-exl3 layer API over the C ABI (include/fe_exl3.h).
+
+Names, argument meaning and error behaviour follow crates/fe-exl3/src/{format,linear}.rs and gpu/mod.rs:
+`Exl3Tensor` (host container and its layout helpers), `Exl3View`, `DeviceExl3`, `Kernels`, `Plan`, `Dtype`,
+`Workspace`, `Linear`. torch tensors hold device memory; every compute call goes to libferrite_amd.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import enum
+from dataclasses import dataclass
+
+import numpy as np
+
+from . import _lib
+from ._lib import FeError, PlanC, View, check
+
+MUL1 = 0x83DCD12D  # crates/fe-exl3/src/format.rs:14
+
+
+class Dtype(enum.IntEnum):
+    """Activation element type; the Add forms are outputs only (crates/fe-exl3/src/linear.rs:12-31)."""
+    Bf16 = 0
+    F32 = 1
+    Bf16Add = 2
+    F32Add = 3
+
+
+class Exl3Tensor:
+    """An EXL3 tensor in host memory (crates/fe-exl3/src/format.rs:16-30): W is [k][n]; trellis = little-endian u32
+    words, tile (kt, nt) at [(kt * n/16 + nt) * 8 * bits ..][.. 8 * bits]; suh fp16 bits [k]; svh fp16 bits [n]."""
+
+    def __init__(self, name, k, n, bits, trellis, suh, svh):
+        self.name, self.k, self.n, self.bits = name, int(k), int(n), int(bits)
+        self.trellis = np.ascontiguousarray(trellis, dtype=np.uint32).reshape(-1)
+        self.suh = np.ascontiguousarray(suh, dtype=np.uint16).reshape(-1)
+        self.svh = np.ascontiguousarray(svh, dtype=np.uint16).reshape(-1)
+        if not 1 <= self.bits <= 8:
+            raise ValueError(f"{name}: {bits} bits")  # format.rs:42-44
+        if self.k % 16 or self.n % 16 or self.trellis.size != self.k // 16 * (self.n // 16) * self.tile_words():
+            raise ValueError(f"{name}: trellis of {self.trellis.size} words for {k}x{n} at {bits} bits")
+        if self.suh.size != self.k or self.svh.size != self.n:
+            raise ValueError(f"{name}: suh {self.suh.size} svh {self.svh.size} for {k}x{n}")  # format.rs:53-55
+
+    def tile_words(self):
+        return 8 * self.bits  # format.rs:60-62
+
+    def tile(self, kt, nt):
+        tw = self.tile_words()
+        i = (kt * (self.n // 16) + nt) * tw
+        return self.trellis[i:i + tw]  # format.rs:64-68
+
+    def strips(self):
+        """[n/128][k/16][8][tw]: each 128-column block's K range contiguous (format.rs:70-84)."""
+        tw, kt, nt = self.tile_words(), self.k // 16, self.n // 16
+        return np.ascontiguousarray(self.trellis.reshape(kt, nt // 8, 8 * tw).transpose(1, 0, 2)).reshape(-1)
+
+    def slice_cols(self, ranges):
+        """Column slice (format.rs:86-110): each range 128-aligned; an exact EXL3 tensor of its own."""
+        nt, tw = self.n // 16, self.tile_words()
+        for a, b in ranges:
+            if a % 128 or b % 128 or a >= b or b > self.n:
+                raise ValueError(f"{self.name}: column range {a}..{b} not 128-aligned in 0..{self.n}")
+        t3 = self.trellis.reshape(self.k // 16, nt, tw)
+        trellis = np.concatenate([t3[:, a // 16:b // 16] for a, b in ranges], axis=1)
+        svh = np.concatenate([self.svh[a:b] for a, b in ranges])
+        return Exl3Tensor(f"{self.name}[cols]", self.k, svh.size, self.bits, trellis, self.suh.copy(), svh)
+
+    def slice_rows(self, k0, k1):
+        """Row (input) slice [k0, k1) (format.rs:112-130): the partials of all slices sum to the full output."""
+        if k0 % 128 or k1 % 128 or k0 >= k1 or k1 > self.k:
+            raise ValueError(f"{self.name}: row range {k0}..{k1} not 128-aligned in 0..{self.k}")
+        row_words = self.n // 16 * self.tile_words()
+        return Exl3Tensor(f"{self.name}[rows {k0}..{k1}]", k1 - k0, self.n, self.bits,
+                          self.trellis[k0 // 16 * row_words:k1 // 16 * row_words].copy(), self.suh[k0:k1].copy(), self.svh.copy())
+
+    def trellis_bytes(self):
+        return self.trellis.size * 4  # format.rs:132-135
+
+
+def value_row(lane, j):
+    return 2 * (lane & 3) + (j & 1) + 8 * ((j >> 1) & 1)  # format.rs:148-150
+
+
+def value_col(lane, j):
+    return (lane >> 2) + 8 * (j >> 2)  # format.rs:154-156
+
+
+@dataclass
+class Exl3View:
+    """Device pointers of one EXL3 tensor (crates/fe-exl3/src/gpu/mod.rs:15-34)."""
+    k: int
+    n: int
+    bits: int
+    trellis: int
+    suh: int
+    svh: int
+    strips: bool
+
+    def strides(self):
+        tw = 8 * self.bits
+        return (8 * tw, self.k // 16 * 8 * tw) if self.strips else (self.n // 16 * tw, 8 * tw)
+
+    def c(self):
+        return View(self.k, self.n, self.bits, self.trellis, self.suh, self.svh, 1 if self.strips else 0)
+
+
+def _dev(arr, torch_dtype=None):
+    import torch
+    if arr.dtype == np.uint32:
+        return torch.from_numpy(arr.view(np.int32)).cuda()
+    if arr.dtype == np.uint16:
+        return torch.from_numpy(arr.view(np.int16)).cuda()
+    return torch.from_numpy(arr).cuda()
+
+
+class DeviceExl3:
+    """An EXL3 tensor uploaded to device memory (crates/fe-exl3/src/gpu/mod.rs:36-75)."""
+
+    def __init__(self, t: Exl3Tensor, strips: bool):
+        _lib.init()
+        self.name = t.name
+        self.trellis = _dev(t.strips() if strips else t.trellis)
+        self.suh = _dev(t.suh)
+        self.svh = _dev(t.svh)
+        self.view = Exl3View(t.k, t.n, t.bits, self.trellis.data_ptr(), self.suh.data_ptr(), self.svh.data_ptr(), strips)
+
+    @classmethod
+    def upload(cls, t):  # stored layout (what reconstruct reads)
+        return cls(t, False)
+
+    @classmethod
+    def upload_strips(cls, t):  # decode GEMV
+        return cls(t, True)
+
+
+@dataclass
+class Plan:
+    """Launch plan (crates/fe-exl3/src/linear.rs:33-55)."""
+    sk: int
+    wk: int = 4
+    ver: int = 1
+    occ: int = 0
+
+    @staticmethod
+    def parse(s: str):
+        p = PlanC()
+        try:
+            check(_lib.lib().fe_exl3_plan_parse(s.encode(), C.byref(p)))
+        except FeError:
+            return None
+        return Plan(p.sk, p.wk, p.ver, p.occ)
+
+    def c(self):
+        return PlanC(self.sk, self.wk, self.ver, self.occ)
+
+
+def default_blocks(cu_count: int) -> int:
+    return 4 * cu_count  # linear.rs:131-134
+
+
+def _stream(s):
+    if s is None:
+        import torch
+        s = torch.cuda.current_stream()
+    return C.c_void_p(getattr(s, "cuda_stream", s))
+
+
+class Kernels:
+    """The gfx950 code object of the EXL3 kernels, loaded into the current context (gpu/mod.rs:77-102)."""
+
+    def __init__(self):
+        _lib.init()
+        self.h = C.c_void_p()
+        check(_lib.lib().fe_exl3_kernels_load(C.byref(self.h)))
+
+    @classmethod
+    def load(cls):
+        return cls()
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            _lib.lib().fe_exl3_kernels_destroy(self.h)
+            self.h = None
+
+    def reconstruct_hat_f16(self, view: Exl3View, out, stream=None):
+        """Rotated-basis W_hat as fp16 [k][n] (gpu/mod.rs:159-165)."""
+        v = view.c()
+        check(_lib.lib().fe_exl3_reconstruct_hat_f16(self.h, _stream(stream), C.byref(v), out.data_ptr()))
+
+    @staticmethod
+    def recon_scratch_bytes(view: Exl3View):
+        return view.k * view.n * 4  # gpu/mod.rs:104-108
+
+    def reconstruct_bf16(self, view: Exl3View, out, layout, scratch, stream=None):
+        """Original-basis W as bf16, layout "KN" or "NK" (gpu/mod.rs:110-157)."""
+        v = view.c()
+        check(_lib.lib().fe_exl3_reconstruct_bf16(self.h, _stream(stream), C.byref(v), out.data_ptr(), 0 if layout == "KN" else 1,
+                                                  scratch.data_ptr(), scratch.numel() * scratch.element_size()))
+
+    def probe_stream_read(self, buf, grid, launches, stream=None):
+        ms = C.c_float()
+        check(_lib.lib().fe_exl3_probe_stream_read(self.h, _stream(stream), buf.data_ptr(), buf.numel() * buf.element_size(), grid,
+                                                   launches, C.byref(ms)))
+        return ms.value
+
+    def probe_decode(self, bits, grid, iters, launches, stream=None):
+        ms = C.c_float()
+        check(_lib.lib().fe_exl3_probe_decode(self.h, _stream(stream), bits, grid, iters, launches, C.byref(ms)))
+        return ms.value
+
+
+def cu_count() -> int:
+    _lib.init()
+    n = C.c_int()
+    check(_lib.lib().fe_hip_cu_count(C.byref(n)))
+    return n.value
+
+
+class Linear:
+    """An EXL3 linear served straight from the trellis (crates/fe-exl3/src/linear.rs:163-342)."""
+
+    def __init__(self, kern: Kernels, name: str, view: Exl3View, plan: Plan, owned=None):
+        self.kern, self.name, self.view, self.owned = kern, name, view, owned
+        self.h = C.c_void_p()
+        v, p = view.c(), plan.c()
+        check(_lib.lib().fe_exl3_linear_from_view(C.byref(self.h), kern.h, name.encode(), C.byref(v), C.byref(p)))
+        self.k, self.n, self.bits, self.plan = view.k, view.n, view.bits, plan
+
+    @staticmethod
+    def plan_for(k, n, bits, blocks) -> Plan:
+        p = PlanC()
+        check(_lib.lib().fe_exl3_plan_for(k, n, bits, blocks, C.byref(p)))
+        return Plan(p.sk, p.wk, p.ver, p.occ)
+
+    @classmethod
+    def new(cls, kern, w: DeviceExl3, blocks: int):
+        return cls.with_plan(kern, w, cls.plan_for(w.view.k, w.view.n, w.view.bits, blocks))
+
+    @classmethod
+    def with_plan(cls, kern, w: DeviceExl3, plan: Plan):
+        return cls(kern, w.name, w.view, plan, owned=w)
+
+    @classmethod
+    def from_view(cls, kern, name, view: Exl3View, plan: Plan):
+        return cls(kern, name, view, plan)
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            _lib.lib().fe_exl3_linear_destroy(self.h)
+            self.h = None
+
+    def weight_bytes(self):
+        return _lib.lib().fe_exl3_linear_weight_bytes(self.h)
+
+    def forward(self, x, x_dtype: Dtype, y, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+        """y[rows][n] = x[rows][k] @ W (linear.rs:273-287)."""
+        check(_lib.lib().fe_exl3_linear_forward(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), y.data_ptr(),
+                                                int(y_dtype), rows, ws.h))
+
+    def rotate_input(self, x, x_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+        check(_lib.lib().fe_exl3_linear_rotate_input(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), rows, ws.h))
+
+    def gemv_rotated(self, xh, y, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+        ptr = xh if isinstance(xh, int) else xh.data_ptr()
+        check(_lib.lib().fe_exl3_linear_gemv_rotated(self.h, _stream(stream), ptr, y.data_ptr(), int(y_dtype), rows, ws.h))
+
+
+class Workspace:
+    """Scratch shared by every Linear on one stream (linear.rs:136-161)."""
+
+    def __init__(self, linears, max_rows: int):
+        _lib.init()
+        self.h = C.c_void_p()
+        arr = (C.c_void_p * max(len(linears), 1))(*[l.h for l in linears])
+        check(_lib.lib().fe_exl3_workspace_create(C.byref(self.h), arr, len(linears), max_rows))
+        xh, mr, mk = C.c_uint64(), C.c_uint32(), C.c_uint32()
+        check(_lib.lib().fe_exl3_workspace_xh(self.h, C.byref(xh), C.byref(mr), C.byref(mk)))
+        self.xh_ptr, self.max_rows, self.max_k = xh.value, mr.value, mk.value
+
+    def xh(self, rows, k):
+        """The first rows x k rotated inputs as a host uint16 array (fp16 bits)."""
+        out = np.empty((rows, k), np.uint16)
+        for r in range(rows):
+            check(_lib.lib().fe_hip_memcpy_dtoh(out[r].ctypes.data_as(C.c_void_p), self.xh_ptr + 2 * r * k, 2 * k))
+        return out
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            _lib.lib().fe_exl3_workspace_destroy(self.h)
+            self.h = None

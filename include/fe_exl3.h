@@ -1,0 +1,107 @@
+/*
+ * fe_exl3: the EXL3 (trellis-coded, Hadamard-rotated) linear layer over fe_hip.
+ *
+ * C ABI of the reference's fe-exl3 layer API: the same packed-weight layout (trellis words in the stored
+ * [k/16][n/16][8*bits] layout or the "strips" relayout, fp16 suh[k] / svh[n] sign-scale vectors), the same launch-plan
+ * and workspace objects and the same call signatures, so that fe-model's `Linear::forward`
+ * (crates/fe-model/src/model.rs:275-346) can bind it in place of `fe_exl3::linear` + `fe_exl3::gpu`.
+ *
+ * All functions return 0 or an error code (HIP's, or FE_ERR_*); fe_hip_last_error() gives the text. Shape and
+ * workspace violations are errors, never aborts (crates/fe-exl3/src/linear.rs:291-307). Calls that share a workspace
+ * must be ordered on one stream. No call synchronizes the host; forward/rotate_input/gemv_rotated only enqueue.
+ */
+#ifndef FE_EXL3_H
+#define FE_EXL3_H
+
+#include "fe_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FE_ERR_SHAPE 10001     /* shape does not fit the kernel or plan */
+#define FE_ERR_WORKSPACE 10002 /* rows or sizes exceed the workspace */
+#define FE_ERR_ARG 10003       /* null or inconsistent argument */
+#define FE_ERR_UNSUPPORTED 10004
+
+/* Activation / output element type; the *_ADD forms are outputs only: y += x @ W, bf16 adds in f32 and rounds once.
+ * Values are the kernels' flag (crates/fe-exl3/src/linear.rs:15-31). */
+enum { FE_DTYPE_BF16 = 0, FE_DTYPE_F32 = 1, FE_DTYPE_BF16_ADD = 2, FE_DTYPE_F32_ADD = 3 };
+
+/* Device pointers of one EXL3 tensor (Exl3View, crates/fe-exl3/src/gpu/mod.rs:17-34). strips != 0: trellis is in the
+ * strips layout [n/128][k/16][8][8*bits] (crates/fe-exl3/src/format.rs:70-84). */
+typedef struct {
+    uint32_t k, n, bits;
+    fe_devptr_t trellis, suh, svh;
+    uint32_t strips;
+} fe_exl3_view;
+
+/* Launch plan (Plan, crates/fe-exl3/src/linear.rs:33-43): sk K splits per 128-column block; wk, ver, occ are kept for
+ * the reference's plan strings ("sk,wk[,ver[,occ]]") and recorded, the gfx950 kernels use one form (256 threads). */
+typedef struct {
+    uint32_t sk, wk, ver, occ;
+} fe_exl3_plan;
+
+typedef struct fe_exl3_kernels fe_exl3_kernels;     /* Kernels, crates/fe-exl3/src/gpu/mod.rs:78-102 */
+typedef struct fe_exl3_linear fe_exl3_linear;       /* Linear, crates/fe-exl3/src/linear.rs:163-176 */
+typedef struct fe_exl3_workspace fe_exl3_workspace; /* Workspace, crates/fe-exl3/src/linear.rs:137-161 */
+
+/* Kernels::load: the embedded gfx950 code object, or the file named by FE_EXL3_HSACO (the reference's FE_EXL3_CUBIN,
+ * crates/fe-exl3/src/gpu/mod.rs:88-93). */
+int fe_exl3_kernels_load(fe_exl3_kernels **out);
+int fe_exl3_kernels_destroy(fe_exl3_kernels *k);
+
+/* Linear::plan_for (crates/fe-exl3/src/linear.rs:217-233): `blocks` is the program target (4 per CU is the default,
+ * default_blocks linear.rs:132-134). Honours FE_EXL3_NOSPLIT=1 / FE_EXL3_SPLIT=0. */
+int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_exl3_plan *out);
+/* Plan::parse "sk,wk[,ver[,occ]]" (linear.rs:47-55). */
+int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out);
+
+/* Linear::from_view (linear.rs:242-266): a linear over device buffers the caller owns and keeps alive. */
+int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, const char *name, const fe_exl3_view *view,
+                             const fe_exl3_plan *plan);
+/* Linear::new(DeviceExl3::upload_strips(tensor)) (linear.rs:212-215, gpu/mod.rs:52-70): host tensor in the stored
+ * layout (trellis words, fp16 suh/svh); the linear owns the device copy. plan == NULL: plan_for(blocks). */
+int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, const char *name, uint32_t k, uint32_t n,
+                          uint32_t bits, const uint32_t *trellis, const uint16_t *suh, const uint16_t *svh, int strips,
+                          const fe_exl3_plan *plan, uint32_t blocks);
+int fe_exl3_linear_destroy(fe_exl3_linear *l);
+int fe_exl3_linear_view(const fe_exl3_linear *l, fe_exl3_view *view, fe_exl3_plan *plan);
+/* Trellis bytes streamed per call (linear.rs:268-271). */
+size_t fe_exl3_linear_weight_bytes(const fe_exl3_linear *l);
+
+/* Workspace::new(&[&Linear], max_rows) (linear.rs:147-160): xh fp16 [max_rows][max k], f32 split partials, split
+ * arrival counters (zero at rest; each call re-arms them). */
+int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows);
+int fe_exl3_workspace_destroy(fe_exl3_workspace *ws);
+int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t *max_rows, uint32_t *max_k);
+
+/* Linear::forward (linear.rs:274-287): y[rows][n] = x[rows][k] @ W; x bf16 or f32, y bf16 or f32 (+ the add forms),
+ * both row-major and contiguous. rows <= 64 run the decode GEMV (HBM-bound); more rows run the LDS-staged MFMA GEMM. */
+int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws);
+/* Linear::rotate_input (linear.rs:289-298): xh = fp16(H(x * suh) / sqrt(128)) into the workspace. */
+int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
+                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws);
+/* Linear::gemv_rotated (linear.rs:300-341): the trellis linear on already rotated fp16 inputs xh [rows][k]. */
+int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
+                                uint32_t rows, const fe_exl3_workspace *ws);
+
+/* Kernels::reconstruct_hat_f16 (gpu/mod.rs:159-165): rotated-basis W_hat as fp16 [k][n]; stored layout only. */
+int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out);
+/* Kernels::reconstruct_bf16 (gpu/mod.rs:110-157): original-basis W as bf16, layout 0 = [k][n], 1 = [n][k];
+ * scratch: f32 workspace of at least k * 128 * 4 bytes; stored layout only. */
+int fe_exl3_reconstruct_bf16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out, int layout,
+                             fe_devptr_t scratch, size_t scratch_bytes);
+
+/* Probes (kernels/k-exl3/src/probe.rs): launch `launches` back-to-back runs and return the average milliseconds.
+ * stream_read: 16-byte loads over `bytes` of `buf`; decode: ALU-only trellis decode of grid * 256 * 32 * iters weights. */
+int fe_exl3_probe_stream_read(const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t buf, size_t bytes, uint32_t grid,
+                              uint32_t launches, float *ms);
+int fe_exl3_probe_decode(const fe_exl3_kernels *kern, fe_stream_t s, uint32_t bits, uint32_t grid, uint32_t iters,
+                         uint32_t launches, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

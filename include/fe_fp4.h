@@ -1,0 +1,58 @@
+/*
+ * fe_fp4: the NVFP4 prompt linear (e2m1 codes, e4m3 scale per 16 along K, fp32 scale per output column) over fe_hip.
+ *
+ * C ABI of the reference's fe-fp4 layer API for its NVFP4 path (crates/fe-fp4/src/lib.rs): HostLinear-style inputs
+ * (codes [n][k/2], row-major scales [n][k/16], alpha[n], g), PromptLinear::{forward, quantize, gemm}, Workspace.
+ * Requirements as in the reference (lib.rs:156-157, 521-537): N % 128 == 0, K % 128 == 0, ldy % 8 == 0, y and res
+ * 16-byte aligned, m == 0 is a no-op, m <= ws.max_rows, k <= ws.max_k. Errors are return codes, as in fe_exl3.h.
+ */
+#ifndef FE_FP4_H
+#define FE_FP4_H
+
+#include "fe_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct fe_fp4_kernels fe_fp4_kernels;     /* Kernels, crates/fe-fp4/src/lib.rs:30-117 */
+typedef struct fe_fp4_linear fe_fp4_linear;       /* PromptLinear, crates/fe-fp4/src/lib.rs:265-283 */
+typedef struct fe_fp4_workspace fe_fp4_workspace; /* Workspace, crates/fe-fp4/src/lib.rs:215-226 */
+
+/* Kernels::load (lib.rs:65-117): the embedded gfx950 code object, or the file named by FE_FP4_HSACO.
+ * FE_FP4_GROUP sets the raster group height in row tiles (default 8, 0 = all). */
+int fe_fp4_kernels_load(fe_fp4_kernels **out);
+int fe_fp4_kernels_destroy(fe_fp4_kernels *k);
+
+/* HostLinear::upload (lib.rs:425-440) of an NVFP4 linear already fused on the host: codes [n][k/2], scales row-major
+ * [n][k/16] (e4m3), alpha[n] = max(input_scale) * weight_scale_2 of the column's part, g = 1 / max(input_scale). */
+int fe_fp4_linear_upload(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, const uint8_t *codes,
+                         const uint8_t *scales, const float *alpha, float g);
+/* A linear over device buffers the caller owns (the reference's streamed form, PromptLinear::set_views lib.rs:485-494). */
+int fe_fp4_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, fe_devptr_t codes,
+                            fe_devptr_t scales, fe_devptr_t alpha, float g);
+int fe_fp4_linear_destroy(fe_fp4_linear *l);
+int fe_fp4_linear_shape(const fe_fp4_linear *l, uint32_t *n, uint32_t *k, float *g);
+
+/* Workspace::new(max_rows, max_k) (lib.rs:221-226): quantized activations: codes, tiled scales
+ * ([rows/128][k/128][128][8], crates/fe-fp4/src/format.rs:98-111), and the fp16 operand the GEMM reads. */
+int fe_fp4_workspace_create(fe_fp4_workspace **out, uint32_t max_rows, uint32_t max_k);
+int fe_fp4_workspace_destroy(fe_fp4_workspace *ws);
+int fe_fp4_workspace_buffers(const fe_fp4_workspace *ws, fe_devptr_t *codes, fe_devptr_t *sf, uint32_t *max_rows,
+                             uint32_t *max_k);
+
+/* PromptLinear::forward (lib.rs:510-516): y (row stride ldy) = x (bf16, row stride lda) . W^T for m rows; with res
+ * (stride ldy, may equal y): y = bf16(bf16(x . W^T) + res). res == 0: none. */
+int fe_fp4_linear_forward(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
+                          fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda, uint32_t m, fe_devptr_t res);
+/* PromptLinear::quantize (lib.rs:518-530). */
+int fe_fp4_linear_quantize(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
+                           fe_devptr_t x, uint32_t lda, uint32_t m);
+/* PromptLinear::gemm (lib.rs:532-543) over activations already quantized into ws by a linear with the same k and g. */
+int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
+                       fe_devptr_t y, uint32_t ldy, uint32_t m, fe_devptr_t res);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

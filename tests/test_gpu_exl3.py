@@ -1,0 +1,260 @@
+"""GPU parity of the EXL3 path against the CPU oracle, through the C ABI. Mirrors the reference's check binaries:
+exl3-gpucheck (reconstruct), exl3-gemvcheck (rot_in, GEMV at rows 1..64, untouched rows, row invariance, fused
+residual add), exl3-tpcheck (slices) and exl3-detcheck (determinism with a shared workspace)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [1, 2, 5, 8, 9, 16, 17, 33, 64]  # crates/fe-exl3/src/bin/exl3-gemvcheck.rs:53
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from ferrite_amd import exl3
+    assert torch.cuda.is_available()
+    kern = exl3.Kernels.load()
+    return torch, exl3, kern
+
+
+def to_oracle(oracle, t):
+    return oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+
+
+def dev_u16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def bf16_to_f64(a):
+    return (a.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 6, 7, 8])
+def test_reconstruct_hat_is_bit_exact(env, oracle, bits):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(256, 384, bits, 100 + bits)
+    d = exl3.DeviceExl3.upload(t)
+    out = torch.zeros((t.k, t.n), dtype=torch.int16, device="cuda")
+    kern.reconstruct_hat_f16(d.view, out)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16)
+    want = oracle.w_hat_f16(to_oracle(oracle, t))
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} values differ"
+
+
+@pytest.mark.parametrize("layout", ["KN", "NK"])
+def test_reconstruct_bf16_within_one_ulp(env, oracle, layout):
+    """crates/fe-exl3/src/bin/exl3-gpucheck.rs:44-98: GPU f32 math vs the f64 reference: at most 1 bf16 ulp apart, and
+    the two layouts exact transposes of each other."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(384, 256, 4, 7)
+    d = exl3.DeviceExl3.upload(t)
+    out = torch.zeros(t.k * t.n, dtype=torch.int16, device="cuda")
+    # a scratch of 128 columns forces the column-sliced path
+    scratch = torch.empty(t.k * 128, dtype=torch.float32, device="cuda")
+    kern.reconstruct_bf16(d.view, out, layout, scratch)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.uint16).reshape((t.k, t.n) if layout == "KN" else (t.n, t.k))
+    want = oracle.weight_bf16(to_oracle(oracle, t), layout=layout)
+    ordered = lambda h: np.where(h & 0x8000, -(h & 0x7FFF).astype(np.int32), h.astype(np.int32))
+    assert np.abs(ordered(got) - ordered(want)).max() <= 1
+    assert (got != want).mean() < 0.02
+
+
+def run_forward(torch, exl3, lin, ws, xd, rows, y_dtype, prefill=None):
+    f32 = y_dtype in (exl3.Dtype.F32, exl3.Dtype.F32Add)
+    if prefill is None:
+        y = torch.full((64 if rows <= 64 else rows, lin.n), float("nan"), dtype=torch.float32 if f32 else torch.bfloat16, device="cuda")
+    else:
+        y = prefill
+    lin.forward(xd, exl3.Dtype.Bf16, y, y_dtype, rows, ws)
+    torch.cuda.synchronize()
+    return y
+
+
+def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    o = to_oracle(oracle, t)
+    mr = 64
+    xb = synth.activations(mr, t.k, seed)
+    x64 = bf16_to_f64(xb)
+    d = exl3.DeviceExl3(t, strips)
+    lin = exl3.Linear.with_plan(kern, d, plan)
+    ws = exl3.Workspace([lin], mr)
+    xd = dev_u16(torch, xb)
+    # rot_in alone vs the f64 reference: a rare 1-ulp tie flip allowed (exl3-gemvcheck.rs:79-88)
+    lin.rotate_input(xd, exl3.Dtype.Bf16, mr, ws)
+    torch.cuda.synchronize()
+    xh_gpu = ws.xh(mr, t.k)
+    xh_ref = oracle.rotate_input_ref(o, x64)
+    far = np.abs(xh_gpu.astype(np.int32) - xh_ref.astype(np.int32)) > 1
+    assert not far.any() and (xh_gpu != xh_ref).mean() < 2e-3
+    hat = oracle.w_hat_f16(o)
+    yref = oracle.gemv_ref(o, hat, xh_gpu)  # on the GPU's own rotated input: what is left is fp32 summation order
+    first5 = None
+    for rows in rows_list:
+        y = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.F32).cpu().numpy().astype(np.float64)
+        yb = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.Bf16).view(torch.int16).cpu().numpy().view(np.uint16)
+        ref = yref[:rows]
+        rms = np.sqrt((ref ** 2).mean())
+        rel_max = np.abs(y[:rows] - ref).max() / rms
+        assert rel_max < 1e-4, (rows, rel_max)  # exl3-gemvcheck.rs:117-121
+        # the north-star bar: max relative error 1e-2 (floored at 1e-2 of the rms)
+        assert (np.abs(y[:rows] - ref) / np.maximum(np.abs(ref), 1e-2 * rms)).max() < 1e-2
+        # bf16 output within one rounding of the exact value (exl3-gemvcheck.rs:106-110)
+        e = np.abs(bf16_to_f64(yb[:rows]) - ref)
+        assert np.all(e <= np.abs(ref) / 256.0 + 1e-5 * rms), rows
+        # rows past `rows` untouched (exl3-gemvcheck.rs:113-116)
+        if rows < 64:
+            assert np.isnan(y[rows:]).all()
+        if rows >= 5:  # row invariance (exl3-gemvcheck.rs:124-141)
+            if first5 is None:
+                first5 = y[:5].copy()
+            else:
+                assert np.array_equal(first5.view(np.uint64), y[:5].view(np.uint64)), rows
+    # fused residual add: y (bf16, prefilled with 1.5) += x @ W, 5 rows (exl3-gemvcheck.rs:142-168)
+    rows = 5
+    pre = torch.full((mr, t.n), 1.5, dtype=torch.bfloat16, device="cuda")
+    ya = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.Bf16Add, prefill=pre).view(torch.int16).cpu().numpy().view(np.uint16)
+    want = 1.5 + yref[:rows]
+    rms = np.sqrt((yref[:rows] ** 2).mean())
+    assert np.all(np.abs(bf16_to_f64(ya[:rows]) - want) <= np.abs(want) / 256.0 + 1e-5 * rms)
+    assert (ya[rows:] == 0x3FC0).all()
+    pre32 = torch.full((mr, t.n), 0.25, dtype=torch.float32, device="cuda")
+    y32 = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.F32Add, prefill=pre32).cpu().numpy().astype(np.float64)
+    assert np.abs(y32[:rows] - 0.25 - yref[:rows]).max() / rms < 1e-4 and (y32[rows:] == 0.25).all()
+    return lin, ws, xd, yref
+
+
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+def test_gemv_all_bit_widths(env, oracle, bits):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(512, 256, bits, 20 + bits)
+    check_linear(env, oracle, t, exl3.Plan(2), strips=True, rows_list=[1, 5, 16, 17, 64])
+
+
+@pytest.mark.parametrize("sk,strips", [(1, True), (1, False), (4, True), (8, False), (16, True)])
+def test_gemv_splits_and_layouts(env, oracle, sk, strips):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(1024, 384, 4, 31)
+    check_linear(env, oracle, t, exl3.Plan(sk), strips=strips)
+
+
+def test_gemv_long_k_streams_inputs_in_chunks(env, oracle):
+    """K long enough that 64 rows of inputs do not fit LDS at once (one split, 68 load steps, chunks of 4)."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(4352, 128, 3, 5)
+    check_linear(env, oracle, t, exl3.Plan(1), strips=True, rows_list=[1, 16, 64])
+
+
+def test_plan_for_default_and_determinism_with_shared_workspace(env, oracle):
+    """crates/fe-exl3/src/bin/exl3-detcheck.rs:36-70: repeated forwards interleaved with a second linear that shares the
+    workspace give identical bits."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    a = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, 256, 4, 1)), exl3.default_blocks(exl3.cu_count()))
+    b = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(512, 384, 3, 2)), exl3.default_blocks(exl3.cu_count()))
+    assert a.plan.sk > 1 and b.plan.sk > 1
+    ws = exl3.Workspace([a, b], 16)
+    xa, xb = dev_u16(torch, synth.activations(16, 1024, 3)), dev_u16(torch, synth.activations(16, 512, 4))
+    ya = torch.empty((16, 256), dtype=torch.float32, device="cuda")
+    yb = torch.empty((16, 384), dtype=torch.float32, device="cuda")
+    first = None
+    for it in range(40):
+        rows = 1 + (it * 7) % 16
+        a.forward(xa, exl3.Dtype.Bf16, ya, exl3.Dtype.F32, 16, ws)
+        b.forward(xb, exl3.Dtype.Bf16, yb, exl3.Dtype.F32, rows, ws)
+        torch.cuda.synchronize()
+        cur = ya.cpu().numpy().copy()
+        if first is None:
+            first = cur
+        assert np.array_equal(first.view(np.uint32), cur.view(np.uint32)), it
+
+
+def test_tp_slices_match_the_whole(env, oracle):
+    """crates/fe-exl3/src/bin/exl3-tpcheck.rs: column slices reproduce their columns, row slices sum to the whole."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(512, 512, 4, 9)
+    xb = synth.activations(4, 512, 9)
+    xd = dev_u16(torch, xb)
+
+    def fwd(tt, x):
+        lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(tt), exl3.Plan(2))
+        ws = exl3.Workspace([lin], 4)
+        y = torch.empty((4, tt.n), dtype=torch.float32, device="cuda")
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 4, ws)
+        torch.cuda.synchronize()
+        return y.cpu().numpy().astype(np.float64)
+
+    whole = fwd(t, xd)
+    rms = np.sqrt((whole ** 2).mean())
+    cols = fwd(t.slice_cols([(128, 256), (384, 512)]), xd)
+    assert np.array_equal(cols, np.concatenate([whole[:, 128:256], whole[:, 384:512]], axis=1))
+    parts = fwd(t.slice_rows(0, 256), dev_u16(torch, xb[:, :256])) + fwd(t.slice_rows(256, 512), dev_u16(torch, xb[:, 256:]))
+    assert np.abs(parts - whole).max() / rms < 2e-5  # exl3-tpcheck.rs:103-105
+
+
+@pytest.mark.parametrize("bits,m", [(4, 200), (3, 129), (5, 65)])
+def test_prefill_gemm_matches_the_oracle(env, oracle, bits, m):
+    """More than 64 rows take the LDS-staged MFMA GEMM; same contract as the GEMV (f64 reference on the GPU's own xh)."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(512, 256, bits, 40 + bits)
+    o = to_oracle(oracle, t)
+    xb = synth.activations(m, t.k, 3, outliers=True)
+    for strips in (True, False):
+        lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3(t, strips), exl3.Plan(2))
+        ws = exl3.Workspace([lin], m)
+        xd = dev_u16(torch, xb)
+        y = torch.full((m + 3, t.n), float("nan"), dtype=torch.float32, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+        yb = torch.zeros((m, t.n), dtype=torch.bfloat16, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, yb, exl3.Dtype.Bf16, m, ws)
+        torch.cuda.synchronize()
+        xh = ws.xh(m, t.k)
+        ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), xh)
+        got = y.cpu().numpy().astype(np.float64)
+        rms = np.sqrt((ref ** 2).mean())
+        assert np.abs(got[:m] - ref).max() / rms < 1e-4
+        assert np.isnan(got[m:]).all()
+        e = np.abs(bf16_to_f64(yb.view(torch.int16).cpu().numpy().view(np.uint16)) - ref)
+        assert np.all(e <= np.abs(ref) / 256.0 + 1e-5 * rms)
+        # against the reference linear on the bf16 inputs themselves (f64 all the way): the 1e-2 bar, floored
+        lin64 = oracle.linear_f64(o, bf16_to_f64(xb), threads=4)
+        assert (np.abs(got[:m] - lin64) / np.maximum(np.abs(lin64), 2e-2 * np.sqrt((lin64 ** 2).mean()))).max() < 1e-2
+
+
+def test_argument_errors_are_results_not_crashes(env):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    from ferrite_amd._lib import FeError
+    t = synth.exl3_tensor(256, 128, 4, 1)
+    d = exl3.DeviceExl3.upload_strips(t)
+    with pytest.raises(FeError):
+        exl3.Linear.with_plan(kern, d, exl3.Plan(3))  # 4 load steps do not divide by 3
+    with pytest.raises(FeError):
+        exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(256, 128, 7, 1)), exl3.Plan(1))
+    lin = exl3.Linear.with_plan(kern, d, exl3.Plan(2))
+    ws = exl3.Workspace([lin], 4)
+    x = dev_u16(torch, synth.activations(8, 256, 1))
+    y = torch.zeros((8, 128), dtype=torch.float32, device="cuda")
+    with pytest.raises(FeError):
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 0, ws)
+    with pytest.raises(FeError):
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 5, ws)  # workspace holds 4 rows
+    small = exl3.Workspace([exl3.Linear.with_plan(kern, d, exl3.Plan(1))], 4)
+    with pytest.raises(FeError):
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 4, small)  # no room for split partials
+    with pytest.raises(FeError):
+        kern.reconstruct_hat_f16(d.view, y)  # strips layout
+    lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 4, ws)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y[:4]).all()

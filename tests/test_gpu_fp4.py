@@ -1,0 +1,120 @@
+"""GPU parity of the NVFP4 path against the CPU oracle, through the C ABI. Mirrors the reference's fp4-check
+(crates/fe-fp4/src/bin/fp4-check.rs:30-208): activation quantizer bit-exact, GEMM vs an f64 GEMM over the same
+quantized operands, the residual epilogue, the strided-output canary, and argument errors."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from ferrite_amd import fp4
+    assert torch.cuda.is_available()
+    return torch, fp4, fp4.Kernels.load()
+
+
+def dev_u16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def bf16_to_f32(a):
+    return (a.astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_bits(x):
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def fp4_check_activations(m, k, g, seed):
+    """Gaussian with a few outliers, amax around the calibrated range 448 * 6 / g (fp4-check.rs:35-47)."""
+    rng = np.random.default_rng(seed)
+    sigma = 448.0 * 6.0 / g / 10.0
+    x = rng.normal(size=m * k).astype(np.float32) * np.float32(sigma)
+    x[::997] *= 6.0
+    x = x.reshape(m, k)
+    x[0, :16] = 0.0  # an all-zero block
+    return bf16_bits(x)
+
+
+@pytest.mark.parametrize("n,k,m,input_scale", [(256, 512, 200, 1.0), (128, 1024, 1, 0.037), (384, 256, 130, 2.5)])
+def test_fp4_linear(env, oracle, n, k, m, input_scale):
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    host = synth.fp4_linear(n, k, 11, input_scale=input_scale)
+    host.alpha[:] = host.alpha * np.linspace(0.5, 2.0, n).astype(np.float32)  # distinct per-column scales
+    lin = host.upload()
+    ws = fp4.Workspace(m, k)
+    xb = fp4_check_activations(m, k, lin.g, 3)
+    xd = dev_u16(torch, xb)
+    y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.forward(kern, ws, y, n, xd, k, m)
+    torch.cuda.synchronize()
+    yg = y.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    # (1) quantizer bit-exactness (fp4-check.rs:69-93); the reference tolerates < 0.1 % code bytes, here: none
+    codes, sf_tiled = ws.read(m, k)
+    sfa = oracle.untile_scales(sf_tiled, m, k // 16).reshape(m, k // 16)
+    want_codes, want_sf = oracle.quant_fp4(xb, lin.g)
+    assert np.array_equal(sfa, want_sf)
+    assert np.array_equal(codes, want_codes)
+    assert want_sf[0, 0] == 0 and not want_codes[0, :8].any()
+
+    # (2) GEMM vs the f64 reference over the same quantized operands (fp4-check.rs:95-144)
+    rows = sorted({r for r in (0, 1, 17, 127, 128, m // 2, m - 1) if r < m})
+    wf = oracle.dequant_fp4(host.codes, host.sf, 1.0)
+    aq = oracle.dequant_fp4(codes[rows], sfa[rows], 1.0)
+    refq = oracle.ref_gemm(aq, wf).astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+    got = bf16_to_f32(yg[rows]).astype(np.float64)
+    scale = np.abs(refq).max(axis=1, keepdims=True).clip(1e-20)
+    assert (np.abs(got - refq) / scale).max() < 8e-3
+    # the north-star bar: max relative error 1e-2 (bf16 out), floored at 1e-2 of the row maximum
+    assert (np.abs(got - refq) / np.maximum(np.abs(refq), 1e-2 * scale)).max() < 1e-2
+
+    # (3) residual epilogue, in place: y2 = bf16(bf16(x.W) + res), exact (fp4-check.rs:160-173)
+    res = bf16_bits(np.random.default_rng(5).normal(size=(m, n)).astype(np.float32))
+    y2 = dev_u16(torch, res)
+    lin.forward(kern, ws, y2, n, xd, k, m, res=y2)
+    torch.cuda.synchronize()
+    want = bf16_bits(bf16_to_f32(yg) + bf16_to_f32(res))
+    assert np.array_equal(y2.cpu().numpy().view(np.uint16), want)
+
+    # (4) canary: strided output inside a larger buffer, nothing outside rows < m, cols < n is written
+    # (fp4-check.rs:175-191)
+    ldy = n + 72
+    yc = torch.full(((m + 3), ldy), -21555, dtype=torch.int16, device="cuda")
+    lin.forward(kern, ws, yc, ldy, xd, k, m)
+    lin.forward(kern, ws, yc, ldy, xd, k, m, res=yc)
+    torch.cuda.synchronize()
+    ych = yc.cpu().numpy()
+    assert (ych[m:] == -21555).all() and (ych[:, n:] == -21555).all()
+    assert np.array_equal(ych[:m, :n].view(np.uint16), bf16_bits(bf16_to_f32(yg) + bf16_to_f32(yg)))
+
+    # (5) quantize once, gemm separately gives the same bits (lib.rs:518-543)
+    y3 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.quantize(kern, ws, xd, k, m)
+    lin.gemm(kern, ws, y3, n, m)
+    torch.cuda.synchronize()
+    assert np.array_equal(y3.view(torch.int16).cpu().numpy().view(np.uint16), yg)
+
+
+def test_fp4_argument_errors(env):
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    from ferrite_amd._lib import FeError
+    lin = synth.fp4_linear(128, 256, 1).upload()
+    ws = fp4.Workspace(8, 256)
+    x = dev_u16(torch, synth.activations(16, 256, 1))
+    y = torch.zeros((16, 136), dtype=torch.bfloat16, device="cuda")
+    lin.forward(kern, ws, y, 136, x, 256, 0)  # m == 0 is a no-op
+    with pytest.raises(FeError):
+        lin.forward(kern, ws, y, 136, x, 256, 9)  # workspace holds 8 rows
+    with pytest.raises(FeError):
+        lin.forward(kern, ws, y, 132, x, 256, 4)  # ldy % 8
+    with pytest.raises(FeError):
+        fp4.Workspace(8, 128) and lin.forward(kern, fp4.Workspace(8, 128), y, 136, x, 256, 4)  # k exceeds the workspace
+    lin.forward(kern, ws, y, 136, x, 256, 8)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y[:8, :128].float()).all()
