@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-prefill]
+
+Workload (BASELINE.json configs[1]): the EXL3 decode MLP of a Qwen3.8-27B-shaped layer at M = 1, at 3, 4 and 5 bits per
+weight: gate and up are K=5120 N=17408, down is K=17408 N=5120. One step = Linear::forward (input rotation + trellis
+GEMV) through all nine linears on seeded synthetic layers, inputs and weights resident in HBM. `value` is the trellis
+bytes streamed per second (the reference's numerator, crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step,
+launch gaps and input rotations included. The nine weight sets total 401 MB, more than L2 plus the 256 MB Infinity
+Cache, so every step streams its weights from HBM.
+
+`roofline` is the dominant kernel alone (the 4-bit GEMV of the 5120x17408 projections): its trellis bytes over its
+average launch duration, measured with HIP events on the launch stream inside the timed region.
+`cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host.
+`m2048` reports the prefill GEMMs (EXL3 4-bit and NVFP4, 5120x17408, M = 2048) in TFLOP/s against the bf16/f16 MFMA
+peak; it is measured after the timed region and is not part of `value`.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+SEED = 20251
+MLP = [("gate", 5120, 17408), ("up", 5120, 17408), ("down", 17408, 5120)]
+BITS = [3, 4, 5]
+
+
+class Events:
+    """HIP events through the C ABI, on the stream the kernels are launched on."""
+
+    def __init__(self, lib, check):
+        self.lib, self.check = lib, check
+
+    def new(self):
+        e = C.c_void_p()
+        self.check(self.lib.fe_hip_event_create(C.byref(e)))
+        return e
+
+    def record(self, e, stream):
+        self.check(self.lib.fe_hip_event_record(e, stream))
+
+    def ms(self, a, b):
+        self.check(self.lib.fe_hip_event_sync(b))
+        out = C.c_float()
+        self.check(self.lib.fe_hip_event_elapsed_ms(C.byref(out), a, b))
+        return out.value
+
+
+def cpu_baseline(sample_bits=4, k=5120, n=17408):
+    """The CPU oracle on the 4-bit gate projection at M = 1, all host cores (a bounded sample of the workload)."""
+    import numpy as np
+    import oracle
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(k, n, sample_bits, SEED, "gate")
+    o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+    x = (synth.activations(1, k, SEED).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    cores = oracle.default_threads(64)
+    t0 = time.perf_counter()
+    y = oracle.linear_f64(o, x, threads=cores)
+    dt = time.perf_counter() - t0
+    return {"value": round(t.trellis_bytes() / dt / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": f"oracle linear_f64 (decode_tile + f64 factored linear), EXL3 {sample_bits}-bit {k}x{n}, M=1, "
+                      f"{dt:.2f} s, threaded over 128-column blocks"}, y
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures the hot path on one GPU; --gpus must be 1 (no multi-GPU path exists)")
+
+    import numpy as np
+    import torch
+    from ferrite_amd import _lib, exl3, fp4, synth
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU")
+    cpu = None
+    if not args.no_cpu:
+        cpu, y_cpu = cpu_baseline()  # first, as the configuration asks
+
+    kern = exl3.Kernels.load()
+    lib = _lib.lib()
+    ev = Events(lib, _lib.check)
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    blocks = exl3.default_blocks(exl3.cu_count())
+
+    # the nine linears, one device copy each
+    linears = []
+    for bits in BITS:
+        for name, k, n in MLP:
+            t = synth.exl3_tensor(k, n, bits, SEED, name)
+            lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), blocks)
+            x = torch.from_numpy(synth.activations(1, k, SEED).view(np.int16)).cuda()
+            y = torch.zeros((1, n), dtype=torch.bfloat16, device="cuda")
+            linears.append((name, bits, lin, x, y))
+    ws = exl3.Workspace([l[2] for l in linears], 1)
+    total_bytes = sum(l[2].weight_bytes() for l in linears)
+
+    if cpu is not None:  # parity of the sampled layer on the GPU against the CPU result just computed
+        name, bits, lin, x, _ = next(l for l in linears if l[0] == "gate" and l[1] == 4)
+        yf = torch.zeros((1, lin.n), dtype=torch.float32, device="cuda")
+        lin.forward(x, exl3.Dtype.Bf16, yf, exl3.Dtype.F32, 1, ws)
+        torch.cuda.synchronize()
+        got = yf.cpu().numpy().astype(np.float64)
+        rel = float(np.abs(got - y_cpu).max() / np.sqrt((y_cpu ** 2).mean()))
+        cpu["gpu_vs_cpu_max_err_over_rms"] = round(rel, 6)
+
+    # an event pair around every GEMV launch of the timed region
+    events = [[(ev.new(), ev.new()) for _ in linears] for _ in range(args.steps)]
+
+    def step(timed_idx=None):
+        for li, (name, bits, lin, x, y) in enumerate(linears):
+            lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
+            if timed_idx is not None:
+                ev.record(events[timed_idx][li][0], stream)
+            lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
+            if timed_idx is not None:
+                ev.record(events[timed_idx][li][1], stream)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt * 1e3 / args.steps
+    value = total_bytes / (dt / args.steps) / 1e9
+
+    per, dom_ms = {}, []
+    for li, (name, bits, lin, x, y) in enumerate(linears):
+        ms = [ev.ms(*events[i][li]) for i in range(args.steps)]
+        us = sum(ms) / len(ms) * 1e3
+        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "sk": lin.plan.sk}
+        if bits == 4 and lin.k == 5120:
+            dom_ms += ms
+            dom_bytes = lin.weight_bytes()
+    dom_avg_ms = sum(dom_ms) / len(dom_ms)
+    achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
+
+    out = {
+        "metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "EXL3 decode MLP, Qwen3.8-27B-shaped layer, M=1, 3/4/5 bpw (gate, up 5120x17408; down 17408x5120)",
+                   "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
+        "roofline": {"bound": "hbm", "kernel": "exl3_gemv_b4_r1 (5120x17408, M=1)", "achieved": round(achieved, 2),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms)},
+        "cpu_baseline": cpu,
+        "per_linear_gemv": per,
+    }
+
+    if not args.no_prefill:
+        out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
+    print(json.dumps(out))
+
+
+def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=17408):
+    """EXL3 4-bit and NVFP4 GEMMs at M = 2048 (activations N(0,1) with 1 % outlier channels x20 for EXL3)."""
+    res = {}
+    flops = 2.0 * m * n * k
+    reps = 10
+    # EXL3
+    t = synth.exl3_tensor(k, n, 4, SEED, "gate")
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 1024)
+    ws = exl3.Workspace([lin], m)
+    x = torch.from_numpy(synth.activations(m, k, SEED, outliers=True).view(np.int16)).cuda()
+    y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.rotate_input(x, exl3.Dtype.Bf16, m, ws)
+    lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
+    a, b = ev.new(), ev.new()
+    ev.record(a, stream)
+    for _ in range(reps):
+        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
+    ev.record(b, stream)
+    ms = ev.ms(a, b) / reps
+    a2, b2 = ev.new(), ev.new()
+    ev.record(a2, stream)
+    for _ in range(reps):
+        lin.rotate_input(x, exl3.Dtype.Bf16, m, ws)
+    ev.record(b2, stream)
+    rot_ms = ev.ms(a2, b2) / reps
+    res["exl3_b4_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                                 "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "rot_in_ms": round(rot_ms, 4)}
+    del lin, ws, y
+    # NVFP4
+    fk = fp4.Kernels.load()
+    flin = synth.fp4_linear(n, k, SEED, input_scale=1.0).upload()
+    fws = fp4.Workspace(m, k)
+    xf = torch.from_numpy(synth.activations(m, k, SEED).view(np.int16)).cuda()
+    yf = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    flin.forward(fk, fws, yf, n, xf, k, m)
+    a, b = ev.new(), ev.new()
+    ev.record(a, stream)
+    for _ in range(reps):
+        flin.gemm(fk, fws, yf, n, m)
+    ev.record(b, stream)
+    ms = ev.ms(a, b) / reps
+    a2, b2 = ev.new(), ev.new()
+    ev.record(a2, stream)
+    for _ in range(reps):
+        flin.quantize(fk, fws, xf, k, m)
+    ev.record(b2, stream)
+    q_ms = ev.ms(a2, b2) / reps
+    res["nvfp4_17408x5120"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "quant_ms": round(q_ms, 4)}
+    return res
+
+
+if __name__ == "__main__":
+    main()

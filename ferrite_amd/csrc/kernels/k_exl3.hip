@@ -10,28 +10,13 @@
 
 // ---- the mul1 codebook ------------------------------------------------------------------------------------------
 
-#define MUL1_LO 0xD12Du
-#define MUL1_HI 0x83DCu
-
-typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
-
 // x = state * 0x83DCD12D mod 2^32 for the 16-bit state in the low (HI = 0) or high (HI = 1) half of r; the other half
-// of r may hold anything. Two full-rate instructions: a packed 16-bit multiply whose low lane is multiplied by zero
-// gives (state * 0x83DC) << 16, and a 16 x 16 + 32 multiply-add supplies state * 0xD12D.
+// of r may hold anything. On gfx950 v_mul_lo_u32 issues at the same rate as the other 3-operand integer instructions,
+// while the shift or mask that isolates the state is one of the double-rate simple instructions.
 template <int HI>
 __device__ __forceinline__ uint32_t mul1_x(uint32_t r) {
-    u16x2 rv = __builtin_bit_cast(u16x2, r);
-    uint16_t s = HI ? rv.y : rv.x;
-    u16x2 ss = {s, s};
-    u16x2 kk = {0, MUL1_HI};
-    uint32_t t = __builtin_bit_cast(uint32_t, (u16x2)(ss * kk));
-    uint32_t x;
-    const uint32_t mlo = MUL1_LO;
-    if (HI)
-        asm("v_mad_u32_u16 %0, %1, %2, %3 op_sel:[1,0,0,0]" : "=v"(x) : "v"(r), "s"(mlo), "v"(t));
-    else
-        asm("v_mad_u32_u16 %0, %1, %2, %3" : "=v"(x) : "v"(r), "s"(mlo), "v"(t));
-    return x;
+    uint32_t s = HI ? (r >> 16) : (r & 0xffffu);
+    return s * 0x83DCD12Du;
 }
 
 // Two codebook values as packed fp16 (x0's in the low half): 0x6400 + byte sum is fp16(1024 + sum); one fused
@@ -242,10 +227,15 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words(const uint32_t* run, 
 template <int BITS, int S>
 __device__ __forceinline__ uint32_t window32(const LaneWords<BITS>& lw) {
     constexpr int wi = S / 32, o = S % 32;
-    if constexpr (o == 0)
+    if constexpr (o == 0) {
         return lw.w[wi];
-    else
-        return __builtin_amdgcn_alignbit(lw.w[wi], lw.w[wi + 1], 32 - o);
+    } else {
+        uint32_t r = __builtin_amdgcn_alignbit(lw.w[wi], lw.w[wi + 1], 32 - o);
+        // opaque to the optimizer: two states share this window (one funnel shift for both); without this the
+        // compiler re-derives each state from the words with its own shift
+        asm("" : "+v"(r));
+        return r;
+    }
 }
 
 // x = state * MUL1 of local position U (0..31): its state ends at local stream bit (U + 1) * BITS + 32.
@@ -378,29 +368,39 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
             }
         }
         __syncthreads();
-        for (uint32_t s0 = 0; s0 < cs; s0 += DEPTH) {
+        auto mma = [&](const f16x8 (&op)[2][2], uint32_t sl) {
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                const unsigned char* xp = lds + xrow[rg] + sl * 128;
+                f16x8 x0 = *(const f16x8*)xp, x1 = *(const f16x8*)(xp + 16);
+                acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[rg][0], 0, 0, 0);
+                acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[rg][1], 0, 0, 0);
+                acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[rg][0], 0, 0, 0);
+                acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
+            }
+        };
+        // whole groups of DEPTH steps: no branches inside, and the refill of a ring slot is unconditional (the step
+        // index is clamped to the last one), so each load lands straight in the slot its words were just decoded from
+        const uint32_t full = cs / DEPTH * DEPTH;
+        for (uint32_t s0 = 0; s0 < full; s0 += DEPTH) {
 #pragma unroll
             for (int j = 0; j < DEPTH; j++) {
-                const uint32_t sl = s0 + j, s = c0 + sl;
-                if (sl < cs) {
-                    f16x8 op[2][2];
-                    decode_lane<BITS>(ring[j], op);
-                    if (s + DEPTH < steps) {
-                        const uint32_t* p = base + (size_t)(s + DEPTH) * step_words;
-                        ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
-                    }
-#pragma unroll
-                    for (int rg = 0; rg < RG; rg++) {
-                        const unsigned char* xp = lds + xrow[rg] + sl * 128;
-                        f16x8 x0 = *(const f16x8*)xp, x1 = *(const f16x8*)(xp + 16);
-                        acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[rg][0], 0, 0, 0);
-                        acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[rg][1], 0, 0, 0);
-                        acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[rg][0], 0, 0, 0);
-                        acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
-                    }
-                }
+                f16x8 op[2][2];
+                decode_lane<BITS>(ring[j], op);
+                uint32_t nxt = c0 + s0 + j + DEPTH;
+                nxt = nxt < steps ? nxt : steps - 1;
+                const uint32_t* p = base + (size_t)nxt * step_words;
+                ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
+                mma(op, s0 + j);
             }
         }
+#pragma unroll
+        for (int j = 0; j < DEPTH - 1; j++)  // the last chunk's remainder
+            if (full + j < cs) {
+                f16x8 op[2][2];
+                decode_lane<BITS>(ring[j], op);
+                mma(op, full + j);
+            }
     }
 
     // the block's sums -> LDS [row][128] (the input rows are no longer needed)
@@ -431,27 +431,33 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
         }
         return;
     }
+    // Split partials cross to another program, possibly on another XCD with its own L2: they are written and read with
+    // agent-scope accesses (write-through / L2-bypassing), ordered by the barrier around the arrival counter, so no
+    // device-wide cache write-back or invalidate is needed.
     for (uint32_t row = hw; row < m; row += 8) {
-        f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
-        *(f32x4*)(z + ((size_t)split * m + row) * n + col0 + 4 * l32) = t;
+        const float* src = red + row * GEMV_RED_PITCH + 4 * l32;
+        float* dst = z + ((size_t)split * m + row) * n + col0 + 4 * l32;
+#pragma unroll
+        for (int e = 0; e < 4; e++) __hip_atomic_store(dst + e, src[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __threadfence();
-    __syncthreads();
+    __syncthreads();  // every lane's stores are acknowledged (s_waitcnt vmcnt(0)) before the barrier
     if (tid == 0) {
-        uint32_t old = atomicAdd(&counters[nb], 1u);
+        uint32_t old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_flag = (old == sk - 1);
     }
     __syncthreads();
     if (last_flag) {
-        __threadfence();
         for (uint32_t row = hw; row < m; row += 8) {
             size_t at = (size_t)row * n + col0 + 4 * l32;
-            f32x4 t = __builtin_nontemporal_load((const f32x4*)(z + at));
-            for (uint32_t sp = 1; sp < sk; sp++) t += __builtin_nontemporal_load((const f32x4*)(z + (size_t)sp * m * n + at));
-            float v[4] = {t[0], t[1], t[2], t[3]};
+            float v[4] = {0.f, 0.f, 0.f, 0.f};
+            for (uint32_t sp = 0; sp < sk; sp++) {
+                const float* src = z + (size_t)sp * m * n + at;
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] += __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
             finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, at);
         }
-        if (tid == 0) counters[nb] = 0;
+        if (tid == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 

