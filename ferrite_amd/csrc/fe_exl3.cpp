@@ -14,6 +14,7 @@
 namespace {
 
 constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
+constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 128 * 132 * 4;  // epilogue tile of the prefill GEMM (covers the A/B tiles too)
@@ -39,6 +40,8 @@ struct fe_exl3_kernels {
     fe_function_t rot_in = nullptr, probe_v4 = nullptr;
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
+    fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
+    uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     uint32_t group_m = 8;
 };
@@ -47,6 +50,7 @@ struct fe_exl3_linear {
     std::string name;
     uint32_t k = 0, n = 0, bits = 0;
     fe_exl3_plan plan{};
+    uint32_t programs = 0;  // grid of the streamed GEMV (plan.ver == 2)
     fe_exl3_view view{};
     FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
     const fe_exl3_kernels *kern = nullptr;
@@ -103,11 +107,18 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
             get(&k->gemv[i][rg - 1], nm);
             if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv[i][rg - 1], 64 * 1024);
         }
+        snprintf(nm, sizeof nm, "exl3_gemv_stream_b%d", kBits[i]);
+        get(&k->gemv_stream[i], nm);
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
     }
     if (const char *g = getenv("FE_EXL3_GROUP")) k->group_m = (uint32_t)atoi(g);
+    if (!c) {
+        int cus = 0;
+        c = fe_hip_cu_count(&cus);
+        k->cus = (uint32_t)cus;
+    }
     if (c) {
         fe_exl3_kernels_destroy(k);
         return c;
@@ -138,7 +149,10 @@ int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_
         if (nb * d >= blocks) break;
     }
     if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) sk = 1;
-    *out = fe_exl3_plan{sk, 4, 1, 0};
+    // ver 2: rows 1..16 run the streamed GEMV with occ programs per CU (FE_EXL3_STREAM=0: the split-K form only)
+    uint32_t ver = env_is("FE_EXL3_STREAM", "0") ? 1 : 2, occ = 2;
+    if (const char *o = getenv("FE_EXL3_OCC")) occ = (uint32_t)atoi(o);
+    *out = fe_exl3_plan{sk, 4, ver, ver == 2 ? occ : 0};
     return 0;
 }
 
@@ -149,6 +163,15 @@ int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out) {
     if (got < 2) return fe_set_error(FE_ERR_ARG, "fe_exl3_plan_parse", s);
     *out = fe_exl3_plan{v[0], v[1], v[2], v[3]};
     return 0;
+}
+
+// Programs of the streamed GEMV: occ per CU, at most one per eight work units (FE_EXL3_PROGRAMS overrides the count).
+static uint32_t stream_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p, uint32_t k, uint32_t n) {
+    if (p.ver != 2) return 0;
+    const uint32_t units = (k / 64) * (n / 128), occ = p.occ ? p.occ : 2;
+    uint32_t progs = std::min(occ * kern->cus, units / 8);
+    if (const char *e = getenv("FE_EXL3_PROGRAMS")) progs = std::min((uint32_t)atoi(e), units);  // tuning and tests
+    return std::max(1u, progs);
 }
 
 static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, const fe_exl3_plan &p) {
@@ -175,6 +198,7 @@ int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, 
     l->plan = *plan;
     l->view = *view;
     l->kern = kern;
+    l->programs = stream_programs(kern, *plan, view->k, view->n);
     *out = l;
     return 0;
 }
@@ -192,6 +216,7 @@ int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, con
     auto *l = new fe_exl3_linear;
     l->name = name ? name : "";
     l->k = k, l->n = n, l->bits = bits, l->plan = p, l->kern = kern;
+    l->programs = stream_programs(kern, p, k, n);
     const size_t tw = 8 * (size_t)bits, kt = k / 16, nt = n / 16, words = kt * nt * tw;
     int c = 0;
     if (strips) {
@@ -231,16 +256,17 @@ size_t fe_exl3_linear_weight_bytes(const fe_exl3_linear *l) { return l ? (size_t
 
 int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows) {
     if (!out || (count && !linears) || !max_rows) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_create", "bad argument");
-    size_t max_k = 128, max_z = 0, max_nb = 1;
+    size_t max_k = 128, max_z = 0, max_zs = 0, max_nb = 1;
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
         max_k = std::max<size_t>(max_k, l->k);
         if (l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
+        if (l->programs) max_zs = std::max<size_t>(max_zs, (size_t)(l->programs + l->n / 128) * 128);
         max_nb = std::max<size_t>(max_nb, l->n / 128);
     }
     auto *ws = new fe_exl3_workspace;
     ws->max_rows = max_rows, ws->max_k = (uint32_t)max_k;
-    ws->z_len = std::max<size_t>(max_z * std::min(max_rows, kMaxRowsPerPass), 4);
+    ws->z_len = std::max<size_t>(std::max(max_z * std::min(max_rows, kMaxRowsPerPass), max_zs * std::min(max_rows, kStreamRows)), 4);
     ws->counters_len = (size_t)((max_rows + 7) / 8) * max_nb;
     int c = ws->xh.alloc((size_t)max_rows * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
@@ -305,6 +331,18 @@ int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devpt
             return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
         }
         return launch_gemm(l, s, xh, y, y_dtype, rows);
+    }
+    if (p.ver == 2 && rows >= 1 && rows <= kStreamRows) {
+        if (rows > ws->max_rows || ws->z_len < (size_t)(l->programs + l->n / 128) * 128 * rows || ws->counters_len < l->n / 128) {
+            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u, z %zu)", l->name.c_str(), rows, ws->max_rows,
+                     ws->z_len);
+            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
+        }
+        uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb;
+        view_strides(l->view, &stride_k, &stride_nb);
+        fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
+        void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &mode, &stride_k, &stride_nb};
+        return fe_hip_launch(l->kern->gemv_stream[bits_slot(l->bits)], l->programs, 1, 1, 256, 1, 1, 0, s, args);
     }
     // linear.rs:302-307
     if (rows == 0 || rows > ws->max_rows || (p.sk > 1 && ws->z_len < (size_t)p.sk * rows * l->n)) {

@@ -323,7 +323,8 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
     constexpr uint32_t tw = 8 * BITS;
-    constexpr int DEPTH = 4;  // load steps in flight per lane
+    constexpr int DEPTH = 4;   // load steps in flight per lane
+    constexpr int GROUP = 16;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
     const uint32_t nbs = n / 128, nb = blockIdx.x % nbs, split = blockIdx.x / nbs;
@@ -379,28 +380,40 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
                 acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
             }
         };
-        // whole groups of DEPTH steps: no branches inside, and the refill of a ring slot is unconditional (the step
-        // index is clamped to the last one), so each load lands straight in the slot its words were just decoded from
-        const uint32_t full = cs / DEPTH * DEPTH;
-        for (uint32_t s0 = 0; s0 < full; s0 += DEPTH) {
+        // Whole groups of GROUP steps run as straight-line code: no branches inside, and the refill of a ring slot is
+        // unconditional (the step index is clamped to the last one), so each load lands straight in the slot its words
+        // were just decoded from and only that slot's next use waits for it. The wait at the top of a group has to
+        // cover every load in flight (the compiler cannot count across the back edge), hence long groups.
+        const uint32_t full = cs / GROUP * GROUP;
+        for (uint32_t s0 = 0; s0 < full; s0 += GROUP) {
 #pragma unroll
-            for (int j = 0; j < DEPTH; j++) {
+            for (int j = 0; j < GROUP; j++) {
                 f16x8 op[2][2];
-                decode_lane<BITS>(ring[j], op);
+                decode_lane<BITS>(ring[j % DEPTH], op);
                 uint32_t nxt = c0 + s0 + j + DEPTH;
                 nxt = nxt < steps ? nxt : steps - 1;
                 const uint32_t* p = base + (size_t)nxt * step_words;
-                ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
+                ring[j % DEPTH] = load_lane_words<BITS>(p + run_off, p + prev_off);
+                // keep each refill where it is issued: left alone, the scheduler sinks the loads to the end of the
+                // group, right in front of the wait for them
+                __builtin_amdgcn_sched_barrier(0);
                 mma(op, s0 + j);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        for (uint32_t s0 = full; s0 < cs; s0 += DEPTH) {  // the remainder, slot by slot
 #pragma unroll
-        for (int j = 0; j < DEPTH - 1; j++)  // the last chunk's remainder
-            if (full + j < cs) {
-                f16x8 op[2][2];
-                decode_lane<BITS>(ring[j], op);
-                mma(op, full + j);
-            }
+            for (int j = 0; j < DEPTH; j++)
+                if (s0 + j < cs) {
+                    f16x8 op[2][2];
+                    decode_lane<BITS>(ring[j], op);
+                    uint32_t nxt = c0 + s0 + j + DEPTH;
+                    nxt = nxt < steps ? nxt : steps - 1;
+                    const uint32_t* p = base + (size_t)nxt * step_words;
+                    ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
+                    mma(op, s0 + j);
+                }
+        }
     }
 
     // the block's sums -> LDS [row][128] (the input rows are no longer needed)
@@ -475,6 +488,200 @@ GEMV_FAMILY(4)
 GEMV_FAMILY(5)
 GEMV_FAMILY(6)
 GEMV_FAMILY(8)
+
+// ---- decode GEMV, streamed over the whole tensor (1..16 rows) -------------------------------------------------------------
+//
+// Work unit = one load step (64 input channels) of one 128-column block; units are ordered column block by column block
+// (in the strips layout that is the byte order of the trellis), and the gridDim.x programs each take one contiguous,
+// equally long run of them, whatever the shape: every CU streams the same number of bytes. A run may start and end in
+// the middle of a column block, so a block's sum is assembled from segments: each wavefront of each segment leaves its
+// partial sums in z[program + block] and bumps the block's arrival counter; the wavefront that arrives last adds the
+// segments in order, applies the output rotation and re-arms the counter. The four wavefronts of a program own two tiles
+// of the block each and never exchange data: no LDS, no barriers; the rotated inputs come straight from L2 with the
+// weights, one ring slot per load step.
+
+template <int BITS>
+struct StreamSlot {
+    LaneWords<BITS> w;
+    f16x8 x0, x1;  // rotated inputs of the lane's input row, k 0..7 and 8..15 of the lane's k step
+    // member-wise copy: a whole-struct copy would also move the padding bytes and pin them to the stack
+    __device__ __forceinline__ void take(const StreamSlot& o) {
+#pragma unroll
+        for (int i = 0; i <= BITS; i++) w.w[i] = o.w.w[i];
+        x0 = o.x0, x1 = o.x1;
+    }
+};
+
+// Program that owns unit u when U units are dealt as base + 1 to the first rem programs and base to the rest.
+__device__ __forceinline__ uint32_t stream_owner(uint32_t u, uint32_t base, uint32_t rem) {
+    uint32_t cut = rem * (base + 1);
+    return u < cut ? u / (base + 1) : rem + (u - cut) / base;
+}
+
+template <int BITS>
+__device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
+                                                 const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
+                                                 uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t stride_k,
+                                                 uint32_t stride_nb) {
+    constexpr uint32_t tw = 8 * BITS;
+    constexpr int DEPTH = 4;  // load steps in flight per lane
+    constexpr int GROUP = 8;  // steps of straight-line code per loop iteration
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
+    const uint32_t steps = k / 64, nbs = n / 128, units = nbs * steps;
+    const uint32_t progs = gridDim.x, p = blockIdx.x;
+    const uint32_t base = units / progs, rem = units % progs;
+    const uint32_t u0 = p * base + (p < rem ? p : rem), u1 = u0 + base + (p < rem ? 1 : 0);
+    if (u0 >= u1) return;
+    // arrivals of this program's wavefronts per column block touched (index: block - first block, wrapped)
+    __shared__ uint32_t arrived[64];
+    if (tid < 64) arrived[tid] = 0;
+    __syncthreads();
+    const uint32_t nb_first = u0 / steps;
+
+    const uint32_t lane_word = (2 * wave + tau) * tw, run_off = lane_word + q * BITS, prev_off = lane_word + (q * BITS + tw - 1) % tw;
+    const uint16_t* xrow = xh + (size_t)(r < m ? r : m - 1) * k + g * 16;
+
+    // refill cursor: the next unit to request, as (column block, step)
+    uint32_t ru = u0, rnb = u0 / steps, rst = u0 % steps;
+    auto issue = [&](StreamSlot<BITS>& slot) {
+        const uint32_t* wp = trellis + (size_t)rnb * stride_nb + (size_t)(4 * rst + g) * stride_k;
+        slot.w = load_lane_words<BITS>(wp + run_off, wp + prev_off);
+        const uint16_t* xp = xrow + rst * 64;
+        slot.x0 = *(const f16x8*)xp;
+        slot.x1 = *(const f16x8*)(xp + 8);
+        if (ru + 1 < u1) {  // past the end of the run the last unit is requested again (and never used)
+            ru++;
+            if (++rst == steps) rst = 0, rnb++;
+        }
+    };
+
+    StreamSlot<BITS> ring[DEPTH];
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) issue(ring[j]);
+
+    f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    auto one = [&](StreamSlot<BITS>& slot) {
+        f16x8 op[2][2];
+        decode_lane<BITS>(slot.w, op);
+        f16x8 x0 = slot.x0, x1 = slot.x1;
+        issue(slot);
+        __builtin_amdgcn_sched_barrier(0);  // the refill stays here, ahead of the matrix work
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[1], 0, 0, 0);
+        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[0], 0, 0, 0);
+        acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint32_t u = u0, nb = u0 / steps, st = u0 % steps;
+    while (u < u1) {
+        const uint32_t seg = (steps - st < u1 - u) ? steps - st : u1 - u;  // units left in this column block
+        const uint32_t full = seg / GROUP * GROUP;
+        for (uint32_t i = 0; i < full; i += GROUP) {
+#pragma unroll
+            for (int j = 0; j < GROUP; j++) one(ring[j % DEPTH]);
+        }
+        const uint32_t tail = seg - full;
+        for (uint32_t i = 0; i < tail; i += DEPTH) {
+#pragma unroll
+            for (int j = 0; j < DEPTH; j++)
+                if (i + j < tail) one(ring[j]);
+        }
+
+        // segment end: partial sums of this wavefront's 32 columns -> z[program + block][row][128]
+        const uint32_t col0 = nb * 128;
+        const uint32_t first_prog = stream_owner(nb * steps, base, rem), last_prog = stream_owner(nb * steps + steps - 1, base, rem);
+        if (r < m) {
+            float* zp = z + ((size_t)(p + nb) * m + r) * 128 + 32 * wave;
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t arow = 4 * g + i;  // row of A: tile arow >> 3 of the pair, n = (arow & 7) + 8 h
+                    __hip_atomic_store(zp + 16 * (arow >> 3) + (arow & 7) + 8 * h, acc[h][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+        }
+        acc[0] = acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums are acknowledged at agent scope
+        // the program's four wavefronts meet on an LDS counter; the last of them reports the segment to the block's
+        // global arrival counter, and the last segment to arrive finishes the block
+        uint32_t old = 0;
+        if (lane == 0) old = __hip_atomic_fetch_add(&arrived[(nb - nb_first) & 63], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        old = __builtin_amdgcn_readfirstlane(old);
+        bool finisher = false;
+        if (old == 3) {
+            uint32_t g_old = 0;
+            if (lane == 0) g_old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            finisher = __builtin_amdgcn_readfirstlane(g_old) == last_prog - first_prog;
+        }
+        if (finisher) {
+            // add the segments in program order, rotate, scale, store; two rows at a time, 8 segments' loads in flight
+            const uint32_t l32 = lane & 31;
+            for (uint32_t row0 = 0; row0 < m; row0 += 2) {
+                const uint32_t row = row0 + (lane >> 5);
+                const bool live = row < m;
+                float v[4] = {0.f, 0.f, 0.f, 0.f};
+                for (uint32_t sp0 = first_prog; sp0 <= last_prog; sp0 += 8) {
+                    float t[8][4];
+#pragma unroll
+                    for (int b = 0; b < 8; b++) {
+                        const uint32_t sp = sp0 + b <= last_prog ? sp0 + b : last_prog;
+                        const float* src = z + ((size_t)(sp + nb) * m + (live ? row : 0)) * 128 + 4 * l32;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) t[b][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+#pragma unroll
+                    for (int b = 0; b < 8; b++)
+                        if (sp0 + b <= last_prog) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[e] += t[b][e];
+                        }
+                }
+                fwht128_half_wave(v, l32);
+                if (live) {
+                    u32x2 sv = *(const u32x2*)(svh + col0 + 4 * l32);
+                    v[0] = v[0] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] & 0xffff);
+                    v[1] = v[1] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] >> 16);
+                    v[2] = v[2] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] & 0xffff);
+                    v[3] = v[3] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] >> 16);
+                    store4(y, y_mode, (size_t)row * n + col0 + 4 * l32, v);
+                }
+            }
+            if (lane == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+
+        // the next unit sits in slot tail % DEPTH: turn the ring so that it is slot 0 again (nothing is in flight here)
+        const uint32_t phase = tail % DEPTH;
+        if (phase == 1) {
+            StreamSlot<BITS> t;
+            t.take(ring[0]), ring[0].take(ring[1]), ring[1].take(ring[2]), ring[2].take(ring[3]), ring[3].take(t);
+        } else if (phase == 2) {
+            StreamSlot<BITS> t0, t1;
+            t0.take(ring[0]), t1.take(ring[1]);
+            ring[0].take(ring[2]), ring[1].take(ring[3]), ring[2].take(t0), ring[3].take(t1);
+        } else if (phase == 3) {
+            StreamSlot<BITS> t;
+            t.take(ring[3]), ring[3].take(ring[2]), ring[2].take(ring[1]), ring[1].take(ring[0]), ring[0].take(t);
+        }
+        u += seg;
+        st += seg;
+        if (st == steps) st = 0, nb++;
+    }
+}
+
+#define GEMV_STREAM_KERNEL(BITS)                                                                                       \
+    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_stream_b##BITS(                                     \
+        const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,        \
+        uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb) {                   \
+        gemv_stream_body<BITS>(xh, trellis, svh, y, z, counters, n, k, m, y_mode, stride_k, stride_nb);                \
+    }
+GEMV_STREAM_KERNEL(2)
+GEMV_STREAM_KERNEL(3)
+GEMV_STREAM_KERNEL(4)
+GEMV_STREAM_KERNEL(5)
+GEMV_STREAM_KERNEL(6)
+GEMV_STREAM_KERNEL(8)
 
 // ---- prefill GEMM ----------------------------------------------------------------------------------------------------
 

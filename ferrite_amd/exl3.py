@@ -179,8 +179,8 @@ class Kernels:
         return cls()
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_exl3_kernels_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_exl3_kernels_destroy(self.h)
             self.h = None
 
     def reconstruct_hat_f16(self, view: Exl3View, out, stream=None):
@@ -246,8 +246,8 @@ class Linear:
         return cls(kern, name, view, plan)
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_exl3_linear_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_exl3_linear_destroy(self.h)
             self.h = None
 
     def weight_bytes(self):
@@ -286,6 +286,6 @@ class Workspace:
         return out
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_exl3_workspace_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_exl3_workspace_destroy(self.h)
             self.h = None

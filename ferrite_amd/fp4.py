@@ -103,8 +103,8 @@ class Kernels:
         return cls()
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_fp4_kernels_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_fp4_kernels_destroy(self.h)
             self.h = None
 
 
@@ -130,8 +130,8 @@ class Workspace:
         return codes, sf
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_fp4_workspace_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_fp4_workspace_destroy(self.h)
             self.h = None
 
 
@@ -148,8 +148,8 @@ class PromptLinear:
                                               alpha.ctypes.data_as(C.c_void_p), host.g))
 
     def __del__(self):
-        if getattr(self, "h", None):
-            _lib.lib().fe_fp4_linear_destroy(self.h)
+        if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
+            _lib._lib.fe_fp4_linear_destroy(self.h)
             self.h = None
 
     def forward(self, kern, ws, y, ldy, x, lda, m, res=None, stream=None):

@@ -102,7 +102,7 @@ def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
     assert not far.any() and (xh_gpu != xh_ref).mean() < 2e-3
     hat = oracle.w_hat_f16(o)
     yref = oracle.gemv_ref(o, hat, xh_gpu)  # on the GPU's own rotated input: what is left is fp32 summation order
-    first5 = None
+    first5 = {}
     for rows in rows_list:
         y = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.F32).cpu().numpy().astype(np.float64)
         yb = run_forward(torch, exl3, lin, ws, xd, rows, exl3.Dtype.Bf16).view(torch.int16).cpu().numpy().view(np.uint16)
@@ -118,11 +118,13 @@ def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
         # rows past `rows` untouched (exl3-gemvcheck.rs:113-116)
         if rows < 64:
             assert np.isnan(y[rows:]).all()
-        if rows >= 5:  # row invariance (exl3-gemvcheck.rs:124-141)
-            if first5 is None:
-                first5 = y[:5].copy()
+        if rows >= 5:  # row invariance (exl3-gemvcheck.rs:124-141): a row's bits do not depend on the row count
+            # (plan ver 2 sums rows 1..16 in the streamed order and 17..64 in the split order: invariant within each)
+            regime = 1 if (plan.ver == 2 and rows <= 16) else 0
+            if regime not in first5:
+                first5[regime] = y[:5].copy()
             else:
-                assert np.array_equal(first5.view(np.uint64), y[:5].view(np.uint64)), rows
+                assert np.array_equal(first5[regime].view(np.uint64), y[:5].view(np.uint64)), rows
     # fused residual add: y (bf16, prefilled with 1.5) += x @ W, 5 rows (exl3-gemvcheck.rs:142-168)
     rows = 5
     pre = torch.full((mr, t.n), 1.5, dtype=torch.bfloat16, device="cuda")
@@ -138,11 +140,24 @@ def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
-def test_gemv_all_bit_widths(env, oracle, bits):
+@pytest.mark.parametrize("ver", [1, 2])
+def test_gemv_all_bit_widths(env, oracle, bits, ver):
+    """ver 1: split-K programs per column block; ver 2: rows 1..16 streamed over the whole tensor."""
     torch, exl3, kern = env
     from ferrite_amd import synth
     t = synth.exl3_tensor(512, 256, bits, 20 + bits)
-    check_linear(env, oracle, t, exl3.Plan(2), strips=True, rows_list=[1, 5, 16, 17, 64])
+    check_linear(env, oracle, t, exl3.Plan(2, 4, ver, 2), strips=True, rows_list=[1, 5, 16, 17, 64])
+
+
+@pytest.mark.parametrize("programs,strips", [(1, True), (5, True), (7, False), (13, True), (48, False), (1000, True)])
+def test_streamed_gemv_any_partition(env, oracle, programs, strips, monkeypatch):
+    """The streamed GEMV cuts the tensor's 48 work units (3 column blocks x 16 load steps) into runs of any length:
+    runs that start and end inside a block, cover whole blocks, or are a single unit."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    monkeypatch.setenv("FE_EXL3_PROGRAMS", str(programs))
+    t = synth.exl3_tensor(1024, 384, 4, 77)
+    check_linear(env, oracle, t, exl3.Plan(4, 4, 2, 2), strips=strips, rows_list=[1, 2, 5, 8, 9, 16])
 
 
 @pytest.mark.parametrize("sk,strips", [(1, True), (1, False), (4, True), (8, False), (16, True)])
