@@ -17,7 +17,7 @@ constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
 constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
-constexpr uint32_t kGemmLds = 128 * 132 * 4;  // epilogue tile of the prefill GEMM (covers the A/B tiles too)
+constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
 
 bool env_is(const char *name, const char *v) {
     const char *e = getenv(name);
@@ -43,6 +43,7 @@ struct fe_exl3_kernels {
     fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
+    fe_function_t gemm_reduce = nullptr;
     uint32_t group_m = 8;
 };
 
@@ -58,7 +59,7 @@ struct fe_exl3_linear {
 
 struct fe_exl3_workspace {
     uint32_t max_rows = 0, max_k = 0;
-    FeBuf xh, z, counters;
+    FeBuf xh, z, counters, part;  // part: partial tiles of the prefill GEMM (rows > 64 only)
     size_t z_len = 0, counters_len = 0;
 };
 
@@ -112,6 +113,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
+        if (i == 0) get(&k->gemm_reduce, "exl3_gemm_reduce");
     }
     if (const char *g = getenv("FE_EXL3_GROUP")) k->group_m = (uint32_t)atoi(g);
     if (!c) {
@@ -271,6 +273,9 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     int c = ws->xh.alloc((size_t)max_rows * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
+    int cus = 0;
+    if (!c && max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
+    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
     if (c) {
         delete ws;
         return c;
@@ -308,15 +313,23 @@ int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *
     return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
 }
 
-static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows) {
+static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
+                       const fe_exl3_workspace *ws) {
     const fe_exl3_kernels *kern = l->kern;
     uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb, group = kern->group_m;
     view_strides(l->view, &stride_k, &stride_nb);
-    uint32_t tiles_m = (rows + 127) / 128;
+    if ((uint64_t)rows * k * 2 >= (1ull << 32))
+        return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear_gemv_rotated", "rotated input of 4 GB or more");
+    const uint32_t tiles_m = (rows + 255) / 256, tiles_n = (n / 128 + 1) / 2;
     if (group == 0 || group > tiles_m) group = tiles_m;
-    fe_devptr_t tr = l->view.trellis, svh = l->view.svh;
-    void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group};
-    return fe_hip_launch(kern->gemm[bits_slot(l->bits)], tiles_m * (n / 128), 1, 1, 256, 1, 1, kGemmLds, s, args);
+    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    uint32_t full = g.full, splits = g.splits;
+    fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
+    void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &full, &splits, &part};
+    FE_TRY(fe_hip_launch(kern->gemm[bits_slot(l->bits)], g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (!g.cut()) return 0;
+    void *rargs[] = {&part, &svh, &y, &n, &rows, &mode, &group, &full, &splits};
+    return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
@@ -330,7 +343,7 @@ int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devpt
             snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
             return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
         }
-        return launch_gemm(l, s, xh, y, y_dtype, rows);
+        return launch_gemm(l, s, xh, y, y_dtype, rows, ws);
     }
     if (p.ver == 2 && rows >= 1 && rows <= kStreamRows) {
         if (rows > ws->max_rows || ws->z_len < (size_t)(l->programs + l->n / 128) * 128 * rows || ws->counters_len < l->n / 128) {

@@ -4,19 +4,23 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <string>
+#include <vector>
 
 #include "fe_exl3.h"  // error codes
 #include "fe_internal.h"
 
 namespace {
 constexpr uint32_t kTile = 128;                 // crates/fe-fp4/src/lib.rs:28
-constexpr uint32_t kGemmLds = 2 * 128 * 72 * 2;  // GM_LDS_TILES
+constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // GM_LDS_TILES: two k tiles of A and W, 256 rows each
+constexpr uint32_t kTileM = 256;                        // GM_BM
+constexpr uint32_t kTileN = 256;                        // GM_BN
 }  // namespace
 
 struct fe_fp4_kernels {
     fe_module_t module = nullptr;
-    fe_function_t quant4 = nullptr, gemm4 = nullptr;
+    fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr;
     uint32_t group_m = 8;  // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
 };
 
@@ -25,11 +29,13 @@ struct fe_fp4_linear {
     uint32_t n = 0, k = 0;
     float g = 1.0f;
     FeBuf w, sw, alpha;
+    // byte strides of the codes / scales of (128-row tile, 64-wide k tile, row in tile); see fe_gemm_nvfp4
+    uint32_t w_snt = 0, w_skt = 0, w_sr = 0, s_snt = 0, s_skt = 0, s_sr = 0;
 };
 
 struct fe_fp4_workspace {
     uint32_t max_rows = 0, max_k = 0;
-    FeBuf codes, sf, aq;
+    FeBuf codes, sf, aq, part;  // part: partial tiles of the GEMM, one slot a CU
 };
 
 extern "C" {
@@ -40,6 +46,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     int c = fe_load_module(&k->module, "FE_FP4_HSACO", fe_k_fp4_hsaco, fe_k_fp4_hsaco_end);
     if (!c) c = fe_hip_module_get_function(&k->quant4, k->module, "fe_fp4_quant");
     if (!c) c = fe_hip_module_get_function(&k->gemm4, k->module, "fe_gemm_nvfp4");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm4, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->reduce4, k->module, "fe_gemm_nvfp4_reduce");
     if (const char *g = getenv("FE_FP4_GROUP")) k->group_m = (uint32_t)atoi(g);
     if (c) {
         fe_fp4_kernels_destroy(k);
@@ -73,8 +81,22 @@ int fe_fp4_linear_upload(fe_fp4_linear **out, const char *name, uint32_t n, uint
     auto *l = new fe_fp4_linear;
     l->name = name ? name : "";
     l->n = n, l->k = k, l->g = g;
-    int c = l->w.from_host(codes, (size_t)n * k / 2);
-    if (!c) c = l->sw.from_host(scales, (size_t)n * k / 16);
+    // k-tile-major device layout: the 128 rows of a tile contribute 32 bytes of codes (4 scales) each to one k tile,
+    // stored contiguously, so a program's weight read for a k tile is one 4 KB (512 byte) run
+    const uint32_t kts = k / 64, nts = n / kTile;
+    std::vector<uint8_t> wt((size_t)n * k / 2), st((size_t)n * k / 16);
+    for (uint32_t nt = 0; nt < nts; nt++)
+        for (uint32_t r = 0; r < kTile; r++) {
+            const uint8_t *wrow = codes + (size_t)(nt * kTile + r) * (k / 2), *srow = scales + (size_t)(nt * kTile + r) * (k / 16);
+            for (uint32_t kt = 0; kt < kts; kt++) {
+                memcpy(&wt[(((size_t)nt * kts + kt) * kTile + r) * 32], wrow + kt * 32, 32);
+                memcpy(&st[(((size_t)nt * kts + kt) * kTile + r) * 4], srow + kt * 4, 4);
+            }
+        }
+    l->w_snt = kts * kTile * 32, l->w_skt = kTile * 32, l->w_sr = 32;
+    l->s_snt = kts * kTile * 4, l->s_skt = kTile * 4, l->s_sr = 4;
+    int c = l->w.from_host(wt.data(), wt.size());
+    if (!c) c = l->sw.from_host(st.data(), st.size());
     if (!c) c = l->alpha.from_host(alpha, (size_t)n * 4);
     if (c) {
         delete l;
@@ -94,6 +116,9 @@ int fe_fp4_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, u
     l->w.view(codes, (size_t)n * k / 2);
     l->sw.view(scales, (size_t)n * k / 16);
     l->alpha.view(alpha, (size_t)n * 4);
+    // the format's row-major layout, read in place
+    l->w_snt = kTile * (k / 2), l->w_skt = 32, l->w_sr = k / 2;
+    l->s_snt = kTile * (k / 16), l->s_skt = 4, l->s_sr = k / 16;
     *out = l;
     return 0;
 }
@@ -120,6 +145,9 @@ int fe_fp4_workspace_create(fe_fp4_workspace **out, uint32_t max_rows, uint32_t 
     int c = ws->codes.alloc(rp * max_k);
     if (!c) c = ws->sf.zeroed(rp * max_k / 16);
     if (!c) c = ws->aq.alloc(rp * max_k * 2);
+    int cus = 0;
+    if (!c) c = fe_hip_cu_count(&cus);
+    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
     if (c) {
         delete ws;
         return c;
@@ -170,11 +198,21 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     if (!y || ldy % 8 || y % 16 || (res && res % 16) || ldy < l->n)
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
-    const uint32_t tiles_m = (m + kTile - 1) / kTile;
+    if ((uint64_t)m * k * 2 >= (1ull << 32) || (uint64_t)n * k / 2 >= (1ull << 32))
+        return fe_set_error(FE_ERR_UNSUPPORTED, "fe_fp4_linear_gemm", "operand of 4 GB or more");
+    const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
     uint32_t group = kern->group_m == 0 || kern->group_m > tiles_m ? tiles_m : kern->group_m;  // lib.rs:148-151
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
-    void *args[] = {&y, &aq, &w, &sw, &alpha, &res, &m, &n, &k, &ldy, &group};
-    return fe_hip_launch(kern->gemm4, tiles_m * (n / kTile), 1, 1, 256, 1, 1, kGemmLds, s, args);
+    uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    uint32_t full = gs.full, splits = gs.splits;
+    fe_devptr_t part = ws->part.p;
+    void *args[] = {&y,     &aq,    &w,    &sw,    &alpha, &res,  &m,      &n,   &k, &ldy,
+                    &group, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr, &full, &splits, &part};
+    FE_TRY(fe_hip_launch(kern->gemm4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (!gs.cut()) return 0;
+    void *rargs[] = {&y, &part, &alpha, &res, &m, &n, &ldy, &group, &full, &splits};
+    return fe_hip_launch(kern->reduce4, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 int fe_fp4_linear_forward(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,

@@ -2,6 +2,7 @@
 #pragma once
 #include <cstddef>
 #include <cstdint>
+#include <cstdlib>
 
 #include "fe_hip.h"
 
@@ -62,3 +63,29 @@ struct FeBuf {
         owned = false;
     }
 };
+
+// How the prefill GEMM's output tiles (256 x 256) are spread over the CUs: `full` tiles are computed whole, one per
+// program; the `tiles - full` tiles of a last, mostly empty round are each cut `splits` ways along K (partials in a
+// workspace, then a reduce kernel). splits == 1 means nothing is cut (full == tiles).
+struct FeGemmSplit {
+    uint32_t tiles = 0, full = 0, splits = 1;
+    uint32_t programs() const { return full + (tiles - full) * splits; }
+    uint32_t cut() const { return tiles - full; }
+};
+constexpr size_t kFeGemmPartBytes = 256 * 256 * 4;  // one partial slot
+// at most `cus` slots are ever used
+inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus) {
+    FeGemmSplit g;
+    g.tiles = g.full = tiles;
+    if (!cus) return g;
+    uint32_t rem = tiles % cus;
+    if (rem == 0 || rem * 2 > cus) return g;  // a last round that is at least half full runs as it is
+    uint32_t splits = cus / rem, cap = 8;
+    if (const char *e = getenv("FE_GEMM_SPLITS")) cap = (uint32_t)atoi(e);  // 1: never cut
+    if (splits > cap) splits = cap;
+    if (splits > ktiles / 4) splits = ktiles / 4;  // at least 4 k tiles a program
+    if (splits < 2) return g;
+    g.full = tiles - rem;
+    g.splits = splits;
+    return g;
+}

@@ -1,18 +1,30 @@
-// LDS-staged f16 MFMA GEMM core for prefill-sized M: C[128 x 128 tile] = A[M][K] (f16, row-major, from global) times a
+// LDS-staged f16 MFMA GEMM core for prefill-sized M: C[256 x 256 tile] = A[M][K] (f16, row-major, from global) times a
 // weight tile that a producer decodes into LDS as f16 [n][k]. 256 threads = 4 wavefronts in a 2 x 2 grid, each owning a
-// 64 x 64 piece as 2 x 2 v_mfma_f32_32x32x16_f16 accumulators. The next k tile's global loads are issued before the
-// current tile's MFMAs, so memory latency overlaps the matrix work.
+// 128 x 128 piece as 4 x 4 v_mfma_f32_32x32x16_f16 accumulators (256 accumulator registers a lane, one wavefront a
+// SIMD). The large tile is what keeps the kernel off the memory system: a k tile of 64 brings 32 KB of activations and
+// the packed weights of 256 columns from L2 for 64 MFMAs a wavefront (half the bytes per flop of a 256 x 128 tile), and
+// moves 64 KB into and 128 KB out of LDS in the time of 2048 MFMA cycles. LDS holds two k tiles (one barrier per
+// k tile). Rows of an LDS tile are 64 f16 = 8 chunks of 16 bytes, chunk c of row r stored at position c ^ (r & 7), so
+// the lanes that read one chunk column of 8 consecutive rows hit 8 different bank groups (measured conflict-free).
 #pragma once
 #include "kcommon.h"
 
-#define GM_BM 128
-#define GM_BN 128
+#define GM_BM 256
+#define GM_BN 256
 #define GM_BK 64
-#define GM_PITCH 72  // f16 elements a row of an LDS tile: 64 + 8 pad (16-byte aligned rows, bank spread)
-#define GM_LDS_TILES (2 * GM_BM * GM_PITCH * 2)  // bytes of the A and B tiles
+#define GM_A_BYTES (GM_BM * GM_BK * 2)
+#define GM_B_BYTES (GM_BN * GM_BK * 2)
+#define GM_STAGE_BYTES (GM_A_BYTES + GM_B_BYTES)
+#define GM_LDS_TILES (2 * GM_STAGE_BYTES)  // 128 KB
+#define GM_EPI_PITCH 132                   // floats a row of a wavefront's 32 x 128 epilogue slab
+#define GM_EPI_SLAB (32 * GM_EPI_PITCH * 4)
+
+// Byte offset of 16-byte chunk c (0..7) of row r inside a [rows][64 f16] tile.
+__device__ __forceinline__ uint32_t gm_swz(uint32_t r, uint32_t c) { return r * 128 + ((c ^ (r & 7)) << 4); }
 
 // Grouped raster: `group` row tiles (fastest) sweep all column tiles before the next group, so programs that run
-// together share weight panels in L2 (kernels/k-fp4/src/lib.rs:298-308).
+// together share weight panels in L2 (kernels/k-fp4/src/lib.rs:298-308). Workgroups go to the 8 XCDs round-robin, so
+// with a group of 8 row tiles each XCD's L2 keeps one 256-row panel of activations.
 __device__ __forceinline__ void gemm_raster(uint32_t pid, uint32_t tiles_m, uint32_t tiles_n, uint32_t group, uint32_t& tm,
                                             uint32_t& tn) {
     uint32_t per_group = group * tiles_n;
@@ -23,66 +35,223 @@ __device__ __forceinline__ void gemm_raster(uint32_t pid, uint32_t tiles_m, uint
     tn = r / gsize;
 }
 
-// acc[i][j]: rows m0 + 64 wm + 32 i .., columns n0 + 64 wn + 32 j ..; lane L holds column L & 31, rows
-// 8 (e >> 2) + 4 (L >> 5) + (e & 3) for element e of the 16.
+// What a program computes. Programs 0 .. full_tiles - 1 take one output tile each over all of K. The remaining tiles
+// (a last round that would leave most CUs idle) are cut `splits` ways along K: program full_tiles + i takes k tiles
+// [kt0, kt0 + ktn) of tile full_tiles + i / splits and leaves its 256 x 256 f32 partial in slot i of the workspace; a
+// reduce kernel adds the slots of a tile in split order and finishes it, so results do not depend on timing.
+struct GemmWork {
+    uint32_t tm, tn, kt0, ktn, slot;
+    bool partial;
+};
+
+__device__ __forceinline__ GemmWork gemm_work(uint32_t pid, uint32_t tiles_m, uint32_t tiles_n, uint32_t group,
+                                              uint32_t ktiles, uint32_t full_tiles, uint32_t splits) {
+    GemmWork w;
+    uint32_t tile = pid, split = 0, ns = 1;
+    w.partial = pid >= full_tiles;
+    w.slot = 0;
+    if (w.partial) {
+        w.slot = pid - full_tiles;
+        tile = full_tiles + w.slot / splits;
+        split = w.slot % splits;
+        ns = splits;
+    }
+    gemm_raster(tile, tiles_m, tiles_n, group, w.tm, w.tn);
+    w.kt0 = split * ktiles / ns;
+    w.ktn = (split + 1) * ktiles / ns - w.kt0;
+    return w;
+}
+
+// acc[i][j]: rows m0 + 128 wm + 32 i .., columns n0 + 128 wn + 32 j ..; lane L holds column L & 31, rows
+// 8 (e >> 2) + 4 (L >> 5) + (e & 3) for element e of the 16. The producer supplies a register image Raw of its share of
+// a weight k tile, load(kt, raw) (global -> registers) and store(raw, Bs) (decode -> LDS tile of GM_BN rows, chunks
+// placed with gm_swz), and kStoreValu, about the number of VALU instructions of store().
+//
+// Schedule of one k tile (a wavefront runs alone on its SIMD, so the overlap is arranged inside the instruction stream):
+// the registers that carry a tile from memory to LDS are reloaded with tile kt + 2 right after they are written out, three
+// quarters of a k tile before they are needed; the LDS writes of tile kt + 1 are issued between the MFMAs of tile kt; MFMA fragments are read from LDS one 16-wide k slice ahead. The barrier sits before the last slice, whose
+// fragments are already in registers, so the first fragments of tile kt + 1 load under the last 16 MFMAs of tile kt.
+// Loads past the end re-read the last tile / row and are never used: the loop body has no branches.
 template <class Producer>
-__device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, uint32_t lda, uint32_t m, uint32_t k,
-                                              uint32_t m0, Producer& prod, unsigned char* lds, f32x16 (&acc)[2][2]) {
-    _Float16* As = (_Float16*)lds;
-    _Float16* Bs = As + GM_BM * GM_PITCH;
+struct GemmRegs {
+    u32x4 a[8];
+    typename Producer::Raw b;
+};
+
+template <class Producer>
+__device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, uint32_t lda, uint32_t m, uint32_t kt0,
+                                              uint32_t ktiles, uint32_t m0, Producer& prod, unsigned char* lds,
+                                              f32x16 (&acc)[4][4]) {
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t wm = wave >> 1, wn = wave & 1;
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < 4; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    // A: 128 rows x 8 chunks of 16 bytes; thread t takes chunk t & 7 of rows (t >> 3) + 32 j
+    // A: 256 rows x 8 chunks; thread t takes chunk t & 7 of rows (t >> 3) + 32 j. Byte offsets from `a` (< 4 GB, checked
+    // by the host), so the address of a load is a uniform base plus a 32-bit lane offset.
     const uint32_t a_chunk = tid & 7, a_row = tid >> 3;
-    u32x4 areg[4];
-    auto load_a = [&](uint32_t kt) {
+    uint32_t aoff[8];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            uint32_t row = m0 + a_row + 32 * j;
-            if (row < m)
-                areg[j] = *(const u32x4*)(a + (size_t)row * lda + kt * GM_BK + a_chunk * 8);
-            else
-                areg[j] = (u32x4){0, 0, 0, 0};
-        }
+    for (int j = 0; j < 8; j++) {
+        uint32_t row = m0 + a_row + 32 * j;
+        row = row < m ? row : m - 1;
+        aoff[j] = (row * lda + a_chunk * 8) * 2;
+    }
+    const unsigned char* abytes = (const unsigned char*)a + kt0 * (GM_BK * 2);  // k tiles kt0 .. kt0 + ktiles - 1
+    auto load_a = [&](GemmRegs<Producer>& r, uint32_t kt) {
+        kt = kt < ktiles ? kt : ktiles - 1;
+        const unsigned char* ak = abytes + kt * (GM_BK * 2);
+#pragma unroll
+        for (int j = 0; j < 8; j++) r.a[j] = *(const u32x4*)(ak + aoff[j]);
     };
-    auto store_a = [&]() {
+    auto load_b = [&](GemmRegs<Producer>& r, uint32_t kt) { prod.load(kt0 + (kt < ktiles ? kt : ktiles - 1), r.b); };
+    const uint32_t a_st = gm_swz(a_row, a_chunk);  // + 32 j rows = + 4096 j bytes (the swizzle depends on row & 7 only)
+    auto store_a = [&](const GemmRegs<Producer>& r, unsigned char* st) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) *(u32x4*)(As + (a_row + 32 * j) * GM_PITCH + a_chunk * 8) = areg[j];
+        for (int j = 0; j < 8; j++) *(u32x4*)(st + a_st + 4096 * j) = r.a[j];
+    };
+    // fragment addresses: row (lane & 31) of each 32-row piece, chunk 2 kk + (lane >> 5)
+    const uint32_t fr = lane & 31, fc = lane >> 5;
+    uint32_t foff[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; kk++) foff[kk] = gm_swz(fr, 2 * kk + fc);
+    const uint32_t fa_base = wm * 128 * 128, fb_base = GM_A_BYTES + wn * 128 * 128;
+    f16x8 fa[2][4], fb[2][4];
+    auto read_frags = [&](int set, const unsigned char* st, int kk) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) fa[set][i] = *(const f16x8*)(st + fa_base + 4096 * i + foff[kk]);
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[set][j] = *(const f16x8*)(st + fb_base + 4096 * j + foff[kk]);
+    };
+    auto mfmas = [&](int set) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
-    const uint32_t ktiles = k / GM_BK;
-    load_a(0);
-    prod.load(0);
+    GemmRegs<Producer> set;
+    load_b(set, 0);
+    load_a(set, 0);
+    prod.store(set.b, lds + GM_A_BYTES);
+    store_a(set, lds);
+    load_b(set, 1);
+    load_a(set, 1);
+    __syncthreads();
+    read_frags(0, lds, 0);
+
+    // One k tile: writes tile kt + 1 from the registers into the other LDS stage and reloads them with tile kt + 2 as
+    // soon as they are free. The sched_group_barrier sequences ask for one MFMA, then a few of the other instructions,
+    // and so on, so that memory instructions are issued while the matrix pipe works instead of in bursts that hold back
+    // the next MFMA.
     for (uint32_t kt = 0; kt < ktiles; kt++) {
-        store_a();
-        prod.store(Bs);
-        __syncthreads();
-        if (kt + 1 < ktiles) {
-            load_a(kt + 1);
-            prod.load(kt + 1);
+        const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
+        unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
+        // slice 0: weights of tile kt + 1 -> LDS
+        read_frags(1, cur, 1);
+        prod.store(set.b, nxt + GM_A_BYTES);
+        mfmas(0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, Producer::kStoreValu / 16 + 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        // slice 1: activations of tile kt + 1 -> LDS, weights of tile kt + 2 <- memory
+        read_frags(0, cur, 2);
+        store_a(set, nxt);
+        load_b(set, kt + 2);
+        mfmas(1);
 #pragma unroll
-        for (int kk = 0; kk < GM_BK / 16; kk++) {
-            f16x8 af[2], bf[2];
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-                af[i] = *(const f16x8*)(As + (wm * 64 + 32 * i + (lane & 31)) * GM_PITCH + kk * 16 + 8 * (lane >> 5));
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-                bf[j] = *(const f16x8*)(Bs + (wn * 64 + 32 * j + (lane & 31)) * GM_PITCH + kk * 16 + 8 * (lane >> 5));
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int j = 0; j < 2; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[i], bf[j], acc[i][j], 0, 0, 0);
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        // slice 2: activations of tile kt + 2 <- memory
+        read_frags(1, cur, 3);
+        load_a(set, kt + 2);
+        mfmas(0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        // slice 3, with the first fragments of tile kt + 1
+        read_frags(0, nxt, 0);
+        mfmas(1);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
     }
+    __syncthreads();  // the LDS tiles are free for the epilogue
+}
+
+// Hands the wavefront's 128 x 128 accumulators out row by row: 32 rows at a time pass through the wavefront's own LDS
+// slab (GM_EPI_SLAB bytes at lds + wave * GM_EPI_SLAB) so that 32 consecutive lanes hold 128 consecutive columns of one
+// row, 4 a lane. fn(row in 0..127, l32, v[4]) is called by both halves of the wavefront, each with its own row. No
+// workgroup barrier: only this wavefront touches its slab.
+template <class RowFn>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[4][4], unsigned char* lds, RowFn fn) {
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, hw = lane >> 5;
+    float* slab = (float*)(lds + wave * GM_EPI_SLAB);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++)
+                slab[(8 * (e >> 2) + 4 * hw + (e & 3)) * GM_EPI_PITCH + 32 * j + l32] = acc[i][j][e];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll 4
+        for (int rr = 0; rr < 16; rr++) {
+            uint32_t row = 2 * rr + hw;
+            f32x4 t = *(const f32x4*)(slab + row * GM_EPI_PITCH + 4 * l32);
+            float v[4] = {t[0], t[1], t[2], t[3]};
+            fn(32 * i + row, l32, v);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+#define GM_PART_FLOATS (GM_BM * GM_BN)  // floats of one partial slot
+
+// Leaves the program's accumulators in its partial slot, row-major [256][256] f32.
+__device__ __forceinline__ void gemm_store_partial(f32x16 (&acc)[4][4], unsigned char* lds, float* slot) {
+    const uint32_t wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
+    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t l32, float (&v)[4]) {
+        *(f32x4*)(slot + (wm * 128 + row) * GM_BN + wn * 128 + 4 * l32) = (f32x4){v[0], v[1], v[2], v[3]};
+    });
+}
+
+// Body of a reduce kernel: grid (tiles cut along K) * 64, 256 threads. Each half wavefront sums the `splits` slots of one
+// row of one 128-column half of a tile, 4 columns a lane, in split order, and hands them to fn(t, row in 0..255,
+// column half, l32, v[4]) with t the tile's index among the cut tiles.
+template <class RowFn>
+__device__ __forceinline__ void gemm_reduce_rows(const float* __restrict__ part, uint32_t splits, RowFn fn) {
+    const uint32_t t = blockIdx.x >> 6, hw = threadIdx.x >> 5, l32 = threadIdx.x & 31;
+    const uint32_t row = 4 * (blockIdx.x & 63) + (hw >> 1), cb = hw & 1;
+    const float* p = part + (size_t)t * splits * GM_PART_FLOATS + row * GM_BN + cb * 128 + 4 * l32;
+    f32x4 sum = *(const f32x4*)p;
+    for (uint32_t sp = 1; sp < splits; sp++) sum += *(const f32x4*)(p + (size_t)sp * GM_PART_FLOATS);
+    float v[4] = {sum[0], sum[1], sum[2], sum[3]};
+    fn(t, row, cb, l32, v);
 }

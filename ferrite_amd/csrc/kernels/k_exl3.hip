@@ -686,78 +686,100 @@ GEMV_STREAM_KERNEL(8)
 // ---- prefill GEMM ----------------------------------------------------------------------------------------------------
 
 // Weight tile producer of the prefill GEMM: a 64-wide k tile of a 128-column block is 4 k steps x 8 tiles; wavefront w
-// takes k step w, lane L tile L >> 3, rows n = (L & 7) and (L & 7) + 8 of it (the same run of words as in the GEMV).
+// takes k step w, lane L tile L >> 3, rows n = (L & 7) and (L & 7) + 8 of it (the same run of words as in the GEMV),
+// in both 128-column blocks of the 256-column output tile.
 template <int BITS>
 struct Exl3Producer {
-    const uint32_t* base;  // block's trellis + this lane's tile
+    const uint32_t* base[2];  // the two blocks' trellis + this lane's tile
     uint32_t stride_k, run_off, prev_off, brow, ks;
-    LaneWords<BITS> lw;
-    __device__ __forceinline__ void load(uint32_t kt) {
-        const uint32_t* p = base + (size_t)(kt * 4 + ks) * stride_k;
-        lw = load_lane_words<BITS>(p + run_off, p + prev_off);
+    struct Raw {
+        LaneWords<BITS> w[2];
+    };
+    static constexpr int kStoreValu = 240;  // about the VALU instructions of store()
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r) const {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            const uint32_t* p = base[b] + (size_t)(kt * 4 + ks) * stride_k;
+            r.w[b] = load_lane_words<BITS>(p + run_off, p + prev_off);
+        }
     }
-    __device__ __forceinline__ void store(_Float16* Bs) const {
-        f16x8 op[2][2];
-        decode_lane<BITS>(lw, op);
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs) const {
 #pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int b = 0; b < 2; b++) {
+            f16x8 op[2][2];
+            decode_lane<BITS>(r.w[b], op);
 #pragma unroll
-            for (int kh = 0; kh < 2; kh++) *(f16x8*)(Bs + (brow + 8 * h) * GM_PITCH + 16 * ks + 8 * kh) = op[h][kh];
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int kh = 0; kh < 2; kh++) *(f16x8*)(Bs + gm_swz(128 * b + brow + 8 * h, 2 * ks + kh)) = op[h][kh];
+        }
     }
 };
 
-#define GEMM_EPI_PITCH 132  // floats a row of the 128 x 128 output tile in LDS
-
-// y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for prefill-sized m: xh fp16 [m][k] (rotated inputs), 128 x 128 output
-// tiles, each exactly one Hadamard block wide so the output rotation is local to the tile. grid ceil(m / 128) * n / 128
-// (grouped raster), 256 threads, dynamic LDS 128 * GEMM_EPI_PITCH * 4 bytes.
+// y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for prefill-sized m: xh fp16 [m][k] (rotated inputs), 256 x 256 output
+// tiles; a wavefront's 128 columns are exactly one Hadamard block, so the output rotation is local to the wavefront.
+// grid full_tiles + (tiles - full_tiles) * splits with tiles = ceil(m / 256) * ceil(n / 256) (grouped raster), 256
+// threads, dynamic LDS GM_LDS_TILES (the epilogue reuses it). Tiles past full_tiles leave partials in `part` for
+// exl3_gemm_reduce.
 template <int BITS>
 __device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, const uint32_t* __restrict__ trellis,
                                                const uint16_t* __restrict__ svh, void* y, uint32_t n, uint32_t k, uint32_t m,
-                                               uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m) {
+                                               uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m,
+                                               uint32_t full_tiles, uint32_t splits, float* part) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    uint32_t tm, tn;
-    gemm_raster(blockIdx.x, (m + GM_BM - 1) / GM_BM, n / GM_BN, group_m, tm, tn);
-    const uint32_t m0 = tm * GM_BM, col0 = tn * GM_BN;
+    const uint32_t nbs = n / 128;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nbs + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
+    const uint32_t m0 = wk.tm * GM_BM, tn = wk.tn;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     constexpr uint32_t tw = 8 * BITS;
     Exl3Producer<BITS> prod;
     {
         uint32_t tj = lane >> 3, q = lane & 7;
-        prod.base = trellis + (size_t)tn * stride_nb + tj * tw;
+        uint32_t nb1 = 2 * tn + 1 < nbs ? 2 * tn + 1 : 2 * tn;  // an odd block count: the last tile decodes block 2 tn twice
+        prod.base[0] = trellis + (size_t)(2 * tn) * stride_nb + tj * tw;
+        prod.base[1] = trellis + (size_t)nb1 * stride_nb + tj * tw;
         prod.stride_k = stride_k;
         prod.run_off = q * BITS;
         prod.prev_off = (q * BITS + tw - 1) % tw;
         prod.brow = tj * 16 + q;
         prod.ks = wave;
     }
-    f32x16 acc[2][2];
-    gemm_mainloop(xh, k, m, k, m0, prod, lds, acc);
-    float* tile = (float*)lds;
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                uint32_t row = wm * 64 + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                tile[row * GEMM_EPI_PITCH + wn * 64 + 32 * j + (lane & 31)] = acc[i][j][e];
-            }
-    __syncthreads();
-    const uint32_t hw = tid >> 5, l32 = tid & 31;
-    for (uint32_t row = hw; row < GM_BM; row += 8) {
-        if (m0 + row >= m) break;
-        f32x4 t = *(const f32x4*)(tile + row * GEMM_EPI_PITCH + 4 * l32);
-        float v[4] = {t[0], t[1], t[2], t[3]};
-        finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)(m0 + row) * n + col0 + 4 * l32);
+    f32x16 acc[4][4];
+    gemm_mainloop(xh, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
+    if (wk.partial) {
+        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
+        return;
     }
+    const uint32_t nb = 2 * tn + wn;
+    if (nb >= nbs) return;
+    const uint32_t col0 = nb * 128;
+    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t l32, float (&v)[4]) {
+        uint32_t grow = m0 + wm * 128 + row;
+        if (grow < m) finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)grow * n + col0 + 4 * l32);
+    });
+}
+
+// Finishes the tiles that exl3_gemm_b* cut along K: sums their partial slots and applies the output rotation and scale.
+// grid (tiles - full_tiles) * 64, 256 threads.
+extern "C" __global__ __launch_bounds__(256) void exl3_gemm_reduce(const float* part, const uint16_t* svh, void* y, uint32_t n,
+                                                                   uint32_t m, uint32_t y_mode, uint32_t group_m,
+                                                                   uint32_t full_tiles, uint32_t splits) {
+    const uint32_t nbs = n / 128;
+    gemm_reduce_rows(part, splits, [&](uint32_t t, uint32_t row, uint32_t cb, uint32_t l32, float (&v)[4]) {
+        uint32_t tm, tn;
+        gemm_raster(full_tiles + t, (m + GM_BM - 1) / GM_BM, (nbs + 1) / 2, group_m, tm, tn);
+        uint32_t grow = tm * GM_BM + row, nb = 2 * tn + cb;
+        if (grow < m && nb < nbs) finish_row(v, l32, svh, nb * 128 + 4 * l32, y, y_mode, (size_t)grow * n + nb * 128 + 4 * l32);
+    });
 }
 
 #define GEMM_KERNEL(BITS)                                                                                              \
-    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemm_b##BITS(                                            \
+    extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_b##BITS(                                            \
         const _Float16* xh, const uint32_t* trellis, const uint16_t* svh, void* y, uint32_t n, uint32_t k, uint32_t m,  \
-        uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m) {                                    \
-        exl3_gemm_body<BITS>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m);                      \
+        uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m, uint32_t full_tiles, uint32_t splits, \
+        float* part) {                                                                                                 \
+        exl3_gemm_body<BITS>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m, full_tiles, splits,    \
+                             part);                                                                                    \
     }
 GEMM_KERNEL(2)
 GEMM_KERNEL(3)

@@ -122,66 +122,104 @@ extern "C" __global__ __launch_bounds__(256) void fe_fp4_quant(uint8_t* codes, u
 
 // ---- GEMM --------------------------------------------------------------------------------------------------------------
 
-// Weight tile producer: thread t expands 32 codes of row n0 + (t >> 1), k half t & 1 of the 64-wide k tile.
+// Weight tile producer: thread t expands the 64 codes of row t of the 256-row weight tile. Codes and scales are
+// addressed through strides, base + kt * skt for the thread's row, so both the row-major layout of the format and the
+// k-tile-major layout of an uploaded linear ([n / 128][k / 64][128 rows][32 bytes of codes | 4 scales], one contiguous
+// 4.5 KB read per 128 rows and k tile) are read by the same kernel.
 struct Fp4Producer {
-    const uint8_t* w;   // codes of row n0 + (t >> 1), at byte (t & 1) * 16
-    const uint8_t* sw;  // row-major scales of that row, at block (t & 1) * 2
-    uint32_t row, half;
-    u32x4 c;
-    uint32_t s2;
-    __device__ __forceinline__ void load(uint32_t kt) {
-        c = __builtin_nontemporal_load((const u32x4*)(w + (size_t)kt * 32));
-        s2 = *(const uint16_t*)(sw + kt * 4);
+    const uint8_t* w;   // codes of this thread's row, k tile 0
+    const uint8_t* sw;  // scales of this thread's row, k tile 0
+    uint32_t w_skt, s_skt, row;
+    struct Raw {
+        u32x4 c[2];
+        uint32_t s4;
+    };
+    static constexpr int kStoreValu = 128;  // about the VALU instructions of store()
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r) const {
+        const uint8_t* p = w + (size_t)kt * w_skt;
+        r.c[0] = *(const u32x4*)p;
+        r.c[1] = *(const u32x4*)(p + 16);
+        r.s4 = *(const uint32_t*)(sw + (size_t)kt * s_skt);
     }
-    __device__ __forceinline__ void store(_Float16* Bs) const {
-        uint32_t o[16];
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs) const {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int d = 0; d < 8; d++) {
             uint32_t t[4];
-            e2m1x8_to_f16(c[j], t);
-            f16x2 sc = e4m3_to_f16x2((s2 >> (8 * (j >> 1))) & 0xff);
+            e2m1x8_to_f16(r.c[d >> 2][d & 3], t);
+            f16x2 sc = e4m3_to_f16x2((r.s4 >> (8 * (d >> 1))) & 0xff);
+            u32x4 o;
 #pragma unroll
-            for (int e = 0; e < 4; e++) o[4 * j + e] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[e]) * sc));
+            for (int e = 0; e < 4; e++) o[e] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[e]) * sc));
+            *(u32x4*)(Bs + gm_swz(row, d)) = o;
         }
-        u32x4* d = (u32x4*)(Bs + row * GM_PITCH + half * 32);
-#pragma unroll
-        for (int j = 0; j < 4; j++) d[j] = (u32x4){o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
     }
 };
 
-// C[M][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res: bf16(bf16(.) + res)); A_q as the fp16 operand of fe_fp4_quant,
-// W codes [N][K/2], scales row-major [N][K/16]. grid ceil(M / 128) * N / 128 (grouped raster), 256 threads, dynamic LDS
-// GM_LDS_TILES. N % 128 == 0, K % 128 == 0. (kernels/k-fp4/src/lib.rs:285-470)
-extern "C" __global__ __launch_bounds__(256, 2) void fe_gemm_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
+// One row piece of the output: 4 columns from `col` of row `grow`, bf16((sum) * alpha) (+ res: bf16(bf16(.) + res)).
+__device__ __forceinline__ void fp4_store4(uint16_t* c, const uint16_t* res, size_t at, const float (&v)[4], f32x4 al) {
+    u32x2 o = {pack_bf16x2(v[0] * al[0], v[1] * al[1]), pack_bf16x2(v[2] * al[2], v[3] * al[3])};
+    if (res) {
+        u32x2 r = *(const u32x2*)(res + at);
+#pragma unroll
+        for (int e = 0; e < 2; e++)
+            o[e] = pack_bf16x2(bf16_bits_to_f32(o[e] & 0xffff) + bf16_bits_to_f32(r[e] & 0xffff),
+                               bf16_bits_to_f32(o[e] >> 16) + bf16_bits_to_f32(r[e] >> 16));
+    }
+    *(u32x2*)(c + at) = o;
+}
+
+// C[M][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res: bf16(bf16(.) + res)); A_q as the fp16 operand of fe_fp4_quant. The
+// codes of row r = 128 nt + i, k tile kt are 32 bytes at w + nt * w_snt + kt * w_skt + i * w_sr, its 4 scales at
+// sw + nt * s_snt + kt * s_skt + i * s_sr. grid full_tiles + (tiles - full_tiles) * splits with tiles =
+// ceil(M / 256) * ceil(N / 256) (grouped raster), 256 threads, dynamic LDS GM_LDS_TILES. Tiles past full_tiles leave
+// partials in `part` for fe_gemm_nvfp4_reduce. N % 128 == 0, K % 128 == 0. (kernels/k-fp4/src/lib.rs:285-470)
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
                                                                    const uint8_t* sw, const float* alpha, const uint16_t* res,
                                                                    uint32_t m, uint32_t n, uint32_t k, uint32_t ldc,
-                                                                   uint32_t group_m) {
+                                                                   uint32_t group_m, uint32_t w_snt, uint32_t w_skt,
+                                                                   uint32_t w_sr, uint32_t s_snt, uint32_t s_skt,
+                                                                   uint32_t s_sr, uint32_t full_tiles, uint32_t splits,
+                                                                   float* part) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    uint32_t tm, tn;
-    gemm_raster(blockIdx.x, (m + GM_BM - 1) / GM_BM, n / GM_BN, group_m, tm, tn);
-    const uint32_t m0 = tm * GM_BM, n0 = tn * GM_BN;
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const uint32_t nts = n / 128;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
+    const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
     Fp4Producer prod;
-    prod.row = tid >> 1, prod.half = tid & 1;
-    prod.w = w + (size_t)(n0 + prod.row) * (k >> 1) + prod.half * 16;
-    prod.sw = sw + (size_t)(n0 + prod.row) * (k >> 4) + prod.half * 2;
-    f32x16 acc[2][2];
-    gemm_mainloop(aq, k, m, k, m0, prod, lds, acc);
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        uint32_t col = n0 + wn * 64 + 32 * j + (lane & 31);
-        float al = alpha[col] * 0.25f;
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) {
-                uint32_t row = m0 + wm * 64 + 32 * i + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (row < m) {
-                    size_t at = (size_t)row * ldc + col;
-                    uint32_t v = f32_to_bf16_bits(acc[i][j][e] * al);
-                    if (res) v = f32_to_bf16_bits(bf16_bits_to_f32(v) + bf16_bits_to_f32(res[at]));
-                    c[at] = (uint16_t)v;
-                }
-            }
+    {
+        uint32_t nt = 2 * wk.tn + (tid >> 7);
+        nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program expands its first tile twice
+        prod.row = tid;
+        prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
+        prod.sw = sw + (size_t)nt * s_snt + (size_t)(tid & 127) * s_sr;
+        prod.w_skt = w_skt, prod.s_skt = s_skt;
     }
+    f32x16 acc[4][4];
+    gemm_mainloop(aq, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
+    if (wk.partial) {
+        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
+        return;
+    }
+    const uint32_t colb = n0 + wn * 128;
+    if (colb >= n) return;
+    const uint32_t col = colb + 4 * (tid & 31);
+    f32x4 al = *(const f32x4*)(alpha + col) * 0.25f;
+    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t, float (&v)[4]) {
+        uint32_t grow = m0 + wm * 128 + row;
+        if (grow < m) fp4_store4(c, res, (size_t)grow * ldc + col, v, al);
+    });
+}
+
+// Finishes the tiles that fe_gemm_nvfp4 cut along K. grid (tiles - full_tiles) * 64, 256 threads.
+extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t* c, const float* part, const float* alpha,
+                                                                       const uint16_t* res, uint32_t m, uint32_t n,
+                                                                       uint32_t ldc, uint32_t group_m, uint32_t full_tiles,
+                                                                       uint32_t splits) {
+    const uint32_t nts = n / 128;
+    gemm_reduce_rows(part, splits, [&](uint32_t t, uint32_t row, uint32_t cb, uint32_t l32, float (&v)[4]) {
+        uint32_t tm, tn;
+        gemm_raster(full_tiles + t, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, tm, tn);
+        uint32_t grow = tm * GM_BM + row, col = tn * GM_BN + cb * 128 + 4 * l32;
+        if (grow < m && col < n) fp4_store4(c, res, (size_t)grow * ldc + col, v, *(const f32x4*)(alpha + col) * 0.25f);
+    });
 }

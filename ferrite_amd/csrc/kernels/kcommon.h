@@ -21,15 +21,14 @@ typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// f32 -> bf16 bits, round to nearest even, NaN kept quiet.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-    uint32_t b = __float_as_uint(f);
-    if (f != f) return (b >> 16) | 0x40;
-    return (b + 0x7fffu + ((b >> 16) & 1u)) >> 16;
-}
+// f32 -> bf16 bits, round to nearest even, NaN stays a quiet NaN: the hardware conversion (v_cvt_pk_bf16_f32).
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-    return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+    f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {

@@ -147,6 +147,19 @@ class PromptLinear:
                                               host.codes.ctypes.data_as(C.c_void_p), host.sf.ctypes.data_as(C.c_void_p),
                                               alpha.ctypes.data_as(C.c_void_p), host.g))
 
+    @classmethod
+    def from_view(cls, name: str, n: int, k: int, codes, scales, alpha, g: float) -> "PromptLinear":
+        """A linear over device tensors in the format's own layout (codes [n][k/2], scales [n][k/16] row-major, alpha
+        f32 [n]); nothing is copied, the tensors are kept alive (place + set_views, lib.rs:445, 486)."""
+        _lib.init()
+        self = cls.__new__(cls)
+        self.n, self.k, self.name, self.parts, self.g, self.swiglu = n, k, name, [], g, False
+        self._keep = (codes, scales, alpha)
+        self.h = C.c_void_p()
+        check(_lib.lib().fe_fp4_linear_from_view(C.byref(self.h), name.encode(), n, k, codes.data_ptr(), scales.data_ptr(),
+                                                 alpha.data_ptr(), g))
+        return self
+
     def __del__(self):
         if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
             _lib._lib.fe_fp4_linear_destroy(self.h)

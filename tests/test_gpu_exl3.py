@@ -282,3 +282,39 @@ def test_argument_errors_are_results_not_crashes(env):
     lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 4, ws)
     torch.cuda.synchronize()
     assert torch.isfinite(y[:4]).all()
+
+
+def test_prefill_gemm_tiles_cut_or_whole(env, oracle, monkeypatch):
+    """Several 256 x 256 tiles with an odd count of 128-column blocks: computed whole (FE_GEMM_SPLITS=1) and cut along K
+    with the reduce kernel (the default for a nearly empty last round)."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    m = 300
+    t = synth.exl3_tensor(1024, 384, 4, 77)
+    o = to_oracle(oracle, t)
+    xb = synth.activations(m, t.k, 5, outliers=True)
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 256)
+    ws = exl3.Workspace([lin], m)
+    xd = dev_u16(torch, xb)
+
+    def run():
+        y = torch.full((m + 2, t.n), float("nan"), dtype=torch.float32, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+        torch.cuda.synchronize()
+        out = y.cpu().numpy().astype(np.float64)
+        assert np.isnan(out[m:]).all()
+        return out[:m]
+
+    cut = run()
+    assert np.array_equal(cut, run())
+    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    whole = run()
+    ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
+    rms = np.sqrt((ref ** 2).mean())
+    assert np.abs(cut - ref).max() / rms < 1e-4
+    assert np.abs(whole - ref).max() / rms < 1e-4
+    # accumulate into y (y dtype flag 3: f32, add)
+    y = torch.ones((m, t.n), dtype=torch.float32, device="cuda")
+    lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32Add, m, ws)
+    torch.cuda.synchronize()
+    assert np.abs(y.cpu().numpy().astype(np.float64) - 1.0 - ref).max() / rms < 1e-4

@@ -100,6 +100,54 @@ def test_fp4_linear(env, oracle, n, k, m, input_scale):
     assert np.array_equal(y3.view(torch.int16).cpu().numpy().view(np.uint16), yg)
 
 
+def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
+    """Several 256 x 256 output tiles with an odd count of 128-row weight tiles, computed whole (FE_GEMM_SPLITS=1), cut
+    along K with the reduce kernel (the default for a nearly empty last round), and from a row-major device view."""
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    n, k, m = 640, 1024, 300
+    host = synth.fp4_linear(n, k, 23, input_scale=1.0)
+    host.alpha[:] = host.alpha * np.linspace(0.5, 2.0, n).astype(np.float32)
+    lin = host.upload()
+    ws = fp4.Workspace(m, k)
+    xd = dev_u16(torch, fp4_check_activations(m, k, lin.g, 4))
+
+    def run(l, res=None):
+        y = torch.full((m + 2, n), -3.0, dtype=torch.bfloat16, device="cuda")
+        l.forward(kern, ws, y, n, xd, k, m, res=res)
+        torch.cuda.synchronize()
+        out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+        assert (out[m:] == bf16_bits(np.float32([-3.0]))[0]).all()
+        return out[:m]
+
+    cut = run(lin)
+    assert np.array_equal(cut, run(lin))  # deterministic
+    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    whole = run(lin)
+    view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), torch.from_numpy(host.sf).cuda(),
+                                      torch.from_numpy(host.alpha).cuda(), host.g)
+    assert np.array_equal(run(view), whole)
+    monkeypatch.delenv("FE_GEMM_SPLITS")
+    assert np.array_equal(run(view), cut)
+    # cut and whole differ only by the order of the f32 sums: at most one bf16 step
+    a, b = bf16_to_f32(cut).astype(np.float64), bf16_to_f32(whole).astype(np.float64)
+    assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all()
+    # against the f64 reference over the quantized operands
+    codes, sf_tiled = ws.read(m, k)
+    sfa = oracle.untile_scales(sf_tiled, m, k // 16).reshape(m, k // 16)
+    rows = [0, 127, 128, 255, 256, 299]
+    refq = oracle.ref_gemm(oracle.dequant_fp4(codes[rows], sfa[rows], 1.0), oracle.dequant_fp4(host.codes, host.sf, 1.0))
+    refq = refq.astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+    scale = np.abs(refq).max(axis=1, keepdims=True).clip(1e-20)
+    for got in (a[rows], b[rows]):
+        assert (np.abs(got - refq) / np.maximum(np.abs(refq), 1e-2 * scale)).max() < 1e-2
+    # residual through the reduce kernel's epilogue
+    res = dev_u16(torch, bf16_bits(np.random.default_rng(6).normal(size=(m + 2, n)).astype(np.float32)))
+    got = run(lin, res=res)
+    want = bf16_bits(bf16_to_f32(cut) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m]))
+    assert np.array_equal(got, want)
+
+
 def test_fp4_argument_errors(env):
     torch, fp4, kern = env
     from ferrite_amd import synth
