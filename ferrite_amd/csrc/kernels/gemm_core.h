@@ -64,20 +64,15 @@ __device__ __forceinline__ GemmWork gemm_work(uint32_t pid, uint32_t tiles_m, ui
 
 // acc[i][j]: rows m0 + 128 wm + 32 i .., columns n0 + 128 wn + 32 j ..; lane L holds column L & 31, rows
 // 8 (e >> 2) + 4 (L >> 5) + (e & 3) for element e of the 16. The producer supplies a register image Raw of its share of
-// a weight k tile, load(kt, raw) (global -> registers) and store(raw, Bs) (decode -> LDS tile of GM_BN rows, chunks
-// placed with gm_swz), and kStoreValu, about the number of VALU instructions of store().
+// a weight k tile, load(kt, raw, half) (global -> the registers of half 0 or 1) and store(raw, Bs, part) for part 0, 1
+// (decode that half of
+// the share -> LDS tile of GM_BN rows, chunks placed with gm_swz), and kStoreValu, about the number of VALU
+// instructions of the two parts together.
 //
 // Schedule of one k tile (a wavefront runs alone on its SIMD, so the overlap is arranged inside the instruction stream):
-// the registers that carry a tile from memory to LDS are reloaded with tile kt + 2 right after they are written out, three
-// quarters of a k tile before they are needed; the LDS writes of tile kt + 1 are issued between the MFMAs of tile kt; MFMA fragments are read from LDS one 16-wide k slice ahead. The barrier sits before the last slice, whose
+// the registers that carry a tile from memory to LDS are reloaded with tile kt + 2 right after they are written out; the LDS writes of tile kt + 1 are issued between the MFMAs of tile kt; MFMA fragments are read from LDS one 16-wide k slice ahead. The barrier sits before the last slice, whose
 // fragments are already in registers, so the first fragments of tile kt + 1 load under the last 16 MFMAs of tile kt.
 // Loads past the end re-read the last tile / row and are never used: the loop body has no branches.
-template <class Producer>
-struct GemmRegs {
-    u32x4 a[8];
-    typename Producer::Raw b;
-};
-
 template <class Producer>
 __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, uint32_t lda, uint32_t m, uint32_t kt0,
                                               uint32_t ktiles, uint32_t m0, Producer& prod, unsigned char* lds,
@@ -102,17 +97,20 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         aoff[j] = (row * lda + a_chunk * 8) * 2;
     }
     const unsigned char* abytes = (const unsigned char*)a + kt0 * (GM_BK * 2);  // k tiles kt0 .. kt0 + ktiles - 1
-    auto load_a = [&](GemmRegs<Producer>& r, uint32_t kt) {
+    u32x4 areg[8];
+    auto load_a = [&](uint32_t kt, int j0, int j1) {
         kt = kt < ktiles ? kt : ktiles - 1;
         const unsigned char* ak = abytes + kt * (GM_BK * 2);
 #pragma unroll
-        for (int j = 0; j < 8; j++) r.a[j] = *(const u32x4*)(ak + aoff[j]);
+        for (int j = j0; j < j1; j++) areg[j] = *(const u32x4*)(ak + aoff[j]);
     };
-    auto load_b = [&](GemmRegs<Producer>& r, uint32_t kt) { prod.load(kt0 + (kt < ktiles ? kt : ktiles - 1), r.b); };
+    auto load_b = [&](typename Producer::Raw& r, uint32_t kt, int half) {
+        prod.load(kt0 + (kt < ktiles ? kt : ktiles - 1), r, half);
+    };
     const uint32_t a_st = gm_swz(a_row, a_chunk);  // + 32 j rows = + 4096 j bytes (the swizzle depends on row & 7 only)
-    auto store_a = [&](const GemmRegs<Producer>& r, unsigned char* st) {
+    auto store_a = [&](unsigned char* st, int j0, int j1) {
 #pragma unroll
-        for (int j = 0; j < 8; j++) *(u32x4*)(st + a_st + 4096 * j) = r.a[j];
+        for (int j = j0; j < j1; j++) *(u32x4*)(st + a_st + 4096 * j) = areg[j];
     };
     // fragment addresses: row (lane & 31) of each 32-row piece, chunk 2 kk + (lane >> 5)
     const uint32_t fr = lane & 31, fc = lane >> 5;
@@ -135,68 +133,77 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
-    GemmRegs<Producer> set;
-    load_b(set, 0);
-    load_a(set, 0);
-    prod.store(set.b, lds + GM_A_BYTES);
-    store_a(set, lds);
-    load_b(set, 1);
-    load_a(set, 1);
+    typename Producer::Raw braw;
+    load_b(braw, 0, 0);
+    load_b(braw, 0, 1);
+    load_a(0, 0, 8);
+#pragma unroll
+    for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
+    store_a(lds, 0, 8);
+    load_b(braw, 1, 0);
+    load_b(braw, 1, 1);
+    load_a(1, 0, 8);
     __syncthreads();
     read_frags(0, lds, 0);
 
-    // One k tile: writes tile kt + 1 from the registers into the other LDS stage and reloads them with tile kt + 2 as
-    // soon as they are free. The sched_group_barrier sequences ask for one MFMA, then a few of the other instructions,
-    // and so on, so that memory instructions are issued while the matrix pipe works instead of in bursts that hold back
-    // the next MFMA.
+    // One k tile: writes tile kt + 1 into the other LDS stage (weights from braw, half in each of the first two slices,
+    // activations from areg in the third) and reloads the registers with tile kt + 2 in the slice after they are
+    // written out, so that every slice carries a similar share of the memory instructions. The
+    // sched_group_barrier sequences ask for one MFMA, then a few of the other instructions, and so on, so that memory
+    // instructions are issued while the matrix pipe works instead of in bursts that hold back the next MFMA.
     for (uint32_t kt = 0; kt < ktiles; kt++) {
         const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
         unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
-        // slice 0: weights of tile kt + 1 -> LDS
+        constexpr int kValu = Producer::kStoreValu / 2 / 16 + 1;  // vector ALU instructions between two MFMAs
+        // slice 0
         read_frags(1, cur, 1);
-        prod.store(set.b, nxt + GM_A_BYTES);
+        prod.store(braw, nxt + GM_A_BYTES, 0);
         mfmas(0);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, Producer::kStoreValu / 16 + 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // slice 1: activations of tile kt + 1 -> LDS, weights of tile kt + 2 <- memory
+        // slice 1
         read_frags(0, cur, 2);
-        store_a(set, nxt);
-        load_b(set, kt + 2);
+        prod.store(braw, nxt + GM_A_BYTES, 1);
+        load_b(braw, kt + 2, 0);
+        load_b(braw, kt + 2, 1);
         mfmas(1);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // slice 2: activations of tile kt + 2 <- memory
+        // slice 2
         read_frags(1, cur, 3);
-        load_a(set, kt + 2);
+        store_a(nxt, 0, 8);
         mfmas(0);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        // slice 3, with the first fragments of tile kt + 1
+        read_frags(0, nxt, 0);
+        load_a(kt + 2, 0, 8);
+        mfmas(1);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        __syncthreads();
-        // slice 3, with the first fragments of tile kt + 1
-        read_frags(0, nxt, 0);
-        mfmas(1);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
     }

@@ -696,16 +696,19 @@ struct Exl3Producer {
         LaneWords<BITS> w[2];
     };
     static constexpr int kStoreValu = 240;  // about the VALU instructions of store()
-    __device__ __forceinline__ void load(uint32_t kt, Raw& r) const {
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
 #pragma unroll
         for (int b = 0; b < 2; b++) {
+            if (b != half) continue;
             const uint32_t* p = base[b] + (size_t)(kt * 4 + ks) * stride_k;
             r.w[b] = load_lane_words<BITS>(p + run_off, p + prev_off);
         }
     }
-    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs) const {
+    // part 0: the first column block, part 1: the second
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
 #pragma unroll
         for (int b = 0; b < 2; b++) {
+            if (b != part) continue;
             f16x8 op[2][2];
             decode_lane<BITS>(r.w[b], op);
 #pragma unroll

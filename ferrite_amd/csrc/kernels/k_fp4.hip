@@ -132,21 +132,21 @@ struct Fp4Producer {
     uint32_t w_skt, s_skt, row;
     struct Raw {
         u32x4 c[2];
-        uint32_t s4;
+        uint32_t s2[2];
     };
     static constexpr int kStoreValu = 128;  // about the VALU instructions of store()
-    __device__ __forceinline__ void load(uint32_t kt, Raw& r) const {
-        const uint8_t* p = w + (size_t)kt * w_skt;
-        r.c[0] = *(const u32x4*)p;
-        r.c[1] = *(const u32x4*)(p + 16);
-        r.s4 = *(const uint32_t*)(sw + (size_t)kt * s_skt);
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
+        r.c[half] = *(const u32x4*)(w + (size_t)kt * w_skt + 16 * half);
+        r.s2[half] = *(const uint16_t*)(sw + (size_t)kt * s_skt + 2 * half);
     }
-    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs) const {
+    // part 0: chunks 0..3 of the row, part 1: 4..7
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
 #pragma unroll
         for (int d = 0; d < 8; d++) {
+            if (d / 4 != part) continue;
             uint32_t t[4];
             e2m1x8_to_f16(r.c[d >> 2][d & 3], t);
-            f16x2 sc = e4m3_to_f16x2((r.s4 >> (8 * (d >> 1))) & 0xff);
+            f16x2 sc = e4m3_to_f16x2((r.s2[d >> 2] >> (8 * ((d >> 1) & 1))) & 0xff);
             u32x4 o;
 #pragma unroll
             for (int e = 0; e < 4; e++) o[e] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[e]) * sc));
