@@ -20,7 +20,8 @@ constexpr uint32_t kTileN = 256;                        // GM_BN
 
 struct fe_fp4_kernels {
     fe_module_t module = nullptr;
-    fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr;
+    fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4 = nullptr;
+    uint32_t cus = 0;
     uint32_t group_m = 8;  // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
 };
 
@@ -35,8 +36,11 @@ struct fe_fp4_linear {
 
 struct fe_fp4_workspace {
     uint32_t max_rows = 0, max_k = 0;
-    FeBuf codes, sf, aq, part;  // part: partial tiles of the GEMM, one slot a CU
+    FeBuf codes, sf, aq, part, counters;  // part: partial sums of the GEMM (one slot a CU) or of the GEMV's splits
 };
+constexpr uint32_t kGemvRows = 16;      // rows of one fe_gemv_nvfp4 pass
+constexpr uint32_t kGemvMaxRows = 64;   // up to here the GEMV runs in passes; above, the GEMM
+constexpr uint32_t kGemvCounters = 8192;  // arrival counters: weight tiles of 128 rows (n <= 1 M)
 
 extern "C" {
 
@@ -48,6 +52,10 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->gemm4, k->module, "fe_gemm_nvfp4");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm4, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->reduce4, k->module, "fe_gemm_nvfp4_reduce");
+    if (!c) c = fe_hip_module_get_function(&k->gemv4, k->module, "fe_gemv_nvfp4");
+    int cus = 0;
+    if (!c) c = fe_hip_cu_count(&cus);
+    k->cus = (uint32_t)cus;
     if (const char *g = getenv("FE_FP4_GROUP")) k->group_m = (uint32_t)atoi(g);
     if (c) {
         fe_fp4_kernels_destroy(k);
@@ -148,6 +156,7 @@ int fe_fp4_workspace_create(fe_fp4_workspace **out, uint32_t max_rows, uint32_t 
     int cus = 0;
     if (!c) c = fe_hip_cu_count(&cus);
     if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
+    if (!c) c = ws->counters.zeroed(kGemvCounters * 4);
     if (c) {
         delete ws;
         return c;
@@ -198,6 +207,25 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     if (!y || ldy % 8 || y % 16 || (res && res % 16) || ldy < l->n)
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
+    if (m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
+        // decode-sized: the weight-read-bound GEMV, 16 rows a pass. Programs: about three a CU.
+        const uint32_t nts = n / kTile, kts = k / 64;
+        uint32_t sk = (3 * kern->cus + nts / 2) / nts;
+        if (const char *e = getenv("FE_FP4_GEMV_SK")) sk = (uint32_t)atoi(e);
+        if (sk > 16) sk = 16;
+        if (sk > kts / 4) sk = kts / 4;
+        while (sk > 1 && (size_t)sk * kGemvRows * n * 4 > ws->part.bytes) sk--;
+        if (sk < 1) sk = 1;
+        fe_devptr_t w = l->w.p, sw = l->sw.p, alpha = l->alpha.p, z = ws->part.p, cnt = ws->counters.p;
+        uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
+        for (uint32_t r0 = 0; r0 < m; r0 += kGemvRows) {
+            uint32_t rows = m - r0 < kGemvRows ? m - r0 : kGemvRows;
+            fe_devptr_t yy = y + (size_t)r0 * ldy * 2, aq = ws->aq.p + (size_t)r0 * k * 2, rr = res ? res + (size_t)r0 * ldy * 2 : 0;
+            void *args[] = {&yy, &aq, &w, &sw, &alpha, &rr, &z, &cnt, &rows, &n, &k, &ldy, &sk, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr};
+            FE_TRY(fe_hip_launch(kern->gemv4, nts * sk, 1, 1, 256, 1, 1, 0, s, args));
+        }
+        return 0;
+    }
     if ((uint64_t)m * k * 2 >= (1ull << 32) || (uint64_t)n * k / 2 >= (1ull << 32))
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_fp4_linear_gemm", "operand of 4 GB or more");
     const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;

@@ -3,10 +3,10 @@
 // is W4A4, crates/fe-fp4/src/lib.rs:512-530), then the GEMM runs over the quantized operands.
 //
 // gfx950's block-scaled MFMA takes e8m0 scales per 32 elements, which cannot express e4m3 per 16. A product
-// e2m1 x e4m3 has at most 6 significant bits and lies in [2^-10, 2688], so twice that value is an exact, normal fp16
-// number: both operands are expanded to fp16 (2 * code value * block scale) and multiplied on the f16 MFMA with fp32
-// accumulation, which reproduces the block-scaled dot product up to summation order; the factor 4 comes off in the
-// epilogue.
+// e2m1 x e4m3 has at most 6 significant bits and lies in [2^-10, 2688], so a small power of two times that value is an
+// exact, normal fp16 number: both operands are expanded to fp16 (activations as 2 * code value * block scale, weights
+// as 8 * ...) and multiplied on the f16 MFMA with fp32 accumulation, which reproduces the block-scaled dot product up
+// to summation order; the factor 16 comes off in the epilogue.
 #include "gemm_core.h"
 
 // ---- number formats ----------------------------------------------------------------------------------------------------
@@ -65,6 +65,33 @@ __device__ __forceinline__ f16x2 e4m3_to_f16x2(uint32_t b) {
     f16x2 v = __builtin_bit_cast(f16x2, h | (h << 16));
     const f16x2 c = {(_Float16)256.0f, (_Float16)256.0f};
     return v * c;
+}
+
+// Weights through the hardware conversion. v_cvt_scalef32_pk_f16_fp4 turns the two e2m1 codes of one byte into fp16 and
+// multiplies by a power of two: it takes only the exponent of its f32 scale operand (measured: scale 1.5 gives x1, 448
+// gives x256). An e4m3 block scale is 2^(max(e, 1) - 7) * t / 8 with t = m (+ 8 for a normal number), so a weight is
+// cvt(code, 2^(max(e, 1) - 7)) * t / 8; code * t has at most 6 significant bits and is exact in fp16. The kernels keep
+// the factor 8 (weights as code * 2^E * t, below 23040) and take it off with alpha in the epilogue.
+struct Fp4Scale {
+    float pow2;  // 2^(max(e, 1) - 7) as f32
+    f16x2 t;     // (t, t) as fp16
+};
+__device__ __forceinline__ Fp4Scale fp4_scale(uint32_t b) {  // b: e4m3 code, sign bit clear
+    uint32_t e = b >> 3, e1 = e < 1 ? e : 1;
+    Fp4Scale s;
+    s.pow2 = __uint_as_float(((e > 1 ? e : 1) + 120) << 23);
+    _Float16 t = (_Float16)(uint16_t)((b & 7) | (e1 << 3));
+    s.t = (f16x2){t, t};
+    return s;
+}
+// 8 codes of one u32 -> 8 fp16 (code * 2^E * t), elements in order
+__device__ __forceinline__ u32x4 fp4x8_to_f16(uint32_t w, Fp4Scale s) {
+    u32x4 o;
+    o[0] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, s.pow2, 0) * s.t));
+    o[1] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, s.pow2, 1) * s.t));
+    o[2] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, s.pow2, 2) * s.t));
+    o[3] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, s.pow2, 3) * s.t));
+    return o;
 }
 
 // ---- activation quantizer ------------------------------------------------------------------------------------------
@@ -134,7 +161,7 @@ struct Fp4Producer {
         u32x4 c[2];
         uint32_t s2[2];
     };
-    static constexpr int kStoreValu = 128;  // about the VALU instructions of store()
+    static constexpr int kStoreValu = 96;  // about the VALU instructions of store()
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
         r.c[half] = *(const u32x4*)(w + (size_t)kt * w_skt + 16 * half);
         r.s2[half] = *(const uint16_t*)(sw + (size_t)kt * s_skt + 2 * half);
@@ -144,16 +171,14 @@ struct Fp4Producer {
 #pragma unroll
         for (int d = 0; d < 8; d++) {
             if (d / 4 != part) continue;
-            uint32_t t[4];
-            e2m1x8_to_f16(r.c[d >> 2][d & 3], t);
-            f16x2 sc = e4m3_to_f16x2((r.s2[d >> 2] >> (8 * ((d >> 1) & 1))) & 0xff);
-            u32x4 o;
-#pragma unroll
-            for (int e = 0; e < 4; e++) o[e] = __builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[e]) * sc));
-            *(u32x4*)(Bs + gm_swz(row, d)) = o;
+            Fp4Scale sc = fp4_scale((r.s2[d >> 2] >> (8 * ((d >> 1) & 1))) & 0xff);
+            *(u32x4*)(Bs + gm_swz(row, d)) = fp4x8_to_f16(r.c[d >> 2][d & 3], sc);
         }
     }
 };
+
+// The fp16 operands are 2 x the quantized activation and 8 x the quantized weight.
+#define FP4_OPERAND_SCALE 0.0625f
 
 // One row piece of the output: 4 columns from `col` of row `grow`, bf16((sum) * alpha) (+ res: bf16(bf16(.) + res)).
 __device__ __forceinline__ void fp4_store4(uint16_t* c, const uint16_t* res, size_t at, const float (&v)[4], f32x4 al) {
@@ -203,7 +228,7 @@ extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, 
     const uint32_t colb = n0 + wn * 128;
     if (colb >= n) return;
     const uint32_t col = colb + 4 * (tid & 31);
-    f32x4 al = *(const f32x4*)(alpha + col) * 0.25f;
+    f32x4 al = *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE;
     gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t, float (&v)[4]) {
         uint32_t grow = m0 + wm * 128 + row;
         if (grow < m) fp4_store4(c, res, (size_t)grow * ldc + col, v, al);
@@ -220,6 +245,159 @@ extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t*
         uint32_t tm, tn;
         gemm_raster(full_tiles + t, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, tm, tn);
         uint32_t grow = tm * GM_BM + row, col = tn * GM_BN + cb * 128 + 4 * l32;
-        if (grow < m && col < n) fp4_store4(c, res, (size_t)grow * ldc + col, v, *(const f32x4*)(alpha + col) * 0.25f);
+        if (grow < m && col < n) fp4_store4(c, res, (size_t)grow * ldc + col, v, *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE);
     });
+}
+
+// ---- GEMV (1..16 rows) -------------------------------------------------------------------------------------------------
+
+#define FP4_GEMV_RG 8  // 16-row groups of a 128-row weight tile
+
+// One k tile of one 128-row weight tile as a wavefront reads it: lane L = 16 g + r takes, of row 16 rg + r, the 16 codes
+// k = 16 g .. 16 g + 15 (8 bytes) and the row's four scale bytes (it uses byte g), and of activation row r the same 16
+// values. The k index inside an MFMA is only a summation index, so the A operand (weights) and the B operand
+// (activations) merely have to agree: MFMA j of a row group multiplies k = 16 g + 8 j .. + 7 of lane group g.
+struct Fp4GemvStage {
+    u32x2 cw[FP4_GEMV_RG];
+    uint32_t sc[FP4_GEMV_RG];
+    f16x8 x[2];
+};
+
+// c[m][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res) for m <= 16 rows: the decode-sized form of fe_gemm_nvfp4, bound by
+// the read of the weights. grid (n / 128) * sk, 256 threads: a program takes one 128-row weight tile and one of sk runs
+// of k tiles, its four wavefronts alternate k tiles. Each wavefront expands its codes in registers straight into the
+// A operand of v_mfma_f32_16x16x32_f16 (rows = weight rows, columns = activation rows); the wavefronts' sums meet in
+// LDS. With sk > 1 the splits leave f32 partials in z[split][16][n]; the last to arrive (counters[tile]) adds them in
+// split order, finishes the tile and re-arms the counter, so the result does not depend on timing. Weight addressing as
+// in fe_gemm_nvfp4.
+extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
+                                                                   const uint8_t* sw, const float* alpha, const uint16_t* res,
+                                                                   float* z, uint32_t* counters, uint32_t m, uint32_t n,
+                                                                   uint32_t k, uint32_t ldc, uint32_t sk, uint32_t w_snt,
+                                                                   uint32_t w_skt, uint32_t w_sr, uint32_t s_snt,
+                                                                   uint32_t s_skt, uint32_t s_sr) {
+    __shared__ f32x4 red[4][FP4_GEMV_RG][64];
+    __shared__ uint32_t last_flag;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    const uint32_t nts = n / 128, nt = blockIdx.x % nts, split = blockIdx.x / nts;
+    const uint32_t ktiles = k / 64, kt_begin = split * ktiles / sk, kt_end = (split + 1) * ktiles / sk;
+    const uint8_t* wp = w + (size_t)nt * w_snt + (size_t)r * w_sr + 8 * g;
+    const uint8_t* sp = sw + (size_t)nt * s_snt + (size_t)r * s_sr;
+    const _Float16* xp = aq + (size_t)(r < m ? r : m - 1) * k + 16 * g;
+
+    auto load = [&](Fp4GemvStage& st, uint32_t kt) {
+        const uint8_t* wk = wp + (size_t)kt * w_skt;
+        const uint8_t* sk_ = sp + (size_t)kt * s_skt;
+#pragma unroll
+        for (int rg = 0; rg < FP4_GEMV_RG; rg++) {
+            st.cw[rg] = __builtin_nontemporal_load((const u32x2*)(wk + (size_t)(16 * rg) * w_sr));
+            st.sc[rg] = __builtin_nontemporal_load((const uint32_t*)(sk_ + (size_t)(16 * rg) * s_sr));
+        }
+        st.x[0] = *(const f16x8*)(xp + kt * 64);
+        st.x[1] = *(const f16x8*)(xp + kt * 64 + 8);
+    };
+    f32x4 acc[FP4_GEMV_RG];
+#pragma unroll
+    for (int rg = 0; rg < FP4_GEMV_RG; rg++) acc[rg] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const Fp4GemvStage& st) {
+#pragma unroll
+        for (int rg = 0; rg < FP4_GEMV_RG; rg++) {
+            Fp4Scale s = fp4_scale((st.sc[rg] >> (8 * g)) & 0xff);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                u32x4 a = fp4x8_to_f16(st.cw[rg][j], s);
+                acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), st.x[j], acc[rg], 0, 0, 0);
+            }
+        }
+    };
+    // Two k tiles in flight per wavefront. Loads past the end re-read the last k tile of the run (never used), which
+    // keeps the loop free of branches around memory instructions.
+    Fp4GemvStage s0, s1;
+    const uint32_t last = kt_end - 1;
+    auto clamp = [&](uint32_t t) { return t < last ? t : last; };
+    uint32_t kt = kt_begin + wave;
+    load(s0, clamp(kt));
+    load(s1, clamp(kt + 4));
+    // (the scheduling barriers keep each refill where it is written: the compiler otherwise sinks the loads to just
+    // before their use, a whole stage later)
+    for (; kt + 4 < kt_end; kt += 8) {
+        compute(s0);
+        __builtin_amdgcn_sched_barrier(0);
+        load(s0, clamp(kt + 8));
+        __builtin_amdgcn_sched_barrier(0);
+        compute(s1);
+        __builtin_amdgcn_sched_barrier(0);
+        load(s1, clamp(kt + 12));
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (kt < kt_end) compute(s0);
+    // the four wavefronts' sums meet in LDS; wavefront v finishes row groups 2 v and 2 v + 1
+#pragma unroll
+    for (int rg = 0; rg < FP4_GEMV_RG; rg++) red[wave][rg][lane] = acc[rg];
+    __syncthreads();
+    f32x4 sum[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        sum[h] = red[0][2 * wave + h][lane];
+#pragma unroll
+        for (int v = 1; v < 4; v++) sum[h] += red[v][2 * wave + h][lane];
+    }
+    // lane (r, g) holds, for row group rg, output row m = r, columns n0 + 16 rg + 4 g .. + 3
+    const uint32_t col = nt * 128 + 32 * wave + 4 * g;  // + 16 h
+    auto finish = [&](const f32x4 (&v)[2]) {
+        if (r >= m) return;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            uint32_t cc = col + 16 * h;
+            float o[4] = {v[h][0], v[h][1], v[h][2], v[h][3]};
+            fp4_store4(c, res, (size_t)r * ldc + cc, o, *(const f32x4*)(alpha + cc) * FP4_OPERAND_SCALE);
+        }
+    };
+    if (sk == 1) {
+        finish(sum);
+        return;
+    }
+    // Partials cross to another program, possibly on another XCD with its own L2: agent-scope accesses, ordered by the
+    // barriers around the arrival counter (the barrier waits for every lane's stores to be acknowledged).
+    if (r < m) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            float* dst = z + ((size_t)split * 16 + r) * n + col + 16 * h;
+#pragma unroll
+            for (int e = 0; e < 4; e++) __hip_atomic_store(dst + e, sum[h][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t old = __hip_atomic_fetch_add(&counters[nt], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_flag = (old == sk - 1);
+    }
+    __syncthreads();
+    if (!last_flag) return;
+    if (tid == 0) __hip_atomic_store(&counters[nt], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (r >= m) return;
+    // the loads of 8 splits are in flight together (an agent-scope load takes a trip to memory); sums in split order
+    f32x4 tot[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    for (uint32_t s0 = 0; s0 < sk; s0 += 8) {
+        float t[8][2][4];
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const uint32_t sp = s0 + b < sk ? s0 + b : sk - 1;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const float* src = z + ((size_t)sp * 16 + r) * n + col + 16 * h;
+#pragma unroll
+                for (int e = 0; e < 4; e++) t[b][h][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < 8; b++)
+            if (s0 + b < sk) {
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) tot[h][e] += t[b][h][e];
+            }
+    }
+    finish(tot);
 }

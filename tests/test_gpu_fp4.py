@@ -39,7 +39,8 @@ def fp4_check_activations(m, k, g, seed):
     return bf16_bits(x)
 
 
-@pytest.mark.parametrize("n,k,m,input_scale", [(256, 512, 200, 1.0), (128, 1024, 1, 0.037), (384, 256, 130, 2.5)])
+@pytest.mark.parametrize("n,k,m,input_scale", [(256, 512, 200, 1.0), (128, 1024, 1, 0.037), (384, 256, 130, 2.5),
+                                               (256, 512, 16, 1.0), (384, 1024, 37, 0.5), (640, 2048, 5, 1.0)])
 def test_fp4_linear(env, oracle, n, k, m, input_scale):
     torch, fp4, kern = env
     from ferrite_amd import synth
@@ -146,6 +147,41 @@ def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
     got = run(lin, res=res)
     want = bf16_bits(bf16_to_f32(cut) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m]))
     assert np.array_equal(got, want)
+
+
+def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
+    """Up to 64 rows run the weight-read-bound GEMV (16 rows a pass, K cut over several programs); FE_FP4_NO_GEMV sends
+    the same rows through the GEMM. Both sum the same exact products in f32, in different orders."""
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    n, k = 384, 2048
+    host = synth.fp4_linear(n, k, 31, input_scale=1.0)
+    host.alpha[:] = host.alpha * np.linspace(0.5, 2.0, n).astype(np.float32)
+    lin = host.upload()
+    view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), torch.from_numpy(host.sf).cuda(),
+                                      torch.from_numpy(host.alpha).cuda(), host.g)
+    for m in (1, 3, 16, 17, 64):
+        ws = fp4.Workspace(m, k)
+        xd = dev_u16(torch, fp4_check_activations(m, k, lin.g, 40 + m))
+        res = dev_u16(torch, bf16_bits(np.random.default_rng(m).normal(size=(m + 1, n)).astype(np.float32)))
+
+        def run(l, r=None):
+            y = torch.full((m + 1, n), -3.0, dtype=torch.bfloat16, device="cuda")
+            l.forward(kern, ws, y, n, xd, k, m, res=r)
+            torch.cuda.synchronize()
+            out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+            assert (out[m:] == bf16_bits(np.float32([-3.0]))[0]).all()
+            return out[:m]
+
+        gemv = run(lin)
+        assert np.array_equal(gemv, run(lin)) and np.array_equal(gemv, run(view))
+        with_res = run(lin, res)
+        assert np.array_equal(with_res, bf16_bits(bf16_to_f32(gemv) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m])))
+        monkeypatch.setenv("FE_FP4_NO_GEMV", "1")
+        gemm = run(lin)
+        monkeypatch.delenv("FE_FP4_NO_GEMV")
+        a, b = bf16_to_f32(gemv).astype(np.float64), bf16_to_f32(gemm).astype(np.float64)
+        assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all()
 
 
 def test_fp4_argument_errors(env):
