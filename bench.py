@@ -180,9 +180,34 @@ def main():
         "per_linear_gemv": per,
     }
 
+    out["graph_replay"] = graph_replay(lib, _lib.check, ev, exl3, linears, ws, total_bytes, args.steps, args.warmup)
     if not args.no_prefill:
         out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
     print(json.dumps(out))
+
+
+def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):
+    """The same step captured once into a HIP graph on a stream of its own and replayed: what the step costs when the
+    host does not launch 18 kernels one by one. Reported beside `value`, which stays the eagerly launched step."""
+    s = C.c_void_p()
+    check(lib.fe_hip_stream_create(C.byref(s)))
+    check(lib.fe_hip_graph_begin(s))
+    for name, bits, lin, x, y in linears:
+        lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws, stream=s)
+        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws, stream=s)
+    g = C.c_void_p()
+    check(lib.fe_hip_graph_end(s, C.byref(g)))
+    for _ in range(max(warmup, 2)):
+        check(lib.fe_hip_graph_launch(g, s))
+    a, b = ev.new(), ev.new()
+    ev.record(a, s)
+    for _ in range(steps):
+        check(lib.fe_hip_graph_launch(g, s))
+    ev.record(b, s)
+    ms = ev.ms(a, b) / steps
+    check(lib.fe_hip_graph_destroy(g))
+    return {"ms_per_step": round(ms, 5), "GB/s": round(total_bytes / ms / 1e6, 1),
+            "pct_hbm_peak": round(100 * total_bytes / ms / 1e6 / HBM_PEAK_GBS, 2)}
 
 
 def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=17408):
@@ -232,8 +257,21 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
         flin.quantize(fk, fws, xf, k, m)
     ev.record(b2, stream)
     q_ms = ev.ms(a2, b2) / reps
-    res["nvfp4_17408x5120"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+    res["nvfp4_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                                "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "quant_ms": round(q_ms, 4)}
+    # NVFP4 at M = 1: the weight-read-bound GEMV over the same linear (codes + block scales = 9/16 byte a weight)
+    flin.quantize(fk, fws, xf, k, 1)
+    reps = 50
+    pairs = [(ev.new(), ev.new()) for _ in range(reps)]
+    flin.gemm(fk, fws, yf, n, 1)
+    for a, b in pairs:
+        ev.record(a, stream)
+        flin.gemm(fk, fws, yf, n, 1)
+        ev.record(b, stream)
+    us = sum(ev.ms(a, b) for a, b in pairs) / reps * 1e3
+    wbytes = n * k // 2 + n * k // 16
+    res["nvfp4_5120x17408_m1"] = {"gemv_us": round(us, 2), "GB/s": round(wbytes / us / 1e3, 1),
+                                  "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res
 
 

@@ -160,9 +160,12 @@ def default_blocks(cu_count: int) -> int:
 
 
 def _stream(s):
+    """A stream argument: None = torch's current stream, a torch stream, a raw handle (int) or a ctypes pointer."""
     if s is None:
         import torch
         s = torch.cuda.current_stream()
+    if isinstance(s, C.c_void_p):
+        return s
     return C.c_void_p(getattr(s, "cuda_stream", s))
 
 
