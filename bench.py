@@ -29,6 +29,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
+# `bench.py --traffic-pass` (profiles/exl3_gemv_stream_b4_m1_hbm_traffic.md): 22534 KiB fetched x 2.0 (the factor that
+# makes the counter read a streaming read and an elementwise update of known size correctly) + 1338 KiB written x 1.0
+ROOFLINE_TRAFFIC_BYTES = int((22534 * 2.0 + 1338 * 1.0) * 1024)
 MFMA_F16_PEAK_TFLOPS = 2500.0
 SEED = 20251
 MLP = [("gate", 5120, 17408), ("up", 5120, 17408), ("down", 17408, 5120)]
@@ -90,6 +94,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--traffic-pass", action="store_true",
+                    help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a streaming read and an elementwise update of "
+                         "known size (the counters' calibration), then the roofline kernel, caches evicted in between")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures the hot path on one GPU; --gpus must be 1 (no multi-GPU path exists)")
@@ -100,6 +107,8 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU")
+    if args.traffic_pass:
+        return traffic_pass(torch, np, exl3, synth)
     cpu = None
     if not args.no_cpu:
         cpu, y_cpu = cpu_baseline()  # first, as the configuration asks
@@ -174,7 +183,7 @@ def main():
                    "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "kernel": "exl3_gemv_stream_b4 (5120x17408, M=1)", "achieved": round(achieved, 2),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ROOFLINE_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms)},
         "cpu_baseline": cpu,
         "per_linear_gemv": per,
@@ -184,6 +193,29 @@ def main():
     if not args.no_prefill:
         out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
     print(json.dumps(out))
+
+
+def traffic_pass(torch, np, exl3, synth):
+    """Three rounds of: evict (an elementwise update of 600 MiB: reads 600 MiB, writes 600 MiB), exl3_probe_v4 reading
+    exactly the roofline kernel's algorithmic bytes, evict, the roofline kernel. Prints the known sizes."""
+    kern = exl3.Kernels.load()
+    k, n = 5120, 17408
+    t = synth.exl3_tensor(k, n, 4, SEED, "gate")
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), exl3.default_blocks(exl3.cu_count()))
+    ws = exl3.Workspace([lin], 1)
+    x = torch.from_numpy(synth.activations(1, k, SEED).view(np.int16)).cuda()
+    y = torch.zeros((1, n), dtype=torch.bfloat16, device="cuda")
+    buf = torch.zeros(lin.weight_bytes(), dtype=torch.uint8, device="cuda")
+    big = torch.zeros(600 << 20, dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        big.add_(1)
+        kern.probe_stream_read(buf, 1024, 1)
+        big.add_(1)
+        lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
+        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
+    torch.cuda.synchronize()
+    print(json.dumps({"exl3_probe_v4_reads_KiB": lin.weight_bytes() / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
+                      "roofline_kernel": "exl3_gemv_stream_b4", "algorithmic_KiB": lin.weight_bytes() / 1024}))
 
 
 def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):

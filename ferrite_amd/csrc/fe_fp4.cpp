@@ -208,9 +208,10 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
     if (m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
-        // decode-sized: the weight-read-bound GEMV, 16 rows a pass. Programs: about three a CU.
+        // decode-sized: the weight-read-bound GEMV, 16 rows a pass. Two programs fit a CU: as many programs as run at
+        // once, not more (a second round of short programs costs more than idle CUs in the first).
         const uint32_t nts = n / kTile, kts = k / 64;
-        uint32_t sk = (3 * kern->cus + nts / 2) / nts;
+        uint32_t sk = 2 * kern->cus / nts;
         if (const char *e = getenv("FE_FP4_GEMV_SK")) sk = (uint32_t)atoi(e);
         if (sk > 16) sk = 16;
         if (sk > kts / 4) sk = kts / 4;
