@@ -449,11 +449,10 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     // device-wide cache write-back or invalidate is needed.
     for (uint32_t row = hw; row < m; row += 8) {
         const float* src = red + row * GEMV_RED_PITCH + 4 * l32;
-        float* dst = z + ((size_t)split * m + row) * n + col0 + 4 * l32;
-#pragma unroll
-        for (int e = 0; e < 4; e++) __hip_atomic_store(dst + e, src[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        store_agent_f32x4(z + ((size_t)split * m + row) * n + col0 + 4 * l32, *(const f32x4*)src);
     }
-    __syncthreads();  // every lane's stores are acknowledged (s_waitcnt vmcnt(0)) before the barrier
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's stores are acknowledged at agent scope
+    __syncthreads();
     if (tid == 0) {
         uint32_t old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         last_flag = (old == sk - 1);
@@ -463,10 +462,17 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
         for (uint32_t row = hw; row < m; row += 8) {
             size_t at = (size_t)row * n + col0 + 4 * l32;
             float v[4] = {0.f, 0.f, 0.f, 0.f};
-            for (uint32_t sp = 0; sp < sk; sp++) {
-                const float* src = z + (size_t)sp * m * n + at;
+            for (uint32_t sp0 = 0; sp0 < sk; sp0 += 8) {  // 8 splits' loads in flight, summed in split order
+                f32x4 t[8];
 #pragma unroll
-                for (int e = 0; e < 4; e++) v[e] += __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                for (int b = 0; b < 8; b++) t[b] = load_agent_f32x4(z + (size_t)(sp0 + b < sk ? sp0 + b : sk - 1) * m * n + at);
+                agent_loads_wait(t);
+#pragma unroll
+                for (int b = 0; b < 8; b++)
+                    if (sp0 + b < sk) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] += t[b][e];
+                    }
             }
             finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, at);
         }
@@ -593,14 +599,10 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh
         const uint32_t col0 = nb * 128;
         const uint32_t first_prog = stream_owner(nb * steps, base, rem), last_prog = stream_owner(nb * steps + steps - 1, base, rem);
         if (r < m) {
-            float* zp = z + ((size_t)(p + nb) * m + r) * 128 + 32 * wave;
-#pragma unroll
-            for (int h = 0; h < 2; h++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    uint32_t arow = 4 * g + i;  // row of A: tile arow >> 3 of the pair, n = (arow & 7) + 8 h
-                    __hip_atomic_store(zp + 16 * (arow >> 3) + (arow & 7) + 8 * h, acc[h][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                }
+            // A rows 4 g .. 4 g + 3 of half h are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32
+            float* zp = z + ((size_t)(p + nb) * m + r) * 128 + 32 * wave + 16 * (g >> 1) + 4 * (g & 1);
+            store_agent_f32x4(zp, acc[0]);
+            store_agent_f32x4(zp + 8, acc[1]);
         }
         acc[0] = acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums are acknowledged at agent scope
@@ -623,14 +625,13 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh
                 const bool live = row < m;
                 float v[4] = {0.f, 0.f, 0.f, 0.f};
                 for (uint32_t sp0 = first_prog; sp0 <= last_prog; sp0 += 8) {
-                    float t[8][4];
+                    f32x4 t[8];
 #pragma unroll
                     for (int b = 0; b < 8; b++) {
                         const uint32_t sp = sp0 + b <= last_prog ? sp0 + b : last_prog;
-                        const float* src = z + ((size_t)(sp + nb) * m + (live ? row : 0)) * 128 + 4 * l32;
-#pragma unroll
-                        for (int e = 0; e < 4; e++) t[b][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        t[b] = load_agent_f32x4(z + ((size_t)(sp + nb) * m + (live ? row : 0)) * 128 + 4 * l32);
                     }
+                    agent_loads_wait(t);
 #pragma unroll
                     for (int b = 0; b < 8; b++)
                         if (sp0 + b <= last_prog) {

@@ -358,15 +358,12 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
         return;
     }
     // Partials cross to another program, possibly on another XCD with its own L2: agent-scope accesses, ordered by the
-    // barriers around the arrival counter (the barrier waits for every lane's stores to be acknowledged).
+    // barriers around the arrival counter.
     if (r < m) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            float* dst = z + ((size_t)split * 16 + r) * n + col + 16 * h;
-#pragma unroll
-            for (int e = 0; e < 4; e++) __hip_atomic_store(dst + e, sum[h][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        for (int h = 0; h < 2; h++) store_agent_f32x4(z + ((size_t)split * 16 + r) * n + col + 16 * h, sum[h]);
     }
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's stores are acknowledged at agent scope
     __syncthreads();
     if (tid == 0) {
         uint32_t old = __hip_atomic_fetch_add(&counters[nt], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -379,24 +376,19 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
     // the loads of 8 splits are in flight together (an agent-scope load takes a trip to memory); sums in split order
     f32x4 tot[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
     for (uint32_t s0 = 0; s0 < sk; s0 += 8) {
-        float t[8][2][4];
+        f32x4 t[16];
 #pragma unroll
         for (int b = 0; b < 8; b++) {
             const uint32_t sp = s0 + b < sk ? s0 + b : sk - 1;
 #pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const float* src = z + ((size_t)sp * 16 + r) * n + col + 16 * h;
-#pragma unroll
-                for (int e = 0; e < 4; e++) t[b][h][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            for (int h = 0; h < 2; h++) t[2 * b + h] = load_agent_f32x4(z + ((size_t)sp * 16 + r) * n + col + 16 * h);
         }
+        agent_loads_wait(t);
 #pragma unroll
         for (int b = 0; b < 8; b++)
             if (s0 + b < sk) {
 #pragma unroll
-                for (int h = 0; h < 2; h++)
-#pragma unroll
-                    for (int e = 0; e < 4; e++) tot[h][e] += t[b][h][e];
+                for (int h = 0; h < 2; h++) tot[h] += t[2 * b + h];
             }
     }
     finish(tot);

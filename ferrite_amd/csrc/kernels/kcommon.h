@@ -80,3 +80,22 @@ __device__ __forceinline__ void fwht128_half_wave(float (&v)[4], uint32_t lane) 
         v[q] = x;
     }
 }
+
+// 16 bytes at agent scope: partial sums that one program leaves for another, possibly on another XCD with its own L2.
+// The store goes through to memory, the load reads past this XCD's L2 (the sc1 forms that clang emits for 4-byte
+// agent-scope atomics; it has no 16-byte ones). The compiler does not count these loads: agent_loads_wait must come
+// between the last load and the first use of any loaded value.
+__device__ __forceinline__ void store_agent_f32x4(float* p, f32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ f32x4 load_agent_f32x4(const float* p) {
+    f32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void agent_loads_wait(f32x4 (&t)[N]) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < N; i++) asm volatile("" : "+v"(t[i]));
+}
