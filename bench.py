@@ -30,9 +30,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
-# `bench.py --traffic-pass` (profiles/exl3_gemv_stream_b4_m1_hbm_traffic.md): 22534 KiB fetched x 2.0 (the factor that
-# makes the counter read a streaming read and an elementwise update of known size correctly) + 1338 KiB written x 1.0
-ROOFLINE_TRAFFIC_BYTES = int((22534 * 2.0 + 1338 * 1.0) * 1024)
+# `bench.py --traffic-pass` (profiles/exl3_gemv_b4_r1_m1_hbm_traffic.md): 22363 KiB fetched x 2.0 (the factor that
+# makes the counter read a streaming read and an elementwise update of known size correctly) + 400 KiB written x 1.0
+ROOFLINE_TRAFFIC_BYTES = int((22363 * 2.0 + 400 * 1.0) * 1024)
 MFMA_F16_PEAK_TFLOPS = 2500.0
 SEED = 20251
 MLP = [("gate", 5120, 17408), ("up", 5120, 17408), ("down", 17408, 5120)]
@@ -171,6 +171,7 @@ def main():
         if bits == 4 and lin.k == 5120:
             dom_ms += ms
             dom_bytes = lin.weight_bytes()
+            dom_kernel = "exl3_gemv_stream_b4" if lin.plan.ver == 2 else "exl3_gemv_b4_r1"
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
 
@@ -182,7 +183,7 @@ def main():
         "config": {"workload": "EXL3 decode MLP, Qwen3.8-27B-shaped layer, M=1, 3/4/5 bpw (gate, up 5120x17408; down 17408x5120)",
                    "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
-        "roofline": {"bound": "hbm", "kernel": "exl3_gemv_stream_b4 (5120x17408, M=1)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (5120x17408, M=1)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ROOFLINE_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms)},
         "cpu_baseline": cpu,
@@ -215,7 +216,7 @@ def traffic_pass(torch, np, exl3, synth):
         lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
     torch.cuda.synchronize()
     print(json.dumps({"exl3_probe_v4_reads_KiB": lin.weight_bytes() / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
-                      "roofline_kernel": "exl3_gemv_stream_b4", "algorithmic_KiB": lin.weight_bytes() / 1024}))
+                      "roofline_kernel": "exl3_gemv_b4_r1", "algorithmic_KiB": lin.weight_bytes() / 1024}))
 
 
 def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):

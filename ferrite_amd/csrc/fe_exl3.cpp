@@ -143,16 +143,20 @@ int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_
     (void)bits;
     if (!out || !k || !n || k % 128 || n % 128) return fe_set_error(FE_ERR_SHAPE, "fe_exl3_plan_for", "k, n must be multiples of 128");
     const uint32_t steps = k / 64, nb = n / 128, min_steps = 2;
+    // the divisor of the step count whose program count nb * d comes closest (as a ratio) to `blocks`
     uint32_t sk = 1;
+    double best = 1e30;
     for (uint32_t d = 1; d <= steps; d++) {
         if (steps % d) continue;
         if (steps / d < min_steps) break;
-        sk = d;
-        if (nb * d >= blocks) break;
+        double ratio = (double)nb * d / (blocks ? blocks : 1);
+        double miss = ratio < 1.0 ? 1.0 / ratio : ratio;
+        if (miss < best) best = miss, sk = d;
     }
     if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) sk = 1;
-    // ver 2: rows 1..16 run the streamed GEMV with occ programs per CU (FE_EXL3_STREAM=0: the split-K form only)
-    uint32_t ver = env_is("FE_EXL3_STREAM", "0") ? 1 : 2, occ = 2;
+    // ver 1: the split-K GEMV for 1..64 rows, one summation order for all of them. ver 2 (FE_EXL3_STREAM=1): rows 1..16
+    // run the streamed GEMV with occ programs per CU instead.
+    uint32_t ver = env_is("FE_EXL3_STREAM", "1") ? 2 : 1, occ = 2;
     if (const char *o = getenv("FE_EXL3_OCC")) occ = (uint32_t)atoi(o);
     *out = fe_exl3_plan{sk, 4, ver, ver == 2 ? occ : 0};
     return 0;
