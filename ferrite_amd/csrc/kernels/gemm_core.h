@@ -212,10 +212,18 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
 
 // Hands the wavefront's 128 x 128 accumulators out row by row: 32 rows at a time pass through the wavefront's own LDS
 // slab (GM_EPI_SLAB bytes at lds + wave * GM_EPI_SLAB) so that 32 consecutive lanes hold 128 consecutive columns of one
-// row, 4 a lane. fn(row in 0..127, l32, v[4]) is called by both halves of the wavefront, each with its own row. No
-// workgroup barrier: only this wavefront touches its slab.
-template <class RowFn>
-__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[4][4], unsigned char* lds, RowFn fn) {
+// row, 4 a lane. Both halves of the wavefront work on a row of their own. Four row pairs are in flight together:
+// transform(v[4][4], l32) works on all four at once (it must not branch, so that its cross-lane exchanges overlap),
+// after that store(row in 0..127, l32, v[4]) is called for each. No workgroup barrier: only this
+// wavefront touches its slab.
+// Orders the wavefront's own LDS writes before its own LDS reads (and the other way round): the lanes of a wavefront
+// issue their LDS instructions together and the LDS executes them in order, so only the compiler has to be kept from
+// moving accesses across this point. (A workgroup-scope fence would also wait for the global stores in flight, once
+// per 32 rows.)
+__device__ __forceinline__ void gm_slab_sync() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+template <class Transform, class Store>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[4][4], unsigned char* lds, Transform transform, Store store) {
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, l32 = lane & 31, hw = lane >> 5;
     float* slab = (float*)(lds + wave * GM_EPI_SLAB);
 #pragma unroll
@@ -225,17 +233,19 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[4][4], unsigned char
 #pragma unroll
             for (int e = 0; e < 16; e++)
                 slab[(8 * (e >> 2) + 4 * hw + (e & 3)) * GM_EPI_PITCH + 32 * j + l32] = acc[i][j][e];
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-        __builtin_amdgcn_wave_barrier();
-#pragma unroll 4
-        for (int rr = 0; rr < 16; rr++) {
-            uint32_t row = 2 * rr + hw;
-            f32x4 t = *(const f32x4*)(slab + row * GM_EPI_PITCH + 4 * l32);
-            float v[4] = {t[0], t[1], t[2], t[3]};
-            fn(32 * i + row, l32, v);
+        gm_slab_sync();
+        for (int rr = 0; rr < 16; rr += 4) {
+            float v[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                f32x4 t = *(const f32x4*)(slab + (2 * (rr + u) + hw) * GM_EPI_PITCH + 4 * l32);
+                v[u][0] = t[0], v[u][1] = t[1], v[u][2] = t[2], v[u][3] = t[3];
+            }
+            transform(v, l32);
+#pragma unroll
+            for (int u = 0; u < 4; u++) store(32 * i + 2 * (rr + u) + hw, l32, v[u]);
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-        __builtin_amdgcn_wave_barrier();
+        gm_slab_sync();
     }
 }
 
@@ -244,9 +254,11 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[4][4], unsigned char
 // Leaves the program's accumulators in its partial slot, row-major [256][256] f32.
 __device__ __forceinline__ void gemm_store_partial(f32x16 (&acc)[4][4], unsigned char* lds, float* slot) {
     const uint32_t wave = threadIdx.x >> 6, wm = wave >> 1, wn = wave & 1;
-    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t l32, float (&v)[4]) {
-        *(f32x4*)(slot + (wm * 128 + row) * GM_BN + wn * 128 + 4 * l32) = (f32x4){v[0], v[1], v[2], v[3]};
-    });
+    gemm_epilogue(
+        acc, lds, [](float (&)[4][4], uint32_t) {},
+        [&](uint32_t row, uint32_t l32, float (&v)[4]) {
+            *(f32x4*)(slot + (wm * 128 + row) * GM_BN + wn * 128 + 4 * l32) = (f32x4){v[0], v[1], v[2], v[3]};
+        });
 }
 
 // Body of a reduce kernel: grid (tiles cut along K) * 64, 256 threads. Each half wavefront sums the `splits` slots of one

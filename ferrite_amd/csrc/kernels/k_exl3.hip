@@ -6,6 +6,8 @@
 // t = 8 * f + i sits at row k = 2 (f & 3) + (i & 1) + 8 ((i >> 1) & 1), column n = (f >> 2) + 8 (i >> 2) of the tile
 // (crates/fe-exl3/src/format.rs:146-156). A state decodes to fp16 by the mul1 codebook
 // (crates/fe-exl3/src/cpu.rs:25-43, kernels/k-exl3/src/util.rs:76-85).
+#include <type_traits>
+
 #include "gemm_core.h"
 
 // ---- the mul1 codebook ------------------------------------------------------------------------------------------
@@ -308,6 +310,12 @@ __device__ __forceinline__ void finish_row(float (&v)[4], uint32_t l32, const ui
     store4(y, mode, at, v);
 }
 
+// The lane's four output scales as finish_row applies them, for callers that finish many rows of the same columns.
+__device__ __forceinline__ f32x4 row_scales(const uint16_t* svh, uint32_t col) {
+    u32x2 s = *(const u32x2*)(svh + col);
+    return (f32x4){f16_bits_to_f32(s[0] & 0xffff), f16_bits_to_f32(s[0] >> 16), f16_bits_to_f32(s[1] & 0xffff),
+                   f16_bits_to_f32(s[1] >> 16)};
+}
 #define GEMV_RED_PITCH 132  // floats a row of the 128-column partial sums (16-byte aligned, banks spread)
 
 // y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for m <= 16 RG rows. grid (n / 128 * sk), 256 threads. The rotated
@@ -756,11 +764,33 @@ __device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, 
     }
     const uint32_t nb = 2 * tn + wn;
     if (nb >= nbs) return;
-    const uint32_t col0 = nb * 128;
-    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t l32, float (&v)[4]) {
-        uint32_t grow = m0 + wm * 128 + row;
-        if (grow < m) finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)grow * n + col0 + 4 * l32);
-    });
+    const uint32_t col = nb * 128 + 4 * (lane & 31);
+    const f32x4 sc = row_scales(svh, col);
+    // one copy of the epilogue per output mode, so that the row loop has no mode branches
+    auto run = [&](auto mode_tag) {
+        constexpr uint32_t MODE = decltype(mode_tag)::value;
+        gemm_epilogue(
+            acc, lds,
+            [&](float (&v)[4][4], uint32_t l32) {
+                fwht128_half_wave_rows(v, l32);
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[u][e] = v[u][e] * FE_HAD_SCALE * sc[e];  // finish_row's products
+            },
+            [&](uint32_t row, uint32_t, float (&v)[4]) {
+                uint32_t grow = m0 + wm * 128 + row;
+                if (grow < m) store4(y, MODE, (size_t)grow * n + col, v);
+            });
+    };
+    if (y_mode == 0)
+        run(std::integral_constant<uint32_t, 0>{});
+    else if (y_mode == 1)
+        run(std::integral_constant<uint32_t, 1>{});
+    else if (y_mode == 2)
+        run(std::integral_constant<uint32_t, 2>{});
+    else
+        run(std::integral_constant<uint32_t, 3>{});
 }
 
 // Finishes the tiles that exl3_gemm_b* cut along K: sums their partial slots and applies the output rotation and scale.

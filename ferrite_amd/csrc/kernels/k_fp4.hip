@@ -229,10 +229,12 @@ extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, 
     if (colb >= n) return;
     const uint32_t col = colb + 4 * (tid & 31);
     f32x4 al = *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE;
-    gemm_epilogue(acc, lds, [&](uint32_t row, uint32_t, float (&v)[4]) {
-        uint32_t grow = m0 + wm * 128 + row;
-        if (grow < m) fp4_store4(c, res, (size_t)grow * ldc + col, v, al);
-    });
+    gemm_epilogue(
+        acc, lds, [](float (&)[4][4], uint32_t) {},
+        [&](uint32_t row, uint32_t, float (&v)[4]) {
+            uint32_t grow = m0 + wm * 128 + row;
+            if (grow < m) fp4_store4(c, res, (size_t)grow * ldc + col, v, al);
+        });
 }
 
 // Finishes the tiles that fe_gemm_nvfp4 cut along K. grid (tiles - full_tiles) * 64, 256 threads.

@@ -48,12 +48,54 @@ __device__ __forceinline__ float swz_xor(float v) {
     return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), (MASK << 10) | 0x1f));
 }
 
+// A DPP move: every lane reads a lane of its own row of 16, so no lane is out of bounds and bound_ctrl costs nothing; it
+// lets the compiler fold the move into the add that consumes it.
+template <int CTRL>
+__device__ __forceinline__ float dpp_mov(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+#define DPP_QUAD_XOR1 0xB1     // quad_perm [1,0,3,2]: lane ^ 1
+#define DPP_QUAD_XOR2 0x4E     // quad_perm [2,3,0,1]: lane ^ 2
+#define DPP_QUAD_XOR3 0x1B     // quad_perm [3,2,1,0]: lane ^ 3
+#define DPP_HALF_MIRROR 0x141  // lane ^ 7 inside 8 lanes
+#define DPP_ROW_MIRROR 0x140   // lane ^ 15 inside 16 lanes
+
 template <int MASK>
 __device__ __forceinline__ float dpp_quad_xor(float v) {
     static_assert(MASK == 1 || MASK == 2, "quad permutes cover lane ^ 1 and lane ^ 2");
-    // quad_perm selectors: [1,0,3,2] = 0xB1, [2,3,0,1] = 0x4E
-    constexpr int ctrl = MASK == 1 ? 0xB1 : 0x4E;
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, 0xf, 0xf, false));
+    return dpp_mov<MASK == 1 ? DPP_QUAD_XOR1 : DPP_QUAD_XOR2>(v);
+}
+
+// One butterfly stage across lanes for N values at once: partner + sign * own, sign -1 on the lane whose bit is set.
+// Written stage by stage over all the values so that the independent chains interleave.
+template <int N>
+__device__ __forceinline__ void fwht_lane_stages(float (&x)[N], uint32_t lane) {
+    const float s1 = (lane & 1) ? -1.f : 1.f, s2 = (lane & 2) ? -1.f : 1.f, s4 = (lane & 4) ? -1.f : 1.f;
+    const float s8 = (lane & 8) ? -1.f : 1.f, s16 = (lane & 16) ? -1.f : 1.f;
+    float t[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) t[i] = x[i] * s1;
+#pragma unroll
+    for (int i = 0; i < N; i++) x[i] = dpp_mov<DPP_QUAD_XOR1>(x[i]) + t[i];
+#pragma unroll
+    for (int i = 0; i < N; i++) t[i] = x[i] * s2;
+#pragma unroll
+    for (int i = 0; i < N; i++) x[i] = dpp_mov<DPP_QUAD_XOR2>(x[i]) + t[i];
+    // lane ^ 4 = mirror of 8 (lane ^ 7), then mirror of 4 (lane ^ 3); lane ^ 8 = mirror of 16, then mirror of 8
+    float u[N];
+#pragma unroll
+    for (int i = 0; i < N; i++) t[i] = x[i] * s4, u[i] = dpp_mov<DPP_HALF_MIRROR>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; i++) x[i] = dpp_mov<DPP_QUAD_XOR3>(u[i]) + t[i];
+#pragma unroll
+    for (int i = 0; i < N; i++) t[i] = x[i] * s8, u[i] = dpp_mov<DPP_ROW_MIRROR>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; i++) x[i] = dpp_mov<DPP_HALF_MIRROR>(u[i]) + t[i];
+    // lane ^ 16 crosses rows of 16: through the LDS crossbar
+#pragma unroll
+    for (int i = 0; i < N; i++) u[i] = swz_xor<16>(x[i]);
+#pragma unroll
+    for (int i = 0; i < N; i++) x[i] = __builtin_fmaf(x[i], s16, u[i]);
 }
 
 // Unscaled natural-order (Sylvester) Walsh-Hadamard transform of 128 f32 held by 32 consecutive lanes, 4 a lane
@@ -64,21 +106,23 @@ __device__ __forceinline__ void fwht128_half_wave(float (&v)[4], uint32_t lane) 
     v[1] = b + d;
     v[2] = a - c;
     v[3] = b - d;
+    fwht_lane_stages(v, lane);
+}
+
+// The same for R rows at once (v[r] as above), the rows' chains interleaved.
+template <int R>
+__device__ __forceinline__ void fwht128_half_wave_rows(float (&v)[R][4], uint32_t lane) {
+    float x[4 * R];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        float x = v[q], o;
-        o = dpp_quad_xor<1>(x);
-        x = (lane & 1) ? o - x : x + o;
-        o = dpp_quad_xor<2>(x);
-        x = (lane & 2) ? o - x : x + o;
-        o = swz_xor<4>(x);
-        x = (lane & 4) ? o - x : x + o;
-        o = swz_xor<8>(x);
-        x = (lane & 8) ? o - x : x + o;
-        o = swz_xor<16>(x);
-        x = (lane & 16) ? o - x : x + o;
-        v[q] = x;
+    for (int r = 0; r < R; r++) {
+        float a = v[r][0] + v[r][1], b = v[r][0] - v[r][1], c = v[r][2] + v[r][3], d = v[r][2] - v[r][3];
+        x[4 * r] = a + c, x[4 * r + 1] = b + d, x[4 * r + 2] = a - c, x[4 * r + 3] = b - d;
     }
+    fwht_lane_stages(x, lane);
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) v[r][q] = x[4 * r + q];
 }
 
 // 16 bytes at agent scope: partial sums that one program leaves for another, possibly on another XCD with its own L2.

@@ -224,7 +224,7 @@ def test_tp_slices_match_the_whole(env, oracle):
     assert np.abs(parts - whole).max() / rms < 2e-5  # exl3-tpcheck.rs:103-105
 
 
-@pytest.mark.parametrize("bits,m", [(4, 200), (3, 129), (5, 65)])
+@pytest.mark.parametrize("bits,m", [(4, 200), (3, 129), (5, 65), (2, 300), (6, 257), (8, 70)])
 def test_prefill_gemm_matches_the_oracle(env, oracle, bits, m):
     """More than 64 rows take the LDS-staged MFMA GEMM; same contract as the GEMV (f64 reference on the GPU's own xh)."""
     torch, exl3, kern = env
