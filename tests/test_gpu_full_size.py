@@ -1,0 +1,153 @@
+"""Parity at the benchmark's own sizes, where the CPU oracle would take minutes per case: the kernels are checked through
+properties that do not depend on the size.
+
+EXL3: the GPU's W_hat (reconstruct_hat_f16, bit-exact against the oracle on whole small tensors in test_gpu_exl3.py) is
+checked here against the oracle's decode_tile on sampled tiles of the full tensor; then every GEMV / GEMM output must
+equal H(xh . W_hat) * svh / sqrt(128) computed by plain torch matmuls over that W_hat and the kernel's own rotated input
+(f64 for decode-sized M, f32 for M = 2048), within the same bounds as the small cases. Rows of a batch must repeat the
+bits of the single-row call (one summation order for 1..64 rows).
+
+NVFP4: outputs against torch matmuls over the oracle's dequantization of the same quantized operands.
+
+Shapes: hidden 5120, 40 heads x 128, 8 KV heads, MLP 17408 (q, o 5120x5120; k, v 5120x1024; gate, up 5120x17408; down
+17408x5120), M in {1, 4, 8, 16, 2048}."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = {"qo": (5120, 5120), "kv": (5120, 1024), "gate_up": (5120, 17408), "down": (17408, 5120)}
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from ferrite_amd import exl3
+    assert torch.cuda.is_available()
+    return torch, exl3, exl3.Kernels.load()
+
+
+def dev_u16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def hadamard128(torch, dtype):
+    i = torch.arange(128, device="cuda")
+    bits = i[:, None] & i[None, :]
+    pop = torch.zeros_like(bits)
+    for b in range(7):
+        pop += (bits >> b) & 1
+    return (1 - 2 * (pop & 1)).to(dtype)  # H[i][j] = (-1)^popcount(i & j)
+
+
+class Layer:
+    """One EXL3 linear at full size with its GPU-reconstructed W_hat."""
+
+    def __init__(self, env, oracle, k, n, bits, seed):
+        torch, exl3, kern = env
+        from ferrite_amd import synth
+        self.t = synth.exl3_tensor(k, n, bits, seed)
+        self.lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(self.t), exl3.default_blocks(exl3.cu_count()))
+        stored = exl3.DeviceExl3.upload(self.t)
+        w = torch.zeros((k, n), dtype=torch.int16, device="cuda")
+        kern.reconstruct_hat_f16(stored.view, w)
+        torch.cuda.synchronize()
+        self.w_hat = w.view(torch.float16)
+        # the decoder at this size: sampled tiles against the oracle, bit for bit
+        rng = np.random.default_rng(seed)
+        for kt, nt in zip(rng.integers(0, k // 16, 48), rng.integers(0, n // 16, 48)):
+            want = oracle.decode_tile(self.t.tile(int(kt), int(nt)), bits)
+            got = w[kt * 16:kt * 16 + 16, nt * 16:nt * 16 + 16].cpu().numpy().view(np.uint16)
+            assert np.array_equal(got, want), (kt, nt)
+        self.svh = torch.from_numpy(self.t.svh.view(np.float16).astype(np.float64)).cuda()
+
+    def reference(self, torch, xh, dtype):
+        """H(xh . W_hat) * svh / sqrt(128) from torch matmuls; xh: fp16 [m][k] on the device."""
+        m, n = xh.shape[0], self.t.n
+        s = xh.to(dtype) @ self.w_hat.to(dtype)
+        s = (s.view(m, n // 128, 128) @ hadamard128(torch, dtype)).view(m, n)
+        return (s.double() * self.svh / np.sqrt(128.0)).cpu().numpy()
+
+
+def run_rows(env, layer, m, seed, outliers=False):
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    lin = layer.lin
+    ws = exl3.Workspace([lin], m)
+    xd = dev_u16(torch, synth.activations(m, lin.k, seed, outliers=outliers))
+    y = torch.full((m + 1, lin.n), float("nan"), dtype=torch.float32, device="cuda")
+    lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+    yb = torch.zeros((m, lin.n), dtype=torch.bfloat16, device="cuda")
+    lin.forward(xd, exl3.Dtype.Bf16, yb, exl3.Dtype.Bf16, m, ws)
+    torch.cuda.synchronize()
+    xh = torch.from_numpy(ws.xh(m, lin.k).view(np.int16)).cuda().view(torch.float16)
+    got = y.cpu().numpy()
+    assert np.isnan(got[m]).all()
+    return xd, xh, got[:m].astype(np.float64), yb.float().cpu().numpy().astype(np.float64), ws
+
+
+def check(got, got_bf16, ref, f32_bound):
+    rms = np.sqrt((ref ** 2).mean())
+    assert np.abs(got - ref).max() / rms < f32_bound
+    # bf16 output: one rounding of the same sum
+    assert np.all(np.abs(got_bf16 - ref) <= np.abs(ref) / 256.0 + f32_bound * rms)
+    # the bar of the benchmark: max relative error 1e-2, denominators floored at the output's rms
+    assert (np.abs(got_bf16 - ref) / np.maximum(np.abs(ref), rms)).max() < 1e-2
+
+
+@pytest.mark.parametrize("shape,bits", [("qo", 4), ("kv", 4), ("gate_up", 3), ("gate_up", 4), ("gate_up", 5), ("down", 4)])
+def test_exl3_decode_rows_at_full_size(env, oracle, shape, bits):
+    torch, exl3, kern = env
+    k, n = SHAPES[shape]
+    layer = Layer(env, oracle, k, n, bits, 500 + bits)
+    single = None
+    for m in (1, 4, 8, 16):
+        xd, xh, got, got_bf16, ws = run_rows(env, layer, m, 9)
+        check(got, got_bf16, layer.reference(torch, xh, torch.float64), 1e-4)
+        if m == 16:  # each row of the batch has the bits of the single-row call
+            for r in (0, 7, 15):
+                y1 = torch.zeros((1, n), dtype=torch.float32, device="cuda")
+                layer.lin.forward(xd[r:r + 1], exl3.Dtype.Bf16, y1, exl3.Dtype.F32, 1, ws)
+                torch.cuda.synchronize()
+                assert np.array_equal(y1.cpu().numpy()[0].astype(np.float64), got[r])
+
+
+@pytest.mark.parametrize("shape", ["gate_up", "down"])
+def test_exl3_prefill_at_full_size(env, oracle, shape):
+    """M = 2048, 1 % outlier channels x20: the MFMA GEMM, including the tiles cut along K and the reduce kernel."""
+    torch, exl3, kern = env
+    k, n = SHAPES[shape]
+    layer = Layer(env, oracle, k, n, 4, 77)
+    xd, xh, got, got_bf16, ws = run_rows(env, layer, 2048, 11, outliers=True)
+    check(got, got_bf16, layer.reference(torch, xh, torch.float32), 1e-4)
+    again = run_rows(env, layer, 2048, 11, outliers=True)[2]
+    assert np.array_equal(again, got)  # deterministic
+
+
+@pytest.mark.parametrize("m", [1, 16, 2048])
+def test_nvfp4_at_full_size(env, oracle, m):
+    torch, exl3, kern = env
+    from ferrite_amd import fp4, synth
+    k, n = SHAPES["gate_up"]
+    fk = fp4.Kernels.load()
+    host = synth.fp4_linear(n, k, 20251, input_scale=1.0)
+    lin = host.upload()
+    ws = fp4.Workspace(m, k)
+    xd = dev_u16(torch, synth.activations(m, k, 5))
+    y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.forward(fk, ws, y, n, xd, k, m)
+    torch.cuda.synchronize()
+    codes, sf_tiled = ws.read(m, k)
+    sfa = oracle.untile_scales(sf_tiled, m, k // 16).reshape(m, k // 16)
+    # the quantizer at this size, bit for bit on sampled rows
+    xb = synth.activations(m, k, 5)
+    for r in sorted({0, m // 2, m - 1}):
+        wc, wsf = oracle.quant_fp4(xb[r:r + 1], lin.g)
+        assert np.array_equal(codes[r:r + 1], wc) and np.array_equal(sfa[r:r + 1], wsf)
+    a = torch.from_numpy(oracle.dequant_fp4(codes, sfa, 1.0)).cuda()
+    w = torch.from_numpy(oracle.dequant_fp4(host.codes, host.sf, 1.0)).cuda()
+    ref = ((a.double() if m <= 16 else a) @ (w.double().T if m <= 16 else w.T)).double().cpu().numpy() * host.alpha.astype(np.float64)
+    got = y.float().cpu().numpy().astype(np.float64)
+    scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+    assert (np.abs(got - ref) / scale).max() < 8e-3  # fp4-check.rs:134-144
+    assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
