@@ -89,6 +89,8 @@ SYMBOLS = {
     "fe_fp4_kernels_destroy": (I, [P]),
     "fe_fp4_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, P, F]),
     "fe_fp4_linear_from_view": (I, [PP, C.c_char_p, U32, U32, U64, U64, U64, F]),
+    "fe_fp8_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, F]),
+    "fe_fp8_linear_from_view": (I, [PP, C.c_char_p, U32, U32, U64, U64, F]),
     "fe_fp4_linear_destroy": (I, [P]),
     "fe_fp4_linear_shape": (I, [P, C.POINTER(U32), C.POINTER(U32), C.POINTER(F)]),
     "fe_fp4_workspace_create": (I, [PP, U32, U32]),
@@ -97,6 +99,7 @@ SYMBOLS = {
     "fe_fp4_linear_forward": (I, [P, P, P, P, U64, U32, U64, U32, U32, U64]),
     "fe_fp4_linear_quantize": (I, [P, P, P, P, U64, U32, U32]),
     "fe_fp4_linear_gemm": (I, [P, P, P, P, U64, U32, U32, U64]),
+    "fe_fp4_linear_forward_swiglu": (I, [P, P, P, P, P, U64, U32, U32, F]),
 }
 
 

@@ -21,6 +21,7 @@ constexpr uint32_t kTileN = 256;                        // GM_BN
 struct fe_fp4_kernels {
     fe_module_t module = nullptr;
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4 = nullptr;
+    fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     uint32_t cus = 0;
     uint32_t group_m = 8;  // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
 };
@@ -29,6 +30,7 @@ struct fe_fp4_linear {
     std::string name;
     uint32_t n = 0, k = 0;
     float g = 1.0f;
+    bool fp8 = false;  // Kind::Fp8 (e4m3 codes [n][k], no block scales), else Kind::Nvfp4 (lib.rs:229-233)
     FeBuf w, sw, alpha;
     // byte strides of the codes / scales of (128-row tile, 64-wide k tile, row in tile); see fe_gemm_nvfp4
     uint32_t w_snt = 0, w_skt = 0, w_sr = 0, s_snt = 0, s_skt = 0, s_sr = 0;
@@ -53,6 +55,12 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm4, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->reduce4, k->module, "fe_gemm_nvfp4_reduce");
     if (!c) c = fe_hip_module_get_function(&k->gemv4, k->module, "fe_gemv_nvfp4");
+    if (!c) c = fe_hip_module_get_function(&k->quant8, k->module, "fe_fp8_quant");
+    if (!c) c = fe_hip_module_get_function(&k->gemm8, k->module, "fe_gemm_fp8");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->swiglu4, k->module, "fe_gemm_nvfp4_swiglu");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->swiglu4, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->swiglu_reduce4, k->module, "fe_gemm_nvfp4_swiglu_reduce");
     int cus = 0;
     if (!c) c = fe_hip_cu_count(&cus);
     k->cus = (uint32_t)cus;
@@ -131,6 +139,47 @@ int fe_fp4_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, u
     return 0;
 }
 
+int fe_fp8_linear_upload(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, const uint8_t *codes,
+                         const float *alpha, float g) {
+    if (!out || !codes || !alpha) return fe_set_error(FE_ERR_ARG, "fe_fp8_linear_upload", "null argument");
+    FE_TRY(check_shape(name, n, k));
+    if (!(g > 0.0f)) return fe_set_error(FE_ERR_ARG, "fe_fp8_linear_upload", "input_scale 0");
+    auto *l = new fe_fp4_linear;
+    l->name = name ? name : "";
+    l->n = n, l->k = k, l->g = g, l->fp8 = true;
+    // k-tile-major like the NVFP4 codes: [n / 128][k / 64][128 rows][64 bytes]
+    const uint32_t kts = k / 64, nts = n / kTile;
+    std::vector<uint8_t> wt((size_t)n * k);
+    for (uint32_t nt = 0; nt < nts; nt++)
+        for (uint32_t r = 0; r < kTile; r++) {
+            const uint8_t *wrow = codes + (size_t)(nt * kTile + r) * k;
+            for (uint32_t kt = 0; kt < kts; kt++) memcpy(&wt[(((size_t)nt * kts + kt) * kTile + r) * 64], wrow + kt * 64, 64);
+        }
+    l->w_snt = kts * kTile * 64, l->w_skt = kTile * 64, l->w_sr = 64;
+    int c = l->w.from_host(wt.data(), wt.size());
+    if (!c) c = l->alpha.from_host(alpha, (size_t)n * 4);
+    if (c) {
+        delete l;
+        return c;
+    }
+    *out = l;
+    return 0;
+}
+
+int fe_fp8_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, fe_devptr_t codes,
+                            fe_devptr_t alpha, float g) {
+    if (!out || !codes || !alpha) return fe_set_error(FE_ERR_ARG, "fe_fp8_linear_from_view", "null argument");
+    FE_TRY(check_shape(name, n, k));
+    auto *l = new fe_fp4_linear;
+    l->name = name ? name : "";
+    l->n = n, l->k = k, l->g = g, l->fp8 = true;
+    l->w.view(codes, (size_t)n * k);
+    l->alpha.view(alpha, (size_t)n * 4);
+    l->w_snt = kTile * k, l->w_skt = 64, l->w_sr = k;
+    *out = l;
+    return 0;
+}
+
 int fe_fp4_linear_destroy(fe_fp4_linear *l) {
     delete l;
     return 0;
@@ -193,6 +242,10 @@ int fe_fp4_linear_quantize(const fe_fp4_linear *l, const fe_fp4_kernels *kern, f
     uint32_t k = l->k;
     float g = l->g;
     fe_devptr_t codes = ws->codes.p, sf = ws->sf.p, aq = ws->aq.p;
+    if (l->fp8) {
+        void *args8[] = {&codes, &aq, &x, &m, &k, &lda, &g};
+        return fe_hip_launch(kern->quant8, (m * (k / 8) + 255) / 256, 1, 1, 256, 1, 1, 0, s, args8);
+    }
     void *args[] = {&codes, &sf, &aq, &x, &m, &k, &lda, &g};
     const uint32_t blocks16 = m * (k / 16);
     return fe_hip_launch(kern->quant4, (blocks16 + 255) / 256, 1, 1, 256, 1, 1, 0, s, args);
@@ -207,7 +260,7 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     if (!y || ldy % 8 || y % 16 || (res && res % 16) || ldy < l->n)
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
-    if (m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
+    if (!l->fp8 && m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
         // decode-sized: the weight-read-bound GEMV, 16 rows a pass. Two programs fit a CU: as many programs as run at
         // once, not more (a second round of short programs costs more than idle CUs in the first).
         const uint32_t nts = n / kTile, kts = k / 64;
@@ -227,7 +280,7 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         }
         return 0;
     }
-    if ((uint64_t)m * k * 2 >= (1ull << 32) || (uint64_t)n * k / 2 >= (1ull << 32))
+    if ((uint64_t)m * k * 2 >= (1ull << 32) || (uint64_t)n * k >= (1ull << 32))
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_fp4_linear_gemm", "operand of 4 GB or more");
     const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
     uint32_t group = kern->group_m == 0 || kern->group_m > tiles_m ? tiles_m : kern->group_m;  // lib.rs:148-151
@@ -236,11 +289,17 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = ws->part.p;
-    void *args[] = {&y,     &aq,    &w,    &sw,    &alpha, &res,  &m,      &n,   &k, &ldy,
-                    &group, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr, &full, &splits, &part};
-    FE_TRY(fe_hip_launch(kern->gemm4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    float scale = l->fp8 ? 1.0f : 0.0625f;  // what the fp16 expansions of the two operands carry (FP4_OPERAND_SCALE)
+    if (l->fp8) {
+        void *args8[] = {&y, &aq, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &full, &splits, &part};
+        FE_TRY(fe_hip_launch(kern->gemm8, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args8));
+    } else {
+        void *args[] = {&y,     &aq,    &w,    &sw,    &alpha, &res,  &m,      &n,   &k, &ldy,
+                        &group, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr, &full, &splits, &part};
+        FE_TRY(fe_hip_launch(kern->gemm4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    }
     if (!gs.cut()) return 0;
-    void *rargs[] = {&y, &part, &alpha, &res, &m, &n, &ldy, &group, &full, &splits};
+    void *rargs[] = {&y, &part, &alpha, &res, &m, &n, &ldy, &group, &full, &splits, &scale};
     return fe_hip_launch(kern->reduce4, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
@@ -248,6 +307,38 @@ int fe_fp4_linear_forward(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe
                           fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda, uint32_t m, fe_devptr_t res) {
     FE_TRY(fe_fp4_linear_quantize(l, kern, s, ws, x, lda, m));
     return fe_fp4_linear_gemm(l, kern, s, ws, y, ldy, m, res);
+}
+
+int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s,
+                                 const fe_fp4_workspace *ws, const fe_fp4_workspace *act, fe_devptr_t x, uint32_t lda,
+                                 uint32_t m, float down_g) {
+    if (!l || !kern || !ws || !act) return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_forward_swiglu", "null argument");
+    if (l->fp8 || l->n % 256) {  // lib.rs:388-392, 500
+        char msg[200];
+        snprintf(msg, sizeof msg, "%s: not an NVFP4 gate|up pair (n %u)", l->name.c_str(), l->n);
+        return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_forward_swiglu", msg);
+    }
+    if (m == 0) return 0;
+    uint32_t n = l->n, k = l->k, inter = n / 2;
+    if (m > act->max_rows || inter > act->max_k)
+        return fe_set_error(FE_ERR_WORKSPACE, "fe_fp4_linear_forward_swiglu", "rows or n / 2 exceed the act workspace");
+    if (!(down_g > 0.0f)) return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_forward_swiglu", "down_g");
+    FE_TRY(fe_fp4_linear_quantize(l, kern, s, ws, x, lda, m));
+    if ((uint64_t)m * k * 2 >= (1ull << 32) || (uint64_t)n * k / 2 >= (1ull << 32))
+        return fe_set_error(FE_ERR_UNSUPPORTED, "fe_fp4_linear_forward_swiglu", "operand of 4 GB or more");
+    const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
+    uint32_t group = kern->group_m == 0 || kern->group_m > tiles_m ? tiles_m : kern->group_m;
+    fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p, part = ws->part.p;
+    fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
+    uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    uint32_t full = gs.full, splits = gs.splits;
+    void *args[] = {&aq,    &w,     &sw,   &alpha, &m,    &n,      &k,    &group,   &w_snt, &w_skt, &w_sr,
+                    &s_snt, &s_skt, &s_sr, &full,  &splits, &part, &q_codes, &q_sf, &q_aq,  &down_g};
+    FE_TRY(fe_hip_launch(kern->swiglu4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (!gs.cut()) return 0;
+    void *rargs[] = {&part, &alpha, &m, &n, &group, &full, &splits, &q_codes, &q_sf, &q_aq, &down_g};
+    return fe_hip_launch(kern->swiglu_reduce4, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 }  // extern "C"

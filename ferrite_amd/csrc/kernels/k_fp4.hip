@@ -193,32 +193,164 @@ __device__ __forceinline__ void fp4_store4(uint16_t* c, const uint16_t* res, siz
     *(u32x2*)(c + at) = o;
 }
 
-// C[M][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res: bf16(bf16(.) + res)); A_q as the fp16 operand of fe_fp4_quant. The
-// codes of row r = 128 nt + i, k tile kt are 32 bytes at w + nt * w_snt + kt * w_skt + i * w_sr, its 4 scales at
-// sw + nt * s_snt + kt * s_skt + i * s_sr. grid full_tiles + (tiles - full_tiles) * splits with tiles =
-// ceil(M / 256) * ceil(N / 256) (grouped raster), 256 threads, dynamic LDS GM_LDS_TILES. Tiles past full_tiles leave
-// partials in `part` for fe_gemm_nvfp4_reduce. N % 128 == 0, K % 128 == 0. (kernels/k-fp4/src/lib.rs:285-470)
-extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
-                                                                   const uint8_t* sw, const float* alpha, const uint16_t* res,
-                                                                   uint32_t m, uint32_t n, uint32_t k, uint32_t ldc,
-                                                                   uint32_t group_m, uint32_t w_snt, uint32_t w_skt,
-                                                                   uint32_t w_sr, uint32_t s_snt, uint32_t s_skt,
-                                                                   uint32_t s_sr, uint32_t full_tiles, uint32_t splits,
-                                                                   float* part) {
+// ---- FP8 (e4m3, one scale per tensor) -------------------------------------------------------------------------------------
+
+// The two e4m3 codes of the low (HI = 0) or high half of w as packed fp16, exact (hardware conversion, scale 1).
+__device__ __forceinline__ uint32_t e4m3x2_to_f16(uint32_t w, int hi) {
+    f16x2 v = hi ? __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true) : __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// f32 -> e4m3 code of either sign, round to nearest even, saturating; NaN -> 0x7f. (crates/fe-fp4/src/format.rs:57-63)
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+    if (x != x) return 0x7f;
+    return f32_to_e4m3_pos(__builtin_fabsf(x)) | ((__float_as_uint(x) >> 24) & 0x80u);
+}
+
+// bf16 x[M][ldx] -> e4m3 codes [M][K], q = e4m3(x * g), and the fp16 operand the GEMM reads (an e4m3 value is an exact
+// fp16 number). One thread per 8 elements: grid ceil(M * K / 8 / 256), 256 threads. K % 8 == 0.
+// (kernels/k-fp4/src/lib.rs:199-214)
+extern "C" __global__ __launch_bounds__(256) void fe_fp8_quant(uint8_t* codes, _Float16* aq, const uint16_t* x, uint32_t m,
+                                                               uint32_t k, uint32_t ldx, float g) {
+    uint32_t i = blockIdx.x * 256 + threadIdx.x, k8 = k >> 3;
+    if (i >= m * k8) return;
+    uint32_t row = i / k8, c = (i - row * k8) * 8;
+    u32x4 r = *(const u32x4*)(x + (size_t)row * ldx + c);
+    uint32_t q[2] = {0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        uint32_t lo = f32_to_e4m3(__uint_as_float(r[j] << 16) * g), hi = f32_to_e4m3(__uint_as_float(r[j] & 0xffff0000u) * g);
+        q[j >> 1] |= (lo | (hi << 8)) << (16 * (j & 1));
+    }
+    *(u32x2*)(codes + (size_t)row * k + c) = (u32x2){q[0], q[1]};
+    u32x4 o;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+        o[j] = e4m3x2_to_f16(q[j >> 1], j & 1);
+    *(u32x4*)(aq + (size_t)row * k + c) = o;
+}
+
+// Weight tile producer for e4m3 weights: thread t expands the 64 codes (64 bytes) of row t of the 256-row weight tile
+// with the hardware conversion (exact). Addressing as Fp4Producer, 64 bytes a row and k tile.
+struct Fp8Producer {
+    const uint8_t* w;
+    uint32_t w_skt, row;
+    struct Raw {
+        u32x4 c[4];
+    };
+    static constexpr int kStoreValu = 40;
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
+        const uint8_t* p = w + (size_t)kt * w_skt + 32 * half;
+        r.c[2 * half] = *(const u32x4*)p;
+        r.c[2 * half + 1] = *(const u32x4*)(p + 16);
+    }
+    // part 0: chunks 0..3 of the row (bytes 0..31), part 1: 4..7
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
+#pragma unroll
+        for (int d = 0; d < 8; d++) {
+            if (d / 4 != part) continue;
+            u32x4 o;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                o[e] = e4m3x2_to_f16(r.c[d >> 1][2 * (d & 1) + (e >> 1)], e & 1);
+            *(u32x4*)(Bs + gm_swz(row, d)) = o;
+        }
+    }
+};
+
+// ---- fused gate|up epilogue: SwiGLU and NVFP4 re-quantization ---------------------------------------------------------------
+
+// act = bf16(bf16(silu(g)) * u), g and u the bf16 GEMM outputs (kernels/k-fp4/src/lib.rs:669-673).
+__device__ __forceinline__ float swiglu(float g, float u) {
+    float s = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g));
+    s = bf16_bits_to_f32(f32_to_bf16_bits(s));
+    return bf16_bits_to_f32(f32_to_bf16_bits(s * u));
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_mov_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xf, 0xf, true);
+}
+
+// The weight rows of a fused gate|up linear are interleaved in blocks of 8 (gate f..f+7, up f..f+7, ...,
+// crates/fe-fp4/src/lib.rs:386-417), so a group of 32 output columns holds 16 features: of the 8 lanes that hold it
+// (4 columns each) lanes 0, 1 have gate f0..7, lanes 2, 3 up f0..7, lanes 4, 5 gate f8..15, lanes 6, 7 up f8..15. Takes
+// the 4 sums of a lane (v, already times alpha's lane values `al`), forms act = SwiGLU(bf16 gate, bf16 up) on the gate
+// lanes, quantizes each 16-feature block to NVFP4 with global scale qg exactly as fe_fp4_quant would quantize the bf16
+// act (block scale from the block's amax, codes, tiled scale, fp16 operand), and stores for rows that exist. Every lane
+// of the half wavefront must call it. col: the lane's first interleaved column; n: interleaved width (2 * inter).
+// (kernels/k-fp4/src/lib.rs:675-745)
+__device__ __forceinline__ void swiglu_quant_store(const float (&v)[4], f32x4 al, uint32_t l32, bool live, uint32_t row,
+                                                   uint32_t col, uint32_t n, uint8_t* q_codes, uint8_t* q_sf, _Float16* q_aq,
+                                                   float qg) {
+    const uint32_t j = l32 & 7;
+    const bool gate = (j & 2) == 0;
+    float act[4], amax = 0.f;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float y = bf16_bits_to_f32(f32_to_bf16_bits(v[e] * al[e]));
+        float u = dpp_mov<DPP_QUAD_XOR2>(y);  // the up value of the same feature, two lanes on
+        act[e] = swiglu(y, u);
+        if (gate) amax = __builtin_fmaxf(amax, __builtin_fabsf(act[e]));
+    }
+    amax = __builtin_fmaxf(amax, dpp_mov<DPP_QUAD_XOR1>(amax));
+    amax = __builtin_fmaxf(amax, dpp_mov<DPP_QUAD_XOR2>(amax));
+    amax = __builtin_fmaxf(amax, dpp_mov<DPP_QUAD_XOR3>(dpp_mov<DPP_HALF_MIRROR>(amax)));  // lane ^ 4
+    const uint32_t s8 = f32_to_e4m3_pos(amax * (1.0f / 6.0f) * qg);
+    const float sv = e4m3_to_f32(s8);
+    const float mul = sv > 0.f ? qg / sv : 0.f;
+    uint32_t q = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) q |= f32_to_e2m1(act[e] * mul) << (4 * e);
+    const uint32_t word = q | (dpp_mov_u32<DPP_QUAD_XOR1>(q) << 16);  // 8 codes: this lane's 4 features and the next lane's
+    if (!live || !gate) return;
+    const uint32_t inter = n >> 1, kb = inter >> 4, blk = col >> 5;
+    const uint32_t feat = blk * 16 + (j >> 2) * 8 + (j & 1) * 4;  // the lane's first feature
+    uint32_t t[4];
+    e2m1x8_to_f16(q, t);
+    const f16x2 sc = e4m3_to_f16x2(s8);
+    u32x2 o = {__builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[0]) * sc)),
+               __builtin_bit_cast(uint32_t, (f16x2)(__builtin_bit_cast(f16x2, t[1]) * sc))};
+    *(u32x2*)(q_aq + (size_t)row * inter + feat) = o;
+    if ((j & 1) == 0) *(uint32_t*)(q_codes + (size_t)row * (inter >> 1) + (feat >> 1)) = word;
+    if (j == 0) q_sf[sf_tiled(row, blk, kb)] = (uint8_t)s8;
+}
+
+// ---- GEMM kernels ------------------------------------------------------------------------------------------------------------
+
+// Where the output of a GEMM goes: C (bf16, + residual) or, for a fused gate|up linear, the NVFP4-quantized SwiGLU.
+struct FpOut {
+    uint16_t* c;
+    const uint16_t* res;
+    uint32_t ldc;
+    uint8_t* q_codes;
+    uint8_t* q_sf;
+    _Float16* q_aq;
+    float qg;
+};
+
+// One row piece: 4 sums of columns col.. of row grow. SWIGLU: every lane of the half wavefront takes part.
+template <bool SWIGLU>
+__device__ __forceinline__ void fp_store_piece(const FpOut& o, const float (&v)[4], f32x4 al, uint32_t l32, uint32_t grow,
+                                               uint32_t m, uint32_t col, uint32_t n) {
+    if constexpr (SWIGLU) {
+        swiglu_quant_store(v, al, l32, grow < m, grow < m ? grow : 0, col, n, o.q_codes, o.q_sf, o.q_aq, o.qg);
+    } else {
+        if (grow < m) fp4_store4(o.c, o.res, (size_t)grow * o.ldc + col, v, al);
+    }
+}
+
+// C[M][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res: bf16(bf16(.) + res)); A_q = the fp16 operand of the quantizer,
+// W_q expanded by the producer; `scale` = 1 / (the factors the two fp16 expansions carry). grid full_tiles +
+// (tiles - full_tiles) * splits with tiles = ceil(M / 256) * ceil(N / 256) (grouped raster), 256 threads, dynamic LDS
+// GM_LDS_TILES. Tiles past full_tiles leave partials in `part` for the reduce kernel. N % 128 == 0, K % 128 == 0.
+// (kernels/k-fp4/src/lib.rs:285-470)
+template <class Producer, bool SWIGLU>
+__device__ __forceinline__ void fp_gemm_body(Producer& prod, const FpOut& out, const _Float16* aq, const float* alpha,
+                                             float scale, uint32_t m, uint32_t n, uint32_t k, const GemmWork& wk, float* part) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    const uint32_t nts = n / 128;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
     const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
     const uint32_t tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    Fp4Producer prod;
-    {
-        uint32_t nt = 2 * wk.tn + (tid >> 7);
-        nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program expands its first tile twice
-        prod.row = tid;
-        prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
-        prod.sw = sw + (size_t)nt * s_snt + (size_t)(tid & 127) * s_sr;
-        prod.w_skt = w_skt, prod.s_skt = s_skt;
-    }
     f32x16 acc[4][4];
     gemm_mainloop(aq, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
     if (wk.partial) {
@@ -228,27 +360,104 @@ extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, 
     const uint32_t colb = n0 + wn * 128;
     if (colb >= n) return;
     const uint32_t col = colb + 4 * (tid & 31);
-    f32x4 al = *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE;
+    const f32x4 al = *(const f32x4*)(alpha + col) * scale;
     gemm_epilogue(
         acc, lds, [](float (&)[4][4], uint32_t) {},
-        [&](uint32_t row, uint32_t, float (&v)[4]) {
-            uint32_t grow = m0 + wm * 128 + row;
-            if (grow < m) fp4_store4(c, res, (size_t)grow * ldc + col, v, al);
-        });
+        [&](uint32_t row, uint32_t l32, float (&v)[4]) { fp_store_piece<SWIGLU>(out, v, al, l32, m0 + wm * 128 + row, m, col, n); });
 }
 
-// Finishes the tiles that fe_gemm_nvfp4 cut along K. grid (tiles - full_tiles) * 64, 256 threads.
-extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t* c, const float* part, const float* alpha,
-                                                                       const uint16_t* res, uint32_t m, uint32_t n,
-                                                                       uint32_t ldc, uint32_t group_m, uint32_t full_tiles,
-                                                                       uint32_t splits) {
+// Finishes the tiles that a GEMM kernel cut along K. grid (tiles - full_tiles) * 64, 256 threads.
+template <bool SWIGLU>
+__device__ __forceinline__ void fp_reduce_body(const FpOut& out, const float* part, const float* alpha, float scale,
+                                               uint32_t m, uint32_t n, uint32_t group_m, uint32_t full_tiles,
+                                               uint32_t splits) {
     const uint32_t nts = n / 128;
     gemm_reduce_rows(part, splits, [&](uint32_t t, uint32_t row, uint32_t cb, uint32_t l32, float (&v)[4]) {
         uint32_t tm, tn;
         gemm_raster(full_tiles + t, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, tm, tn);
         uint32_t grow = tm * GM_BM + row, col = tn * GM_BN + cb * 128 + 4 * l32;
-        if (grow < m && col < n) fp4_store4(c, res, (size_t)grow * ldc + col, v, *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE);
+        if (tn * GM_BN + cb * 128 >= n) return;  // the absent half of an odd last tile (uniform over the half wavefront)
+        fp_store_piece<SWIGLU>(out, v, *(const f32x4*)(alpha + col) * scale, l32, grow, m, col, n);
     });
+}
+
+__device__ __forceinline__ Fp4Producer fp4_producer(const uint8_t* w, const uint8_t* sw, uint32_t tn, uint32_t nts,
+                                                    uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt,
+                                                    uint32_t s_skt, uint32_t s_sr) {
+    const uint32_t tid = threadIdx.x;
+    uint32_t nt = 2 * tn + (tid >> 7);
+    nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program expands its first tile twice
+    Fp4Producer prod;
+    prod.row = tid;
+    prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
+    prod.sw = sw + (size_t)nt * s_snt + (size_t)(tid & 127) * s_sr;
+    prod.w_skt = w_skt, prod.s_skt = s_skt;
+    return prod;
+}
+
+// NVFP4: the codes of row r = 128 nt + i, k tile kt are 32 bytes at w + nt * w_snt + kt * w_skt + i * w_sr, its 4 scales
+// at sw + nt * s_snt + kt * s_skt + i * s_sr.
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
+                                                                   const uint8_t* sw, const float* alpha, const uint16_t* res,
+                                                                   uint32_t m, uint32_t n, uint32_t k, uint32_t ldc,
+                                                                   uint32_t group_m, uint32_t w_snt, uint32_t w_skt,
+                                                                   uint32_t w_sr, uint32_t s_snt, uint32_t s_skt,
+                                                                   uint32_t s_sr, uint32_t full_tiles, uint32_t splits,
+                                                                   float* part) {
+    const uint32_t nts = n / 128;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
+    Fp4Producer prod = fp4_producer(w, sw, wk.tn, nts, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
+    FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
+    fp_gemm_body<Fp4Producer, false>(prod, out, aq, alpha, FP4_OPERAND_SCALE, m, n, k, wk, part);
+}
+
+extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t* c, const float* part, const float* alpha,
+                                                                       const uint16_t* res, uint32_t m, uint32_t n,
+                                                                       uint32_t ldc, uint32_t group_m, uint32_t full_tiles,
+                                                                       uint32_t splits, float scale) {
+    FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
+    fp_reduce_body<false>(out, part, alpha, scale, m, n, group_m, full_tiles, splits);
+}
+
+// Fused MLP front: act = SwiGLU(x . [gate|up]^T), NVFP4-quantized with global scale qg (1 / input_scale of the down
+// projection) into q_codes [M][inter/2], q_sf (tiled, kb = inter/16) and the fp16 operand q_aq [M][inter]; w, sw, alpha =
+// gate and up interleaved in blocks of 8 rows, N = 2 inter, N % 256 == 0. (kernels/k-fp4/src/lib.rs:747-752)
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_swiglu(
+    const _Float16* aq, const uint8_t* w, const uint8_t* sw, const float* alpha, uint32_t m, uint32_t n, uint32_t k,
+    uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt, uint32_t s_sr,
+    uint32_t full_tiles, uint32_t splits, float* part, uint8_t* q_codes, uint8_t* q_sf, _Float16* q_aq, float qg) {
+    const uint32_t nts = n / 128;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
+    Fp4Producer prod = fp4_producer(w, sw, wk.tn, nts, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
+    FpOut out = {nullptr, nullptr, 0, q_codes, q_sf, q_aq, qg};
+    fp_gemm_body<Fp4Producer, true>(prod, out, aq, alpha, FP4_OPERAND_SCALE, m, n, k, wk, part);
+}
+
+extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_swiglu_reduce(const float* part, const float* alpha, uint32_t m,
+                                                                              uint32_t n, uint32_t group_m, uint32_t full_tiles,
+                                                                              uint32_t splits, uint8_t* q_codes, uint8_t* q_sf,
+                                                                              _Float16* q_aq, float qg) {
+    FpOut out = {nullptr, nullptr, 0, q_codes, q_sf, q_aq, qg};
+    fp_reduce_body<true>(out, part, alpha, FP4_OPERAND_SCALE, m, n, group_m, full_tiles, splits);
+}
+
+// FP8: the 64 codes of row r = 128 nt + i, k tile kt are at w + nt * w_snt + kt * w_skt + i * w_sr; both fp16 expansions
+// are the values themselves. Finished by fe_gemm_nvfp4_reduce with scale 1. (kernels/k-fp4/src/lib.rs:472-484)
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8(uint16_t* c, const _Float16* aq, const uint8_t* w,
+                                                                 const float* alpha, const uint16_t* res, uint32_t m, uint32_t n,
+                                                                 uint32_t k, uint32_t ldc, uint32_t group_m, uint32_t w_snt,
+                                                                 uint32_t w_skt, uint32_t w_sr, uint32_t full_tiles,
+                                                                 uint32_t splits, float* part) {
+    const uint32_t nts = n / 128, tid = threadIdx.x;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
+    uint32_t nt = 2 * wk.tn + (tid >> 7);
+    nt = nt < nts ? nt : nts - 1;
+    Fp8Producer prod;
+    prod.row = tid;
+    prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
+    prod.w_skt = w_skt;
+    FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
+    fp_gemm_body<Fp8Producer, false>(prod, out, aq, alpha, 1.0f, m, n, k, wk, part);
 }
 
 // ---- GEMV (1..16 rows) -------------------------------------------------------------------------------------------------

@@ -40,6 +40,7 @@ class HostLinear:
     alpha: np.ndarray
     g: float
     swiglu: bool = False
+    kind: str = "nvfp4"  # or "fp8": e4m3 codes [n][k], no block scales (Kind, lib.rs:229-233)
 
     @staticmethod
     def fuse(parts):
@@ -73,9 +74,37 @@ class HostLinear:
                           np.ascontiguousarray(np.concatenate([s for _, _, s, _, _ in parts]), dtype=np.uint8), alpha,
                           float(np.float32(1.0) / in_scale))
 
+    @staticmethod
+    def fuse_fp8(parts):
+        """The same for FP8 parts: (name, codes [n][k] e4m3, weight_scale, input_scale)."""
+        if not parts:
+            raise ValueError("no parts")
+        k = parts[0][1].shape[1]
+        ps, n = [], 0
+        for name, codes, wscale, in_scale in parts:
+            pn, pk = codes.shape
+            if pk != k:
+                raise ValueError(f"{name}: k {pk} != {k}")
+            if pn % TILE or n % TILE:
+                raise ValueError(f"{name}: n {pn} not a multiple of {TILE}")
+            ps.append(Part(name, n, pn, float(wscale), float(in_scale)))
+            n += pn
+        if k % 128:
+            raise ValueError(f"{parts[0][0]}: k {k} not a multiple of 128")
+        in_scale = max(np.float32(p.input_scale) for p in ps)
+        if not in_scale > 0:
+            raise ValueError(f"{parts[0][0]}: input_scale 0")
+        alpha = np.empty(n, np.float32)
+        for p in ps:
+            p.alpha = float(np.float32(p.alpha) * in_scale)
+            alpha[p.n0:p.n0 + p.n] = p.alpha
+        return HostLinear(n, k, "+".join(p.name for p in ps), ps,
+                          np.ascontiguousarray(np.concatenate([c for _, c, _, _ in parts]), dtype=np.uint8),
+                          np.zeros((0,), np.uint8), alpha, float(np.float32(1.0) / in_scale), False, "fp8")
+
     def into_swiglu(self):
         """gate|up rows interleaved in blocks of 8 (lib.rs:386-417)."""
-        if len(self.parts) != 2 or self.parts[0].n != self.parts[1].n:
+        if self.kind != "nvfp4" or len(self.parts) != 2 or self.parts[0].n != self.parts[1].n:
             raise ValueError(f"{self.name}: not an NVFP4 gate|up pair")
         if self.n % 256:
             raise ValueError(f"{self.name}: n {self.n}")
@@ -120,6 +149,12 @@ class Workspace:
         check(_lib.lib().fe_fp4_workspace_buffers(self.h, C.byref(c), C.byref(s), None, None))
         self.codes_ptr, self.sf_ptr = c.value, s.value
 
+    def read_fp8(self, m, k):
+        """e4m3 codes [m][k] as a host array."""
+        codes = np.empty((m, k), np.uint8)
+        check(_lib.lib().fe_hip_memcpy_dtoh(codes.ctypes.data_as(C.c_void_p), self.codes_ptr, codes.size))
+        return codes
+
     def read(self, m, k):
         """(codes [m][k/2], tiled scale bytes of ceil(m/128)*128 rows) as host arrays."""
         codes = np.empty((m, k // 2), np.uint8)
@@ -141,8 +176,14 @@ class PromptLinear:
     def __init__(self, host: HostLinear):
         _lib.init()
         self.n, self.k, self.name, self.parts, self.g, self.swiglu = host.n, host.k, host.name, host.parts, host.g, host.swiglu
+        self.kind = host.kind
         self.h = C.c_void_p()
         alpha = np.ascontiguousarray(host.alpha, dtype=np.float32)
+        if host.kind == "fp8":
+            check(_lib.lib().fe_fp8_linear_upload(C.byref(self.h), host.name.encode(), host.n, host.k,
+                                                  host.codes.ctypes.data_as(C.c_void_p), alpha.ctypes.data_as(C.c_void_p),
+                                                  host.g))
+            return
         check(_lib.lib().fe_fp4_linear_upload(C.byref(self.h), host.name.encode(), host.n, host.k,
                                               host.codes.ctypes.data_as(C.c_void_p), host.sf.ctypes.data_as(C.c_void_p),
                                               alpha.ctypes.data_as(C.c_void_p), host.g))
@@ -156,6 +197,11 @@ class PromptLinear:
         self.n, self.k, self.name, self.parts, self.g, self.swiglu = n, k, name, [], g, False
         self._keep = (codes, scales, alpha)
         self.h = C.c_void_p()
+        if scales is None:  # FP8: e4m3 codes [n][k]
+            self.kind = "fp8"
+            check(_lib.lib().fe_fp8_linear_from_view(C.byref(self.h), name.encode(), n, k, codes.data_ptr(), alpha.data_ptr(), g))
+            return self
+        self.kind = "nvfp4"
         check(_lib.lib().fe_fp4_linear_from_view(C.byref(self.h), name.encode(), n, k, codes.data_ptr(), scales.data_ptr(),
                                                  alpha.data_ptr(), g))
         return self
@@ -168,6 +214,12 @@ class PromptLinear:
     def forward(self, kern, ws, y, ldy, x, lda, m, res=None, stream=None):
         check(_lib.lib().fe_fp4_linear_forward(self.h, kern.h, _stream(stream), ws.h, y.data_ptr(), ldy, x.data_ptr(), lda, m,
                                                res.data_ptr() if res is not None else 0))
+
+    def forward_swiglu(self, kern, ws, act, x, lda, m, down_g, stream=None):
+        """act = SwiGLU(x . [gate|up]^T), NVFP4-quantized with down_g into the workspace `act` (lib.rs:496-508); then
+        down.gemm(kern, act, y, ldy, m, res) finishes the MLP."""
+        check(_lib.lib().fe_fp4_linear_forward_swiglu(self.h, kern.h, _stream(stream), ws.h, act.h, x.data_ptr(), lda, m,
+                                                      down_g))
 
     def quantize(self, kern, ws, x, lda, m, stream=None):
         check(_lib.lib().fe_fp4_linear_quantize(self.h, kern.h, _stream(stream), ws.h, x.data_ptr(), lda, m))

@@ -56,3 +56,11 @@ def fp4_linear(n: int, k: int, seed: int, input_scale: float = 1.0, name: str = 
     codes = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
     s = np.clip(np.abs(rng.normal(size=(n, k // 16))).astype(np.float32) * np.float32(0.1), 2.0 ** -9, 448.0)
     return HostLinear.fuse([(name, codes, e4m3_from_f32(s), 1.0, input_scale)])
+
+
+def fp8_linear(n: int, k: int, seed: int, input_scale: float = 1.0, weight_scale: float = 1.0, name: str = "synthetic") -> HostLinear:
+    """e4m3 codes of N(0, 1) weights scaled into the format's range, one weight scale for the tensor."""
+    rng = np.random.default_rng([seed, n, k, 8])
+    w = rng.normal(size=(n, k)).astype(np.float32) * np.float32(32.0)
+    codes = e4m3_from_f32(np.abs(w)) | (np.signbit(w).astype(np.uint8) << 7)
+    return HostLinear.fuse_fp8([(name, codes.astype(np.uint8), weight_scale, input_scale)])

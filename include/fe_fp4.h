@@ -1,5 +1,6 @@
 /*
- * fe_fp4: the NVFP4 prompt linear (e2m1 codes, e4m3 scale per 16 along K, fp32 scale per output column) over fe_hip.
+ * fe_fp4: the NVFP4 prompt linear (e2m1 codes, e4m3 scale per 16 along K, fp32 scale per output column) over fe_hip,
+ * with the FP8 (e4m3, per-tensor scale) linears and the fused gate|up SwiGLU front of the same layer API.
  *
  * C ABI of the reference's fe-fp4 layer API for its NVFP4 path (crates/fe-fp4/src/lib.rs): HostLinear-style inputs
  * (codes [n][k/2], row-major scales [n][k/16], alpha[n], g), PromptLinear::{forward, quantize, gemm}, Workspace.
@@ -31,6 +32,12 @@ int fe_fp4_linear_upload(fe_fp4_linear **out, const char *name, uint32_t n, uint
 /* A linear over device buffers the caller owns (the reference's streamed form, PromptLinear::set_views lib.rs:485-494). */
 int fe_fp4_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, fe_devptr_t codes,
                             fe_devptr_t scales, fe_devptr_t alpha, float g);
+/* The same for an FP8 linear (Kind::Fp8, lib.rs:229-233, 305-384): e4m3 codes [n][k], no block scales,
+ * alpha[n] = max(input_scale) * weight_scale. forward / quantize / gemm below take either kind. */
+int fe_fp8_linear_upload(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, const uint8_t *codes,
+                         const float *alpha, float g);
+int fe_fp8_linear_from_view(fe_fp4_linear **out, const char *name, uint32_t n, uint32_t k, fe_devptr_t codes,
+                            fe_devptr_t alpha, float g);
 int fe_fp4_linear_destroy(fe_fp4_linear *l);
 int fe_fp4_linear_shape(const fe_fp4_linear *l, uint32_t *n, uint32_t *k, float *g);
 
@@ -51,6 +58,15 @@ int fe_fp4_linear_quantize(const fe_fp4_linear *l, const fe_fp4_kernels *kern, f
 /* PromptLinear::gemm (lib.rs:532-543) over activations already quantized into ws by a linear with the same k and g. */
 int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
                        fe_devptr_t y, uint32_t ldy, uint32_t m, fe_devptr_t res);
+
+/* PromptLinear::forward_swiglu (lib.rs:496-508): the fused MLP front for prompt rows. l = gate and up fused with their
+ * rows interleaved in blocks of 8 (HostLinear::into_swiglu, lib.rs:386-417), n = 2 * inter, n % 256 == 0. Quantizes x
+ * into ws, then act = SwiGLU(x . [gate|up]^T) is written NVFP4-quantized with global scale down_g (the down
+ * projection's g) into the workspace `act` (rows <= act.max_rows, inter <= act.max_k), ready for
+ * fe_fp4_linear_gemm(down, kern, s, act, y, ldy, m, res). */
+int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s,
+                                 const fe_fp4_workspace *ws, const fe_fp4_workspace *act, fe_devptr_t x, uint32_t lda,
+                                 uint32_t m, float down_g);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,138 @@
+"""GPU parity of the two neighbours of the NVFP4 GEMM in the prompt path: the FP8 (e4m3, per-tensor scale) linear
+(crates/fe-fp4/src/bin/fp4-check.rs runs the same checks for it) and the fused gate|up front whose epilogue applies SwiGLU
+and re-quantizes to NVFP4 for the down projection (PromptLinear::forward_swiglu, crates/fe-fp4/src/lib.rs:496-508)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    from ferrite_amd import fp4
+    assert torch.cuda.is_available()
+    return torch, fp4, fp4.Kernels.load()
+
+
+def dev_u16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def bf16_to_f32(a):
+    return (a.astype(np.uint32) << 16).view(np.float32)
+
+
+def bf16_bits(x):
+    b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+@pytest.mark.parametrize("n,k,m,input_scale", [(256, 512, 200, 0.05), (128, 1024, 1, 0.02), (640, 256, 300, 0.1)])
+def test_fp8_linear(env, oracle, n, k, m, input_scale):
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    host = synth.fp8_linear(n, k, 17, input_scale=input_scale, weight_scale=0.003)
+    host.alpha[:] = host.alpha * np.linspace(0.5, 2.0, n).astype(np.float32)
+    lin = host.upload()
+    ws = fp4.Workspace(m, k)
+    rng = np.random.default_rng(m)
+    x = rng.normal(size=(m, k)).astype(np.float32) * np.float32(input_scale * 100.0)
+    x[0, :8] = [0.0, -0.0, 1e9, -1e9, np.float32(input_scale * 448.0), 1e-12, -1e-12, 3.0]  # zeros, saturation, underflow
+    xb = bf16_bits(x)
+    xd = dev_u16(torch, xb)
+    y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.forward(kern, ws, y, n, xd, k, m)
+    torch.cuda.synchronize()
+    yg = y.view(torch.int16).cpu().numpy().view(np.uint16)
+
+    # quantizer: q = e4m3(x * g), bit-exact (crates/fe-fp4/src/format.rs:93-95)
+    codes = ws.read_fp8(m, k)
+    want = np.stack([oracle.quant_fp8_row(xb[r], lin.g) for r in range(m)])
+    assert np.array_equal(codes, want)
+    assert codes[0, 2] == 0x7E and codes[0, 3] == 0xFE  # satfinite
+
+    # GEMM vs f64 over the same quantized operands, times alpha
+    rows = sorted({r for r in (0, 1, 17, 127, 128, m // 2, m - 1) if r < m})
+    a = np.stack([oracle.dequant_fp8_row(codes[r], 1.0) for r in rows])
+    w = np.stack([oracle.dequant_fp8_row(host.codes[c], 1.0) for c in range(n)])
+    ref = oracle.ref_gemm(a, w).astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+    got = bf16_to_f32(yg[rows]).astype(np.float64)
+    scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+    assert (np.abs(got - ref) / scale).max() < 8e-3
+    assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
+
+    # residual epilogue, in place, exact; untouched rows; a row-major device view gives the same bits
+    res = bf16_bits(rng.normal(size=(m + 1, n)).astype(np.float32))
+    y2 = dev_u16(torch, res)
+    lin.forward(kern, ws, y2, n, xd, k, m, res=y2)
+    view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), None,
+                                      torch.from_numpy(host.alpha).cuda(), host.g)
+    y3 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    view.forward(kern, ws, y3, n, xd, k, m)
+    torch.cuda.synchronize()
+    out2 = y2.cpu().numpy().view(np.uint16)
+    assert np.array_equal(out2[:m], bf16_bits(bf16_to_f32(yg) + bf16_to_f32(res[:m]))) and np.array_equal(out2[m], res[m])
+    assert np.array_equal(y3.view(torch.int16).cpu().numpy().view(np.uint16), yg)
+
+
+@pytest.mark.parametrize("inter,k,m", [(256, 512, 200), (384, 1024, 300), (128, 256, 3)])
+def test_swiglu_front(env, oracle, inter, k, m):
+    """gate|up interleaved by 8, SwiGLU and NVFP4 re-quantization in the epilogue: against the same steps done on the
+    host from the unfused bf16 output of the same linear. silu is evaluated with the hardware exponential and
+    reciprocal, so a bf16 rounding of it may flip where the exact value sits on a tie; such flips are counted."""
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    g, u = synth.fp4_linear(inter, k, 1, name="gate"), synth.fp4_linear(inter, k, 2, name="up")
+    fused = fp4.HostLinear.fuse([("gate", g.codes, g.sf, 1.0, 1.0), ("up", u.codes, u.sf, 1.0, 1.0)])
+    fused.alpha[:] = fused.alpha * np.float32(0.02)  # outputs of order 1, where silu bends
+    sw_host = fused.into_swiglu()
+    sw = sw_host.upload()
+    down_host = synth.fp4_linear(256, inter, 3, input_scale=0.5, name="down")
+    down = down_host.upload()
+    ws, act = fp4.Workspace(m, k), fp4.Workspace(m, inter)
+    xd = dev_u16(torch, synth.activations(m, k, 9))
+
+    # the unfused path: interleaved bf16 output, then SwiGLU and the quantizer on the host
+    yi = torch.zeros((m, 2 * inter), dtype=torch.bfloat16, device="cuda")
+    sw.forward(kern, ws, yi, 2 * inter, xd, k, m)
+    torch.cuda.synchronize()
+    y = bf16_to_f32(yi.view(torch.int16).cpu().numpy().view(np.uint16)).reshape(m, inter // 8, 2, 8)
+    gate, up = y[:, :, 0, :].reshape(m, inter).astype(np.float64), y[:, :, 1, :].reshape(m, inter)
+    silu = bf16_to_f32(bf16_bits((gate / (1.0 + np.exp(-gate))).astype(np.float32)))
+    want_act = bf16_bits(silu * up)
+    want_codes, want_sf = oracle.quant_fp4(want_act, down.g)
+
+    sw.forward_swiglu(kern, ws, act, xd, k, m, down.g)
+    yd = torch.zeros((m, 256), dtype=torch.bfloat16, device="cuda")
+    down.gemm(kern, act, yd, 256, m)
+    torch.cuda.synchronize()
+    codes, sf_tiled = act.read(m, inter)
+    sfa = oracle.untile_scales(sf_tiled, m, inter // 16).reshape(m, inter // 16)
+    bad_sf = (sfa != want_sf).mean()
+    bad_codes = (codes != want_codes).mean()
+    assert bad_sf < 2e-3 and bad_codes < 5e-3, (bad_sf, bad_codes)
+    # dequantized, the two activations agree everywhere up to one rounding flip of an element
+    a_got, a_want = oracle.dequant_fp4(codes, sfa, 1.0), oracle.dequant_fp4(want_codes, want_sf, 1.0)
+    assert np.abs(a_got - a_want).max() <= 0.26 * np.abs(a_want).max()
+
+    # the down projection over the GPU's own quantized activation: f64 reference over the same operands
+    ref = oracle.ref_gemm(a_got, oracle.dequant_fp4(down_host.codes, down_host.sf, 1.0)).astype(np.float64)
+    ref = ref * down_host.alpha.astype(np.float64)[None, :]
+    got = yd.float().cpu().numpy().astype(np.float64)
+    scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+    assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
+
+
+def test_swiglu_front_argument_errors(env):
+    torch, fp4, kern = env
+    from ferrite_amd import _lib, synth
+    plain = synth.fp4_linear(384, 256, 1).upload()  # n = 384 is not a gate|up pair of 256-multiples
+    ws, act = fp4.Workspace(4, 256), fp4.Workspace(4, 256)
+    x = torch.zeros((4, 256), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(_lib.FeError):
+        plain.forward_swiglu(kern, ws, act, x, 256, 4, 1.0)
+    pair = synth.fp4_linear(512, 256, 1).upload()
+    with pytest.raises(_lib.FeError):
+        pair.forward_swiglu(kern, ws, fp4.Workspace(4, 128), x, 256, 4, 1.0)  # act workspace narrower than n / 2
+    pair.forward_swiglu(kern, ws, act, x, 256, 0, 1.0)  # m = 0: a no-op
