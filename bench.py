@@ -305,6 +305,35 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     wbytes = n * k // 2 + n * k // 16
     res["nvfp4_5120x17408_m1"] = {"gemv_us": round(us, 2), "GB/s": round(wbytes / us / 1e3, 1),
                                   "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    del flin, yf
+    # the two neighbours of that GEMM in the prompt path: the fused gate|up front (SwiGLU + NVFP4 re-quantization in the
+    # epilogue, 2 x 17408 output columns) and an FP8 linear of the same shape
+    reps = 5
+    gate, up = synth.fp4_linear(n, k, SEED, name="gate"), synth.fp4_linear(n, k, SEED + 1, name="up")
+    pair = fp4.HostLinear.fuse([("gate", gate.codes, gate.sf, 1.0, 1.0), ("up", up.codes, up.sf, 1.0, 1.0)]).into_swiglu().upload()
+    del gate, up
+    act = fp4.Workspace(m, n)
+    pair.forward_swiglu(fk, fws, act, xf, k, m, 1.0)
+    a, b = ev.new(), ev.new()
+    ev.record(a, stream)
+    for _ in range(reps):
+        pair.forward_swiglu(fk, fws, act, xf, k, m, 1.0)
+    ev.record(b, stream)
+    ms = ev.ms(a, b) / reps
+    res["nvfp4_swiglu_front_5120x34816"] = {"quant_plus_gemm_ms": round(ms, 4), "TFLOP/s": round(2 * flops / ms / 1e9, 1),
+                                            "frac_mfma_peak": round(2 * flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    del pair, act
+    f8 = synth.fp8_linear(n, k, SEED).upload()
+    y8 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    f8.forward(fk, fws, y8, n, xf, k, m)
+    a, b = ev.new(), ev.new()
+    ev.record(a, stream)
+    for _ in range(reps):
+        f8.gemm(fk, fws, y8, n, m)
+    ev.record(b, stream)
+    ms = ev.ms(a, b) / reps
+    res["fp8_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                             "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
     return res
 
 

@@ -96,6 +96,7 @@ SYMBOLS = {
     "fe_fp4_workspace_create": (I, [PP, U32, U32]),
     "fe_fp4_workspace_destroy": (I, [P]),
     "fe_fp4_workspace_buffers": (I, [P, C.POINTER(U64), C.POINTER(U64), C.POINTER(U32), C.POINTER(U32)]),
+    "fe_fp4_workspace_operand": (I, [P, C.POINTER(U64)]),
     "fe_fp4_linear_forward": (I, [P, P, P, P, U64, U32, U64, U32, U32, U64]),
     "fe_fp4_linear_quantize": (I, [P, P, P, P, U64, U32, U32]),
     "fe_fp4_linear_gemm": (I, [P, P, P, P, U64, U32, U32, U64]),

@@ -229,6 +229,12 @@ int fe_fp4_workspace_buffers(const fe_fp4_workspace *ws, fe_devptr_t *codes, fe_
     return 0;
 }
 
+int fe_fp4_workspace_operand(const fe_fp4_workspace *ws, fe_devptr_t *aq) {
+    if (!ws || !aq) return fe_set_error(FE_ERR_ARG, "fe_fp4_workspace_operand", "null argument");
+    *aq = ws->aq.p;
+    return 0;
+}
+
 int fe_fp4_linear_quantize(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
                            fe_devptr_t x, uint32_t lda, uint32_t m) {
     if (!l || !kern || !ws) return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_quantize", "null argument");

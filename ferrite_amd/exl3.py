@@ -293,3 +293,38 @@ class Workspace:
         if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
             _lib._lib.fe_exl3_workspace_destroy(self.h)
             self.h = None
+
+
+def tune(kern: Kernels, t: Exl3Tensor, iters: int = 50, w16: float = 0.25, copies_bytes: int = 600 << 20):
+    """Times every fitting plan on one tensor shape at 1 and 16 rows and returns (best plan, table), the table a list of
+    (plan, us at 1 row, us at 16 rows) sorted by us1 + w16 * us16 (the measure of
+    crates/fe-exl3/src/bin/exl3-tune.rs:75-118). Launches cycle over enough copies of the weights that none is served
+    from a cache; candidates are the split counts that divide the K steps (ver 1) and the streamed form at 2 and 3
+    programs per CU (ver 2)."""
+    import torch
+    steps = t.k // 64
+    cands = [Plan(sk, 4, 1, 0) for sk in range(1, steps // 2 + 1) if steps % sk == 0 and sk <= 64]
+    cands += [Plan(1, 4, 2, occ) for occ in (2, 3)]
+    copies = max(2, min(64, copies_bytes // max(1, t.trellis_bytes()) + 1))
+    devs = [DeviceExl3.upload_strips(t) for _ in range(copies)]
+    x = torch.full((16, t.k), 1.0, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros((16, t.n), dtype=torch.bfloat16, device="cuda")
+    table = []
+    for p in cands:
+        lins = [Linear.from_view(kern, d.name, d.view, p) for d in devs]
+        ws = Workspace(lins[:1], 16)
+        us = []
+        for rows in (1, 16):
+            lins[0].rotate_input(x, Dtype.Bf16, rows, ws)
+            for lin in lins[:2]:
+                lin.gemv_rotated(ws.xh_ptr, y, Dtype.Bf16, rows, ws)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for i in range(iters):
+                lins[i % copies].gemv_rotated(ws.xh_ptr, y, Dtype.Bf16, rows, ws)
+            b.record()
+            torch.cuda.synchronize()
+            us.append(a.elapsed_time(b) * 1e3 / iters)
+        table.append((p, us[0], us[1]))
+    table.sort(key=lambda e: e[1] + w16 * e[2])
+    return table[0][0], table

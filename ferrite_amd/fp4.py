@@ -148,6 +148,9 @@ class Workspace:
         c, s = C.c_uint64(), C.c_uint64()
         check(_lib.lib().fe_fp4_workspace_buffers(self.h, C.byref(c), C.byref(s), None, None))
         self.codes_ptr, self.sf_ptr = c.value, s.value
+        a = C.c_uint64()
+        check(_lib.lib().fe_fp4_workspace_operand(self.h, C.byref(a)))
+        self.operand_ptr = a.value
 
     def read_fp8(self, m, k):
         """e4m3 codes [m][k] as a host array."""

@@ -48,6 +48,10 @@ int fe_fp4_workspace_destroy(fe_fp4_workspace *ws);
 int fe_fp4_workspace_buffers(const fe_fp4_workspace *ws, fe_devptr_t *codes, fe_devptr_t *sf, uint32_t *max_rows,
                              uint32_t *max_k);
 
+/* The fp16 operand [rows][k] the quantizer leaves beside the codes (what the GEMM kernels read): a small power of two
+ * times the quantized value, exact. No counterpart in the reference, whose tensor cores read the codes. */
+int fe_fp4_workspace_operand(const fe_fp4_workspace *ws, fe_devptr_t *aq);
+
 /* PromptLinear::forward (lib.rs:510-516): y (row stride ldy) = x (bf16, row stride lda) . W^T for m rows; with res
  * (stride ldy, may equal y): y = bf16(bf16(x . W^T) + res). res == 0: none. */
 int fe_fp4_linear_forward(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,

@@ -113,14 +113,18 @@ def test_plans():
     assert Plan.parse("2,8") == Plan(2, 8, 1, 0)
     assert Plan.parse("10,4,9,2") == Plan(10, 4, 9, 2)
     assert Plan.parse("x") is None
-    # every plan divides the K range into whole load steps of 64 channels and reaches the program target when it can
+    # every plan divides the K range into whole load steps of 64 channels (at least 2 a program) and, among the split
+    # counts that do, takes the one whose program count is closest to the target as a ratio
+    import math
     for k, n in [(5120, 17408), (17408, 5120), (5120, 5120), (5120, 1024), (128, 128), (1024, 256)]:
-        for blocks in (256, 1024):
+        for blocks in (256, 704, 1024):
             p = Linear.plan_for(k, n, 4, blocks)
-            assert (k // 64) % p.sk == 0 and k // 64 // p.sk >= min(2, k // 64)
-            if p.sk > 1:
-                smaller = [d for d in range(1, p.sk) if (k // 64) % d == 0]
-                assert all(n // 128 * d < blocks for d in smaller)
+            steps = k // 64
+            assert steps % p.sk == 0 and steps // p.sk >= min(2, steps) and p.ver == 1
+            miss = lambda d: abs(math.log(n // 128 * d / blocks))
+            fits = [d for d in range(1, steps + 1) if steps % d == 0 and steps // d >= 2] or [1]
+            assert miss(p.sk) <= min(miss(d) for d in fits) + 1e-12
+    assert Linear.plan_for(5120, 17408, 4, 704).sk == 5 and Linear.plan_for(17408, 5120, 4, 704).sk == 17
     os.environ["FE_EXL3_NOSPLIT"] = "1"
     try:
         assert Linear.plan_for(5120, 1024, 4, 1024).sk == 1

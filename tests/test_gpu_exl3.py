@@ -318,3 +318,15 @@ def test_prefill_gemm_tiles_cut_or_whole(env, oracle, monkeypatch):
     lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32Add, m, ws)
     torch.cuda.synchronize()
     assert np.abs(y.cpu().numpy().astype(np.float64) - 1.0 - ref).max() / rms < 1e-4
+
+
+def test_tuner_returns_a_fitting_plan(env):
+    """ferrite_amd.exl3.tune (the role of exl3-tune): every candidate is timed at 1 and 16 rows, the best one fits."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(1024, 512, 4, 3)
+    best, table = exl3.tune(kern, t, iters=5, copies_bytes=1 << 20)
+    assert (t.k // 64) % best.sk == 0 and len(table) >= 4
+    assert all(us1 > 0 and us16 > 0 for _, us1, us16 in table)
+    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), best)
+    assert lin.plan.sk == best.sk
