@@ -142,13 +142,19 @@ def main():
 
     # an event pair around every GEMV launch of the timed region
     events = [[(ev.new(), ev.new()) for _ in linears] for _ in range(args.steps)]
+    one_launch = [l[2].forward_is_one_launch(1) for l in linears]
 
     def step(timed_idx=None):
         for li, (name, bits, lin, x, y) in enumerate(linears):
-            lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
+            one = one_launch[li]  # forward() is the GEMV alone (it rotates its own input): the pair brackets that launch
+            if not one:
+                lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
             if timed_idx is not None:
                 ev.record(events[timed_idx][li][0], stream)
-            lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
+            if one:
+                lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws)
+            else:
+                lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
             if timed_idx is not None:
                 ev.record(events[timed_idx][li][1], stream)
 
@@ -167,7 +173,8 @@ def main():
     for li, (name, bits, lin, x, y) in enumerate(linears):
         ms = [ev.ms(*events[i][li]) for i in range(args.steps)]
         us = sum(ms) / len(ms) * 1e3
-        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "plan": [lin.plan.sk, lin.plan.ver, lin.plan.occ]}
+        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "plan": [lin.plan.sk, lin.plan.ver, lin.plan.occ],
+                                   "launches": 1 if one_launch[li] else 2}
         if bits == 4 and lin.k == 5120:
             dom_ms += ms
             dom_bytes = lin.weight_bytes()
@@ -212,8 +219,7 @@ def traffic_pass(torch, np, exl3, synth):
         big.add_(1)
         kern.probe_stream_read(buf, 1024, 1)
         big.add_(1)
-        lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
-        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws)
     torch.cuda.synchronize()
     print(json.dumps({"exl3_probe_v4_reads_KiB": lin.weight_bytes() / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
                       "roofline_kernel": "exl3_gemv_b4_r1", "algorithmic_KiB": lin.weight_bytes() / 1024}))
@@ -226,8 +232,7 @@ def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):
     check(lib.fe_hip_stream_create(C.byref(s)))
     check(lib.fe_hip_graph_begin(s))
     for name, bits, lin, x, y in linears:
-        lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws, stream=s)
-        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws, stream=s)
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws, stream=s)
     g = C.c_void_p()
     check(lib.fe_hip_graph_end(s, C.byref(g)))
     for _ in range(max(warmup, 2)):

@@ -336,8 +336,26 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
+// Decode-sized rows. With x != 0 the split-K kernel rotates x itself and leaves the rotated rows in xh (callers check
+// fused_rotation_fits first); otherwise it reads xh.
+static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
+                       const fe_exl3_workspace *ws, fe_devptr_t x, uint32_t x_f32);
+
+// The split-K kernel can rotate its own input when every program's K range is whole 128-element blocks.
+static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
+    const char *e = getenv("FE_EXL3_NO_FUSED_ROT");  // read per call: tests compare both paths in one process
+    const bool off = e && atoi(e) != 0;
+    const fe_exl3_plan &p = l->plan;
+    return !off && rows >= 1 && rows <= kMaxRowsPerPass && p.ver != 2 && (l->k / 64 / p.sk) % 2 == 0;
+}
+
 int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
                                 uint32_t rows, const fe_exl3_workspace *ws) {
+    return launch_rows(l, s, xh, y, y_dtype, rows, ws, 0, 0);
+}
+
+static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
+                       const fe_exl3_workspace *ws, fe_devptr_t x, uint32_t x_f32) {
     if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "null argument");
     if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "bad y dtype");
     const fe_exl3_plan &p = l->plan;
@@ -381,12 +399,25 @@ int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devpt
     uint32_t n = l->n, k = l->k, sk = p.sk, mode = (uint32_t)y_dtype, stride_k, stride_nb;
     view_strides(l->view, &stride_k, &stride_nb);
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
-    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk};
+    fe_devptr_t suh = l->view.suh;
+    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk, &x, &x_f32, &suh, &xh};
     return fe_hip_launch(l->kern->gemv[bits_slot(l->bits)][rg - 1], n / 128 * sk, 1, 1, 256, 1, 1, lds, s, args);
 }
 
+int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }
+
 int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
                            fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (l && kern && ws && x && fused_rotation_fits(l, rows)) {  // one launch: the GEMV rotates its own input
+        if (rows > ws->max_rows || l->k > ws->max_k) {
+            char msg[160];
+            snprintf(msg, sizeof msg, "%s: rows %u (workspace %u x %u)", l->name.c_str(), rows, ws->max_rows, ws->max_k);
+            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_forward", msg);
+        }
+        if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+            return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "x is bf16 or f32");
+        return launch_rows(l, s, ws->xh.p, y, y_dtype, rows, ws, x, (uint32_t)x_dtype & 1);
+    }
     FE_TRY(fe_exl3_linear_rotate_input(l, kern, s, x, x_dtype, rows, ws));
     return fe_exl3_linear_gemv_rotated(l, s, ws->xh.p, y, y_dtype, rows, ws);
 }

@@ -151,6 +151,40 @@ extern "C" __global__ __launch_bounds__(128) void exl3_had_cols_bf16(const float
 
 // ---- input rotation ------------------------------------------------------------------------------------------------
 
+// One 128-element block of a row: fp16(H(x * suh) / sqrt(128)), 4 elements a lane of a half wavefront. `at` indexes x
+// (bf16, or f32 with x_f32), `c` the block's channel of this lane. Split in two so that a caller can issue the loads
+// early; all 32 lanes of the half wavefront take part in rot_finish.
+struct RotRaw {
+    f32x4 xf;
+    u32x2 xb, s;
+};
+__device__ __forceinline__ RotRaw rot_load(const void* x, uint32_t x_f32, const uint16_t* suh, size_t at, uint32_t c) {
+    RotRaw r;
+    if (x_f32)
+        r.xf = *(const f32x4*)((const float*)x + at);
+    else
+        r.xb = *(const u32x2*)((const uint16_t*)x + at);
+    r.s = *(const u32x2*)(suh + c);
+    return r;
+}
+__device__ __forceinline__ u32x2 rot_finish(const RotRaw& r, uint32_t x_f32, uint32_t l32) {
+    float v[4];
+    if (x_f32) {
+        v[0] = r.xf[0], v[1] = r.xf[1], v[2] = r.xf[2], v[3] = r.xf[3];
+    } else {
+        v[0] = __uint_as_float(r.xb[0] << 16), v[1] = __uint_as_float(r.xb[0] & 0xffff0000u);
+        v[2] = __uint_as_float(r.xb[1] << 16), v[3] = __uint_as_float(r.xb[1] & 0xffff0000u);
+    }
+    v[0] *= f16_bits_to_f32(r.s[0] & 0xffff), v[1] *= f16_bits_to_f32(r.s[0] >> 16);
+    v[2] *= f16_bits_to_f32(r.s[1] & 0xffff), v[3] *= f16_bits_to_f32(r.s[1] >> 16);
+    fwht128_half_wave(v, l32);
+    return (u32x2){pack_f16x2(v[0] * FE_HAD_SCALE, v[1] * FE_HAD_SCALE), pack_f16x2(v[2] * FE_HAD_SCALE, v[3] * FE_HAD_SCALE)};
+}
+__device__ __forceinline__ u32x2 rot_block(const void* x, uint32_t x_f32, const uint16_t* suh, size_t at, uint32_t c,
+                                           uint32_t l32) {
+    return rot_finish(rot_load(x, x_f32, suh, at, c), x_f32, l32);
+}
+
 // xh[row][k] = fp16(H(x * suh) / sqrt(128)), x bf16 (x_f32 = 0) or f32. grid (ceil(k / 512), rows), 128 threads: each
 // half wavefront one 128-element block, 4 elements a lane. (kernels/k-exl3/src/gemv.rs:147-170)
 extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_f32, const uint16_t* suh,
@@ -160,23 +194,8 @@ extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uin
     bool live = blk * 128 < k;
     uint32_t c = (live ? blk : 0) * 128 + 4 * l32;
     size_t at = (size_t)blockIdx.y * k + c;
-    float v[4];
-    if (x_f32) {
-        f32x4 t = *(const f32x4*)((const float*)x + at);
-        v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
-    } else {
-        u32x2 t = *(const u32x2*)((const uint16_t*)x + at);
-        v[0] = __uint_as_float(t[0] << 16), v[1] = __uint_as_float(t[0] & 0xffff0000u);
-        v[2] = __uint_as_float(t[1] << 16), v[3] = __uint_as_float(t[1] & 0xffff0000u);
-    }
-    u32x2 s = *(const u32x2*)(suh + c);
-    v[0] *= f16_bits_to_f32(s[0] & 0xffff), v[1] *= f16_bits_to_f32(s[0] >> 16);
-    v[2] *= f16_bits_to_f32(s[1] & 0xffff), v[3] *= f16_bits_to_f32(s[1] >> 16);
-    fwht128_half_wave(v, l32);
-    if (live) {
-        u32x2 o = {pack_f16x2(v[0] * FE_HAD_SCALE, v[1] * FE_HAD_SCALE), pack_f16x2(v[2] * FE_HAD_SCALE, v[3] * FE_HAD_SCALE)};
-        *(u32x2*)(xh + at) = o;
-    }
+    u32x2 o = rot_block(x, x_f32, suh, at, c, l32);
+    if (live) *(u32x2*)(xh + at) = o;
 }
 
 // ---- decode GEMV -----------------------------------------------------------------------------------------------------
@@ -322,12 +341,15 @@ __device__ __forceinline__ f32x4 row_scales(const uint16_t* svh, uint32_t col) {
 // inputs of the program's K range pass through LDS in chunks of `chunk` load steps (a multiple of 4): dynamic LDS
 // max(m * (chunk * 128 + 16), m * GEMV_RED_PITCH * 4) bytes. With sk > 1 the splits leave f32 partials in
 // z[split][m][n]; the last to arrive (counters[column block]) adds them in split order, finishes the block and re-arms
-// the counter. (kernels/k-exl3/src/gemv.rs:412-587)
+// the counter. With x != nullptr the kernel rotates its own inputs from x (as exl3_rot_in does, bit for bit) instead of
+// reading xh, and leaves them in xh_out: one launch for the whole linear. That needs every staged K range to be whole
+// 128-element blocks: k / 64 / sk and chunk even. (kernels/k-exl3/src/gemv.rs:412-587)
 template <int BITS, int RG>
 __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
                                           const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
                                           uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode,
-                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk) {
+                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk, const void* x,
+                                          uint32_t x_f32, const uint16_t* __restrict__ suh, uint16_t* xh_out) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
     constexpr uint32_t tw = 8 * BITS;
@@ -358,6 +380,26 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
 #pragma unroll
     for (int rg = 0; rg < RG; rg++) acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+    // Rotating here: the first block's loads go out ahead of the trellis loads (loads return in order), so that the
+    // rotation runs while the first trellis words are still on their way.
+    const uint32_t rot_hw = tid >> 5, rot_l32 = tid & 31;
+    auto rot_at = [&](uint32_t c0, uint32_t nblk, uint32_t p, size_t& at, uint32_t& c, uint32_t& off) {
+        uint32_t row = p / nblk, b = p - row * nblk;
+        c = (kt0 + 4 * c0) * 16 + b * 128 + 4 * rot_l32;
+        at = (size_t)row * k + c;
+        off = row * xpitch + b * 256 + 8 * rot_l32;
+    };
+    RotRaw rot_raw = {};
+    if (x) {
+        const uint32_t nblk = (steps < chunk ? steps : chunk) / 2;
+        if (rot_hw < m * nblk) {
+            size_t at;
+            uint32_t c, off;
+            rot_at(0, nblk, rot_hw, at, c, off);
+            rot_raw = rot_load(x, x_f32, suh, at, c);
+        }
+    }
+
     // the ring is indexed by constants only, so it stays in registers
     LaneWords<BITS> ring[DEPTH];
 #pragma unroll
@@ -368,7 +410,28 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     for (uint32_t c0 = 0; c0 < steps; c0 += chunk) {
         const uint32_t cs = steps - c0 < chunk ? steps - c0 : chunk;
         if (c0) __syncthreads();
-        {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
+        if (x) {
+            // the input rotation of this K range, done here: half wavefronts take (row, 128-block) pairs; the programs
+            // of column block 0 also leave the rotated input in xh_out. The range starts and ends on block boundaries
+            // (the launcher's condition for passing x).
+            const uint32_t nblk = cs / 2, total = m * nblk;
+            uint32_t p = rot_hw, c = 0, off = 0;
+            size_t at = 0;
+            if (p < total) {
+                rot_at(c0, nblk, p, at, c, off);
+                if (c0) rot_raw = rot_load(x, x_f32, suh, at, c);
+            }
+            while (p < total) {
+                u32x2 o = rot_finish(rot_raw, x_f32, rot_l32);
+                *(u32x2*)(lds + off) = o;
+                if (nb == 0) *(u32x2*)(xh_out + at) = o;
+                p += 8;
+                if (p < total) {
+                    rot_at(c0, nblk, p, at, c, off);
+                    rot_raw = rot_load(x, x_f32, suh, at, c);
+                }
+            }
+        } else {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
             const uint32_t chunks16 = cs * 8;  // 16-byte pieces a row
             for (uint32_t i = tid; i < m * chunks16; i += 256) {
                 uint32_t row = i / chunks16, c = i - row * chunks16;
@@ -492,8 +555,9 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_b##BITS##_r##RG(                                      \
         const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,       \
         uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb,       \
-        uint32_t chunk) {                                                                                             \
-        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk);       \
+        uint32_t chunk, const void* x, uint32_t x_f32, const uint16_t* suh, uint16_t* xh_out) {                        \
+        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk, x,     \
+                            x_f32, suh, xh_out);                                                                      \
     }
 #define GEMV_FAMILY(BITS) GEMV_KERNEL(BITS, 1) GEMV_KERNEL(BITS, 2) GEMV_KERNEL(BITS, 3) GEMV_KERNEL(BITS, 4)
 GEMV_FAMILY(2)

@@ -262,6 +262,10 @@ class Linear:
         check(_lib.lib().fe_exl3_linear_forward(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), y.data_ptr(),
                                                 int(y_dtype), rows, ws.h))
 
+    def forward_is_one_launch(self, rows: int) -> bool:
+        """Whether forward() with this many rows is the decode GEMV alone, rotating its own input."""
+        return bool(_lib.lib().fe_exl3_linear_forward_is_one_launch(self.h, rows))
+
     def rotate_input(self, x, x_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
         check(_lib.lib().fe_exl3_linear_rotate_input(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), rows, ws.h))
 

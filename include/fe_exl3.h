@@ -77,9 +77,13 @@ int fe_exl3_workspace_destroy(fe_exl3_workspace *ws);
 int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t *max_rows, uint32_t *max_k);
 
 /* Linear::forward (linear.rs:274-287): y[rows][n] = x[rows][k] @ W; x bf16 or f32, y bf16 or f32 (+ the add forms),
- * both row-major and contiguous. rows <= 64 run the decode GEMV (HBM-bound); more rows run the LDS-staged MFMA GEMM. */
+ * both row-major and contiguous. rows <= 64 run the decode GEMV (HBM-bound); more rows run the LDS-staged MFMA GEMM.
+ * The workspace's xh holds the rotated input afterwards, as after rotate_input. */
 int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
                            fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws);
+/* 1 if forward() with this many rows is a single launch (the decode GEMV rotates its own input: every program's K range
+ * is whole 128-element Hadamard blocks), 0 if it is rotate_input followed by gemv_rotated. Same bits either way. */
+int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows);
 /* Linear::rotate_input (linear.rs:289-298): xh = fp16(H(x * suh) / sqrt(128)) into the workspace. */
 int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
                                 int x_dtype, uint32_t rows, const fe_exl3_workspace *ws);

@@ -330,3 +330,42 @@ def test_tuner_returns_a_fitting_plan(env):
     assert all(us1 > 0 and us16 > 0 for _, us1, us16 in table)
     lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), best)
     assert lin.plan.sk == best.sk
+
+
+@pytest.mark.parametrize("k,sk,fits", [(1024, 1, True), (1024, 4, True), (2048, 16, True), (1024, 8, True), (1024, 16, False),
+                                       (1280, 2, True), (1280, 4, False)])
+def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, monkeypatch):
+    """forward() for up to 64 rows is one launch when every program's K range is whole 128-element blocks (the GEMV
+    rotates its own input and leaves it in the workspace), two launches otherwise. Both give the same bits, in y and in
+    the workspace's rotated input, for bf16 and f32 inputs."""
+    torch, exl3, kern = env
+    from ferrite_amd import _lib, synth
+    from ferrite_amd._lib import check
+    assert ((k // 64 // sk) % 2 == 0) == fits
+    t = synth.exl3_tensor(k, 384, 4, 70 + sk)
+    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(sk=sk, wk=1, ver=1, occ=2))
+    assert lin.forward_is_one_launch(1) == fits and lin.forward_is_one_launch(64) == fits and not lin.forward_is_one_launch(65)
+    ws = exl3.Workspace([lin], 64)
+    xb = synth.activations(64, k, 8, outliers=True)
+    xd = dev_u16(torch, xb)
+    xf = xd.view(torch.bfloat16).float().contiguous()
+    for rows in (1, 7, 16, 33, 64):
+        for x, xdt in ((xd, exl3.Dtype.Bf16), (xf, exl3.Dtype.F32)):
+            out = {}
+            for mode in ("fused", "separate"):
+                if mode == "separate":
+                    monkeypatch.setenv("FE_EXL3_NO_FUSED_ROT", "1")
+                check(_lib.lib().fe_hip_memset_d8(ws.xh_ptr, 0x7e, 64 * k * 2, None))  # fp16 NaNs: stale inputs would show
+                y = torch.full((65, lin.n), float("nan"), dtype=torch.float32, device="cuda")
+                lin.forward(x, xdt, y, exl3.Dtype.F32, rows, ws)
+                torch.cuda.synchronize()
+                out[mode] = (y.cpu().numpy(), ws.xh(rows, k))
+                monkeypatch.delenv("FE_EXL3_NO_FUSED_ROT", raising=False)
+            assert np.array_equal(out["fused"][1], out["separate"][1]), (rows, xdt)
+            assert np.array_equal(out["fused"][0][:rows].view(np.uint32), out["separate"][0][:rows].view(np.uint32)), (rows, xdt)
+            assert np.isnan(out["fused"][0][rows:]).all()
+    # the rotated input the fused launch leaves behind is the oracle's (as for the separate kernel)
+    # (outlier channels: the f32 butterflies leave an absolute error, so small results may be off by more than an ulp)
+    want = oracle.rotate_input_ref(to_oracle(oracle, t), bf16_to_f64(xb)).view(np.float16).astype(np.float64)
+    got = out["fused"][1].view(np.float16).astype(np.float64)
+    assert np.all(np.abs(got - want) <= np.abs(want) / 1024.0 + 1e-5 * np.sqrt((want ** 2).mean()))
