@@ -14,6 +14,7 @@
 namespace {
 
 constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
+constexpr uint32_t kHatRows = 513;          // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
 constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
@@ -44,6 +45,8 @@ struct fe_exl3_kernels {
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     fe_function_t gemm_reduce = nullptr;
+    fe_function_t hat_tiles[6] = {};  // trellis -> fp16 weights as the GEMM's LDS images
+    fe_function_t gemm_hat = nullptr; // the GEMM over them
     uint32_t group_m = 8;
 };
 
@@ -60,6 +63,7 @@ struct fe_exl3_linear {
 struct fe_exl3_workspace {
     uint32_t max_rows = 0, max_k = 0;
     FeBuf xh, z, counters, part;  // part: partial tiles of the prefill GEMM (rows > 64 only)
+    FeBuf hat;                    // decoded fp16 weights of one linear (workspaces of kHatRows rows or more)
     size_t z_len = 0, counters_len = 0;
 };
 
@@ -113,8 +117,12 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
+        snprintf(nm, sizeof nm, "exl3_hat_tiles_b%d", kBits[i]);
+        get(&k->hat_tiles[i], nm);
         if (i == 0) get(&k->gemm_reduce, "exl3_gemm_reduce");
     }
+    get(&k->gemm_hat, "exl3_gemm_hat");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm_hat, kGemmLds);
     if (const char *g = getenv("FE_EXL3_GROUP")) k->group_m = (uint32_t)atoi(g);
     if (!c) {
         int cus = 0;
@@ -260,11 +268,24 @@ int fe_exl3_linear_view(const fe_exl3_linear *l, fe_exl3_view *view, fe_exl3_pla
 
 size_t fe_exl3_linear_weight_bytes(const fe_exl3_linear *l) { return l ? (size_t)l->k * l->n * l->bits / 8 : 0; }
 
+// Many rows: decoding the trellis once into fp16 tiles and running the GEMM over them beats decoding inside the GEMM,
+// where each 256-row tile of the output decodes its weights again. From kHatRows rows on (FE_EXL3_HAT_ROWS overrides; 0
+// turns the form off) and only with a workspace created for that many rows, which then holds the largest linear's
+// decoded weights (2 bytes a weight).
+static uint32_t hat_rows() {
+    const char *e = getenv("FE_EXL3_HAT_ROWS");  // read per call: tests compare both forms in one process
+    if (!e) return kHatRows;
+    int v = atoi(e);
+    return v <= 0 ? 0xffffffffu : std::max<uint32_t>((uint32_t)v, kMaxRowsPerPass + 1);
+}
+static size_t hat_bytes(const fe_exl3_linear *l) { return (size_t)((l->n / 128 + 1) / 2) * 256 * l->k * 2; }
+
 int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows) {
     if (!out || (count && !linears) || !max_rows) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_create", "bad argument");
-    size_t max_k = 128, max_z = 0, max_zs = 0, max_nb = 1;
+    size_t max_k = 128, max_z = 0, max_zs = 0, max_nb = 1, max_hat = 0;
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
+        max_hat = std::max(max_hat, hat_bytes(l));
         max_k = std::max<size_t>(max_k, l->k);
         if (l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
         if (l->programs) max_zs = std::max<size_t>(max_zs, (size_t)(l->programs + l->n / 128) * 128);
@@ -280,6 +301,8 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     int cus = 0;
     if (!c && max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
     if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
+    // zeroed once: the unused half of the last tile of an odd count of column blocks is read (and its sums discarded)
+    if (!c && max_rows >= hat_rows() && max_hat) c = ws->hat.zeroed(max_hat);
     if (c) {
         delete ws;
         return c;
@@ -329,8 +352,19 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = g.full, splits = g.splits;
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
-    void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &full, &splits, &part};
-    FE_TRY(fe_hip_launch(kern->gemm[bits_slot(l->bits)], g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (rows >= hat_rows() && ws->hat.bytes >= hat_bytes(l)) {
+        fe_devptr_t hat = ws->hat.p;
+        const uint32_t ktiles = k / 64, nbs = n / 128;
+        const uint32_t gy = std::min(ktiles, std::max(1u, (8 * std::max(kern->cus, 1u) + nbs - 1) / nbs));
+        void *dargs[] = {&tr, &hat, &k, &stride_k, &stride_nb};
+        FE_TRY(fe_hip_launch(kern->hat_tiles[bits_slot(l->bits)], nbs, gy, 1, 256, 1, 1, 0, s, dargs));
+        group = 0;  // the raster that deals column tiles to the XCDs: each decoded weight panel goes through one L2
+        void *args[] = {&xh, &hat, &svh, &y, &n, &k, &rows, &mode, &group, &full, &splits, &part};
+        FE_TRY(fe_hip_launch(kern->gemm_hat, g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    } else {
+        void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &full, &splits, &part};
+        FE_TRY(fe_hip_launch(kern->gemm[bits_slot(l->bits)], g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    }
     if (!g.cut()) return 0;
     void *rargs[] = {&part, &svh, &y, &n, &rows, &mode, &group, &full, &splits};
     return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);

@@ -25,8 +25,26 @@ __device__ __forceinline__ uint32_t gm_swz(uint32_t r, uint32_t c) { return r * 
 // Grouped raster: `group` row tiles (fastest) sweep all column tiles before the next group, so programs that run
 // together share weight panels in L2 (kernels/k-fp4/src/lib.rs:298-308). Workgroups go to the 8 XCDs round-robin, so
 // with a group of 8 row tiles each XCD's L2 keeps one 256-row panel of activations.
+//
+// group == 0 is the raster for weights that are large in memory (decoded fp16 tiles): column tiles are dealt to the XCDs
+// instead, tile tn of a band of 8 to XCD tn % 8, all row tiles of it in turn, so that each weight panel is fetched into
+// one L2 only and the (smaller) activations into all of them. A last band of fewer than 8 column tiles is swept column
+// tile fastest.
 __device__ __forceinline__ void gemm_raster(uint32_t pid, uint32_t tiles_m, uint32_t tiles_n, uint32_t group, uint32_t& tm,
                                             uint32_t& tn) {
+    if (group == 0) {
+        uint32_t bands = tiles_n / 8, in_bands = bands * 8 * tiles_m;
+        if (pid < in_bands) {
+            uint32_t q = pid / 8;
+            tn = (q / tiles_m) * 8 + pid % 8;
+            tm = q % tiles_m;
+        } else {
+            uint32_t r = tiles_n - bands * 8, idx = pid - in_bands;
+            tn = bands * 8 + idx % r;
+            tm = idx / r;
+        }
+        return;
+    }
     uint32_t per_group = group * tiles_n;
     uint32_t first_m = (pid / per_group) * group;
     uint32_t gsize = tiles_m - first_m < group ? tiles_m - first_m : group;

@@ -796,30 +796,18 @@ struct Exl3Producer {
 // tiles; a wavefront's 128 columns are exactly one Hadamard block, so the output rotation is local to the wavefront.
 // grid full_tiles + (tiles - full_tiles) * splits with tiles = ceil(m / 256) * ceil(n / 256) (grouped raster), 256
 // threads, dynamic LDS GM_LDS_TILES (the epilogue reuses it). Tiles past full_tiles leave partials in `part` for
-// exl3_gemm_reduce.
-template <int BITS>
-__device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, const uint32_t* __restrict__ trellis,
-                                               const uint16_t* __restrict__ svh, void* y, uint32_t n, uint32_t k, uint32_t m,
-                                               uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m,
-                                               uint32_t full_tiles, uint32_t splits, float* part) {
+// exl3_gemm_reduce. make_producer(tn) builds the weight producer of 256-column tile tn.
+template <class MakeProducer>
+__device__ __forceinline__ void exl3_gemm_tile(const _Float16* __restrict__ xh, const uint16_t* __restrict__ svh, void* y,
+                                               uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t group_m,
+                                               uint32_t full_tiles, uint32_t splits, float* part,
+                                               MakeProducer make_producer) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t nbs = n / 128;
     const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nbs + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
     const uint32_t m0 = wk.tm * GM_BM, tn = wk.tn;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    constexpr uint32_t tw = 8 * BITS;
-    Exl3Producer<BITS> prod;
-    {
-        uint32_t tj = lane >> 3, q = lane & 7;
-        uint32_t nb1 = 2 * tn + 1 < nbs ? 2 * tn + 1 : 2 * tn;  // an odd block count: the last tile decodes block 2 tn twice
-        prod.base[0] = trellis + (size_t)(2 * tn) * stride_nb + tj * tw;
-        prod.base[1] = trellis + (size_t)nb1 * stride_nb + tj * tw;
-        prod.stride_k = stride_k;
-        prod.run_off = q * BITS;
-        prod.prev_off = (q * BITS + tw - 1) % tw;
-        prod.brow = tj * 16 + q;
-        prod.ks = wave;
-    }
+    auto prod = make_producer(tn);
     f32x16 acc[4][4];
     gemm_mainloop(xh, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
     if (wk.partial) {
@@ -857,6 +845,111 @@ __device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, 
         run(std::integral_constant<uint32_t, 3>{});
 }
 
+// The GEMM decoding the trellis itself: every 256-row tile of the output decodes its weights again.
+template <int BITS>
+__device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, const uint32_t* __restrict__ trellis,
+                                               const uint16_t* __restrict__ svh, void* y, uint32_t n, uint32_t k, uint32_t m,
+                                               uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m,
+                                               uint32_t full_tiles, uint32_t splits, float* part) {
+    exl3_gemm_tile(xh, svh, y, n, k, m, y_mode, group_m, full_tiles, splits, part, [&](uint32_t tn) {
+        constexpr uint32_t tw = 8 * BITS;
+        const uint32_t lane = threadIdx.x & 63, nbs = n / 128;
+        Exl3Producer<BITS> prod;
+        uint32_t tj = lane >> 3, q = lane & 7;
+        uint32_t nb1 = 2 * tn + 1 < nbs ? 2 * tn + 1 : 2 * tn;  // an odd block count: the last tile decodes block 2 tn twice
+        prod.base[0] = trellis + (size_t)(2 * tn) * stride_nb + tj * tw;
+        prod.base[1] = trellis + (size_t)nb1 * stride_nb + tj * tw;
+        prod.stride_k = stride_k;
+        prod.run_off = q * BITS;
+        prod.prev_off = (q * BITS + tw - 1) % tw;
+        prod.brow = tj * 16 + q;
+        prod.ks = threadIdx.x >> 6;
+        return prod;
+    });
+}
+
+// ---- prefill over decoded weights -----------------------------------------------------------------------------------
+//
+// For many rows the trellis is decoded once per call into `hat`, fp16, as the very images the GEMM keeps in LDS: block
+// (tn, kt) of 32 KB = rows n = 256 tn .. + 255 of k tile kt, 128 bytes a row, 16-byte chunk c of row r at position
+// c ^ (r & 7). The GEMM over it then copies blocks instead of decoding, with the same fragments, the same MFMA order and
+// so the same bits as exl3_gemm_b*.
+
+// grid (n / 128, gy), 256 threads; program (nb, j) decodes k tiles j, j + gy, ... of column block nb with the lane
+// mapping of Exl3Producer. The 16 KB of a k tile pass through LDS (two buffers, one barrier a tile) so that they leave
+// as whole 1 KB runs per wavefront instead of scattered 16-byte pieces.
+template <int BITS>
+__device__ __forceinline__ void exl3_hat_tiles_body(const uint32_t* __restrict__ trellis, unsigned char* __restrict__ hat,
+                                                    uint32_t k, uint32_t stride_k, uint32_t stride_nb) {
+    __shared__ __attribute__((aligned(16))) unsigned char img[2][GM_B_BYTES / 2];
+    constexpr uint32_t tw = 8 * BITS;
+    const uint32_t lane = threadIdx.x & 63, ks = threadIdx.x >> 6, tj = lane >> 3, q = lane & 7;
+    const uint32_t nb = blockIdx.x, ktiles = k / GM_BK;
+    const uint32_t* base = trellis + (size_t)nb * stride_nb + tj * tw;
+    const uint32_t run_off = q * BITS, prev_off = (q * BITS + tw - 1) % tw;
+    const uint32_t row = tj * 16 + q;
+    unsigned char* out = hat + (size_t)(nb >> 1) * ktiles * GM_B_BYTES + (nb & 1) * (GM_B_BYTES / 2) + 16 * threadIdx.x;
+    uint32_t kt = blockIdx.y;
+    if (kt >= ktiles) return;
+    const uint32_t* p = base + (size_t)(kt * 4 + ks) * stride_k;
+    LaneWords<BITS> cur = load_lane_words<BITS>(p + run_off, p + prev_off);
+    for (uint32_t it = 0; kt < ktiles; kt += gridDim.y, it++) {
+        uint32_t nk = kt + gridDim.y < ktiles ? kt + gridDim.y : kt;
+        const uint32_t* pn = base + (size_t)(nk * 4 + ks) * stride_k;
+        LaneWords<BITS> nxt = load_lane_words<BITS>(pn + run_off, pn + prev_off);
+        f16x8 op[2][2];
+        decode_lane<BITS>(cur, op);
+        unsigned char* buf = img[it & 1];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int kh = 0; kh < 2; kh++) *(f16x8*)(buf + gm_swz(row + 8 * h, 2 * ks + kh)) = op[h][kh];
+        __syncthreads();
+        unsigned char* blk = out + (size_t)kt * GM_B_BYTES;
+#pragma unroll
+        for (int j = 0; j < 4; j++) *(u32x4*)(blk + 4096 * j) = *(const u32x4*)(buf + 16 * threadIdx.x + 4096 * j);
+        cur = nxt;
+    }
+}
+
+// Weight producer over `hat`: a k tile of the 256-column tile is one 32 KB block, copied as it is; thread t moves chunks
+// t + 256 j (j < 4) of each 16 KB half.
+struct HatProducer {
+    const unsigned char* base;  // the tile's blocks + 16 * thread
+    struct Raw {
+        u32x4 c[2][4];
+    };
+    static constexpr int kStoreValu = 0;
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            if (b != half) continue;
+            const unsigned char* p = base + (size_t)kt * GM_B_BYTES + b * (GM_B_BYTES / 2);
+#pragma unroll
+            for (int j = 0; j < 4; j++) r.c[b][j] = *(const u32x4*)(p + 4096 * j);
+        }
+    }
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            if (b != part) continue;
+#pragma unroll
+            for (int j = 0; j < 4; j++) *(u32x4*)(Bs + b * (GM_B_BYTES / 2) + 16 * threadIdx.x + 4096 * j) = r.c[b][j];
+        }
+    }
+};
+
+extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_hat(const _Float16* xh, const unsigned char* hat,
+                                                                   const uint16_t* svh, void* y, uint32_t n, uint32_t k,
+                                                                   uint32_t m, uint32_t y_mode, uint32_t group_m,
+                                                                   uint32_t full_tiles, uint32_t splits, float* part) {
+    exl3_gemm_tile(xh, svh, y, n, k, m, y_mode, group_m, full_tiles, splits, part, [&](uint32_t tn) {
+        HatProducer prod;
+        prod.base = hat + (size_t)tn * (k / GM_BK) * GM_B_BYTES + 16 * threadIdx.x;
+        return prod;
+    });
+}
+
 // Finishes the tiles that exl3_gemm_b* cut along K: sums their partial slots and applies the output rotation and scale.
 // grid (tiles - full_tiles) * 64, 256 threads.
 extern "C" __global__ __launch_bounds__(256) void exl3_gemm_reduce(const float* part, const uint16_t* svh, void* y, uint32_t n,
@@ -879,6 +972,17 @@ extern "C" __global__ __launch_bounds__(256) void exl3_gemm_reduce(const float* 
         exl3_gemm_body<BITS>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m, full_tiles, splits,    \
                              part);                                                                                    \
     }
+#define HAT_KERNEL(BITS)                                                                                      \
+    extern "C" __global__ __launch_bounds__(256) void exl3_hat_tiles_b##BITS(                                 \
+        const uint32_t* trellis, unsigned char* hat, uint32_t k, uint32_t stride_k, uint32_t stride_nb) {     \
+        exl3_hat_tiles_body<BITS>(trellis, hat, k, stride_k, stride_nb);                                      \
+    }
+HAT_KERNEL(2)
+HAT_KERNEL(3)
+HAT_KERNEL(4)
+HAT_KERNEL(5)
+HAT_KERNEL(6)
+HAT_KERNEL(8)
 GEMM_KERNEL(2)
 GEMM_KERNEL(3)
 GEMM_KERNEL(4)

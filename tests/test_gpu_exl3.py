@@ -369,3 +369,55 @@ def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, 
     want = oracle.rotate_input_ref(to_oracle(oracle, t), bf16_to_f64(xb)).view(np.float16).astype(np.float64)
     got = out["fused"][1].view(np.float16).astype(np.float64)
     assert np.all(np.abs(got - want) <= np.abs(want) / 1024.0 + 1e-5 * np.sqrt((want ** 2).mean()))
+
+
+@pytest.mark.parametrize("bits,n,strips", [(2, 384, True), (3, 256, False), (4, 640, True), (5, 384, False), (6, 128, True),
+                                           (8, 384, True), (4, 2304, True), (3, 4224, False)])
+def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracle, bits, n, strips, monkeypatch):
+    """Many rows: the trellis is decoded once into fp16 tiles (the GEMM's own LDS images) and the GEMM copies them instead
+    of decoding per output tile row. Same fragments and MFMA order, so with whole tiles the same bits in every output
+    mode; the two forms walk the tiles in different orders, so with a last round cut along K other tiles are the cut
+    ones and those differ by the order of their f32 sums. FE_EXL3_HAT_ROWS moves the row count from which this form
+    runs (0: never). 2304 and 4224 columns: 9 and 17 column tiles, dealt to the XCDs in bands of 8."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    m = 600
+    t = synth.exl3_tensor(1024, n, bits, 90 + bits)
+    xd = dev_u16(torch, synth.activations(m, t.k, 6, outliers=True))
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3(t, strips), 256)
+    monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+    ws = exl3.Workspace([lin], m)  # created for the decoded form
+
+    def run(rows, dt, torch_dt, pre):
+        y = torch.full((m + 1, t.n), pre, dtype=torch_dt, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, y, dt, rows, ws)
+        torch.cuda.synchronize()
+        return y.view(torch.int16 if torch_dt == torch.bfloat16 else torch.int32).cpu().numpy()
+
+    for splits in (None, "1"):
+        if splits:
+            monkeypatch.setenv("FE_GEMM_SPLITS", splits)
+        for rows in (65, 300, 600):
+            for dt, tdt, pre in ((exl3.Dtype.F32, torch.float32, float("nan")), (exl3.Dtype.Bf16, torch.bfloat16, 7.0),
+                                 (exl3.Dtype.Bf16Add, torch.bfloat16, 1.5), (exl3.Dtype.F32Add, torch.float32, 0.25)):
+                monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+                tiles = run(rows, dt, tdt, pre)
+                monkeypatch.setenv("FE_EXL3_HAT_ROWS", "0")
+                fused = run(rows, dt, tdt, pre)
+                if splits:
+                    assert np.array_equal(tiles, fused), (splits, rows, dt)
+                else:
+                    as_f = lambda a: (a.astype(np.int32) << 16).view(np.float32) if a.dtype == np.int16 else a.view(np.float32)
+                    a, b = as_f(tiles[:rows]).astype(np.float64), as_f(fused[:rows]).astype(np.float64)
+                    rms = np.sqrt((b ** 2).mean())
+                    assert np.all(np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * rms), (rows, dt)
+                assert (tiles[rows:] == tiles[m]).all()  # rows past `rows` keep the prefill
+    monkeypatch.delenv("FE_GEMM_SPLITS", raising=False)
+    # and against the oracle
+    monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+    y = torch.zeros((m, t.n), dtype=torch.float32, device="cuda")
+    lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+    torch.cuda.synchronize()
+    o = to_oracle(oracle, t)
+    ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
+    assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
