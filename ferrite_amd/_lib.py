@@ -102,6 +102,21 @@ SYMBOLS = {
     "fe_fp4_linear_quantize": (I, [P, P, P, P, U64, U32, U32]),
     "fe_fp4_linear_gemm": (I, [P, P, P, P, U64, U32, U32, U64]),
     "fe_fp4_linear_forward_swiglu": (I, [P, P, P, P, P, U64, U32, U32, F]),
+    # fe_route.h
+    "fe_route_ctx_create": (I, [PP, P, P, P, P, P, U32]),
+    "fe_route_ctx_destroy": (I, [P]),
+    "fe_route_ctx_set_dec": (I, [P, U32]),
+    "fe_route_ctx_set_x3_gemm": (I, [P, I]),
+    "fe_route_linear_create": (I, [PP, C.c_char_p, U32, U32, P, P]),
+    "fe_route_linear_destroy": (I, [P]),
+    "fe_route_linear_forward": (I, [P, P, U64, U32, U64, U32, U32, U64]),
+    "fe_route_proj_create": (I, [PP, PP, C.POINTER(C.POINTER(U32)), C.POINTER(U32), SZ, P, U32]),
+    "fe_route_proj_destroy": (I, [P]),
+    "fe_route_proj_total_n": (U32, [P]),
+    "fe_route_proj_forward": (I, [P, P, U64, U64, U32, U32, C.POINTER(U64), C.POINTER(U32), SZ, C.POINTER(SZ)]),
+    "fe_route_silu_mul": (I, [P, U64, U64, U64, U32, U32, U32]),
+    "fe_route_copy2d": (I, [P, U64, U32, U64, U32, U32, U32]),
+    "fe_route_mlp_forward": (I, [P, P, P, P, P, U64, U64, U64, U64, U32, U32, U32]),
 }
 
 

@@ -13,4 +13,10 @@ fe_k_fp4_hsaco:
     .incbin "k_fp4.hsaco"
     .global fe_k_fp4_hsaco_end
 fe_k_fp4_hsaco_end:
+    .balign 4096
+    .global fe_k_route_hsaco
+fe_k_route_hsaco:
+    .incbin "k_route.hsaco"
+    .global fe_k_route_hsaco_end
+fe_k_route_hsaco_end:
     .section .note.GNU-stack,"",@progbits

@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_symbols():
     names = []
-    for h in ("fe_hip.h", "fe_exl3.h", "fe_fp4.h"):
+    for h in ("fe_hip.h", "fe_exl3.h", "fe_fp4.h", "fe_route.h"):
         text = open(os.path.join(ROOT, "include", h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(fe_[a-z0-9_]+)\s*\(", text)
@@ -36,7 +36,7 @@ def test_embedded_code_objects_are_gfx950_elf():
     out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ROOT, "ferrite_amd", "libferrite_amd.so")],
                          stdout=subprocess.PIPE, text=True).stdout
     # the code objects are private data of the library; check them through the build directory instead
-    for k in ("k_exl3", "k_fp4"):
+    for k in ("k_exl3", "k_fp4", "k_route"):
         p = os.path.join(ROOT, "ferrite_amd", "_build", k + ".hsaco")
         if os.path.exists(p):
             head = open(p, "rb").read(20)
