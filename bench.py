@@ -11,7 +11,9 @@ launch gaps and input rotations included. The nine weight sets total 401 MB, mor
 Cache, so every step streams its weights from HBM.
 
 `roofline` is the dominant kernel alone (the 4-bit GEMV of the 5120x17408 projections): its trellis bytes over its
-average launch duration, measured with HIP events on the launch stream inside the timed region.
+average launch duration, measured with HIP event pairs on the launch stream around its launches inside the timed
+region (the other launches of the timed region carry no events: every record is a packet of its own on the queue; a
+pass after the timed region brackets all nine for `per_linear_gemv`).
 `cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host.
 `m2048` reports the prefill GEMMs (EXL3 4-bit and NVFP4, 5120x17408, M = 2048) in TFLOP/s against the bf16/f16 MFMA
 peak; it is measured after the timed region and is not part of `value`.
@@ -140,47 +142,69 @@ def main():
         rel = float(np.abs(got - y_cpu).max() / np.sqrt((y_cpu ** 2).mean()))
         cpu["gpu_vs_cpu_max_err_over_rms"] = round(rel, 6)
 
-    # an event pair around every GEMV launch of the timed region
-    events = [[(ev.new(), ev.new()) for _ in linears] for _ in range(args.steps)]
+    # Event pairs on the launch stream. In the timed region only the dominant kernel's launches carry them (each record is
+    # a packet of its own on the queue and costs a few microseconds of the step); one more pass after the timed region
+    # brackets every linear for the per-linear table.
     one_launch = [l[2].forward_is_one_launch(1) for l in linears]
+    dominant = [bits == 4 and lin.k == 5120 for name, bits, lin, x, y in linears]
+    events = [[(ev.new(), ev.new()) if dominant[li] else None for li in range(len(linears))] for _ in range(args.steps)]
+    table_events = [(ev.new(), ev.new()) for _ in linears]
 
-    def step(timed_idx=None):
-        for li, (name, bits, lin, x, y) in enumerate(linears):
-            one = one_launch[li]  # forward() is the GEMV alone (it rotates its own input): the pair brackets that launch
-            if not one:
-                lin.rotate_input(x, exl3.Dtype.Bf16, 1, ws)
-            if timed_idx is not None:
-                ev.record(events[timed_idx][li][0], stream)
-            if one:
-                lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws)
-            else:
-                lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, 1, ws)
-            if timed_idx is not None:
-                ev.record(events[timed_idx][li][1], stream)
+    # The step's calls into the C ABI, with every argument prepared once.
+    f_forward, f_rotate, f_rotated, f_record = (lib.fe_exl3_linear_forward, lib.fe_exl3_linear_rotate_input,
+                                                lib.fe_exl3_linear_gemv_rotated, lib.fe_hip_event_record)
+    bf16 = int(exl3.Dtype.Bf16)
+    calls = []
+    for li, (name, bits, lin, x, y) in enumerate(linears):
+        if one_launch[li]:  # forward() is the GEMV alone (it rotates its own input): the pair brackets that launch
+            calls.append((None, (f_forward, (lin.h, kern.h, stream, x.data_ptr(), bf16, y.data_ptr(), bf16, 1, ws.h))))
+        else:
+            calls.append(((f_rotate, (lin.h, kern.h, stream, x.data_ptr(), bf16, 1, ws.h)),
+                          (f_rotated, (lin.h, stream, ws.xh_ptr, y.data_ptr(), bf16, 1, ws.h))))
+
+    def step(pairs=None):
+        rc = 0
+        for li, (pre, (fn, a)) in enumerate(calls):
+            if pre is not None:
+                rc |= pre[0](*pre[1])
+            pair = pairs[li] if pairs is not None else None
+            if pair is not None:
+                rc |= f_record(pair[0], stream)
+            rc |= fn(*a)
+            if pair is not None:
+                rc |= f_record(pair[1], stream)
+        _lib.check(rc)
 
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(i)
+        step(events[i])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
     value = total_bytes / (dt / args.steps) / 1e9
 
-    per, dom_ms = {}, []
+    dom_ms = []
     for li, (name, bits, lin, x, y) in enumerate(linears):
-        ms = [ev.ms(*events[i][li]) for i in range(args.steps)]
-        us = sum(ms) / len(ms) * 1e3
-        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "plan": [lin.plan.sk, lin.plan.ver, lin.plan.occ],
-                                   "launches": 1 if one_launch[li] else 2}
-        if bits == 4 and lin.k == 5120:
-            dom_ms += ms
+        if dominant[li]:
+            dom_ms += [ev.ms(*events[i][li]) for i in range(args.steps)]
             dom_bytes = lin.weight_bytes()
             dom_kernel = "exl3_gemv_stream_b4" if lin.plan.ver == 2 else "exl3_gemv_b4_r1"
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
+
+    per, reps = {}, max(args.steps, 5)
+    acc = [0.0] * len(linears)
+    for _ in range(reps):  # after the timed region: every linear bracketed
+        step(table_events)
+        for li in range(len(linears)):
+            acc[li] += ev.ms(*table_events[li])
+    for li, (name, bits, lin, x, y) in enumerate(linears):
+        us = acc[li] / reps * 1e3
+        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "plan": [lin.plan.sk, lin.plan.ver, lin.plan.occ],
+                                   "launches": 1 if one_launch[li] else 2}
 
     out = {
         "metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048",
