@@ -22,6 +22,7 @@ struct fe_fp4_kernels {
     fe_module_t module = nullptr;
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4 = nullptr;
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
+    fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
     uint32_t cus = 0;
     uint32_t group_m = 8;  // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
 };
@@ -58,6 +59,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->quant8, k->module, "fe_fp8_quant");
     if (!c) c = fe_hip_module_get_function(&k->gemm8, k->module, "fe_gemm_fp8");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->gemm8c, k->module, "fe_gemm_fp8_codes");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8c, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->swiglu4, k->module, "fe_gemm_nvfp4_swiglu");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->swiglu4, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->swiglu_reduce4, k->module, "fe_gemm_nvfp4_swiglu_reduce");
@@ -292,11 +295,19 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     uint32_t group = kern->group_m == 0 || kern->group_m > tiles_m ? tiles_m : kern->group_m;  // lib.rs:148-151
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    // FP8 runs on the 8-bit matrix instruction over the codes of both operands, k tiles of 128 (FE_FP8_F16=1: the fp16
+    // expansion on the 16-bit instruction, k tiles of 64; same products, another order of the f32 sums)
+    const char *f16env = getenv("FE_FP8_F16");
+    const bool codes8 = l->fp8 && !(f16env && atoi(f16env) != 0);
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = ws->part.p;
     float scale = l->fp8 ? 1.0f : 0.0625f;  // what the fp16 expansions of the two operands carry (FP4_OPERAND_SCALE)
-    if (l->fp8) {
+    if (codes8) {
+        fe_devptr_t codes = ws->codes.p;
+        void *args8[] = {&y, &codes, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &full, &splits, &part};
+        FE_TRY(fe_hip_launch(kern->gemm8c, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args8));
+    } else if (l->fp8) {
         void *args8[] = {&y, &aq, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &full, &splits, &part};
         FE_TRY(fe_hip_launch(kern->gemm8, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args8));
     } else {

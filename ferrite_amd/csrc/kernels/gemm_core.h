@@ -228,6 +228,133 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
     __syncthreads();  // the LDS tiles are free for the epilogue
 }
 
+// The same loop for 8-bit operands (e4m3 codes on both sides) on v_mfma_f32_32x32x64_f8f6f4: a k tile is 128 codes
+// wide, so rows are again 128 bytes and tiles, swizzle, loads and LDS writes are those of gemm_mainloop; a lane's
+// operand of one MFMA is 32 consecutive codes of its row (two 16-byte chunks), the k tile is two MFMA steps of 64.
+// The k index inside an MFMA is a summation index only, and both operands are read with the same lane mapping.
+// a: codes [m][lda] (bytes). The producer's store writes 128 code bytes a row (no expansion).
+typedef int gm_i32x8 __attribute__((ext_vector_type(8)));
+template <class Producer>
+__device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, uint32_t lda, uint32_t m, uint32_t kt0,
+                                                 uint32_t ktiles, uint32_t m0, Producer& prod, unsigned char* lds,
+                                                 f32x16 (&acc)[4][4]) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+
+    const uint32_t a_chunk = tid & 7, a_row = tid >> 3;
+    uint32_t aoff[8];
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+        uint32_t row = m0 + a_row + 32 * j;
+        row = row < m ? row : m - 1;
+        aoff[j] = row * lda + a_chunk * 16;
+    }
+    const unsigned char* abytes = (const unsigned char*)a + kt0 * 128;
+    u32x4 areg[8];
+    auto load_a = [&](uint32_t kt, int j0, int j1) {
+        kt = kt < ktiles ? kt : ktiles - 1;
+        const unsigned char* ak = abytes + kt * 128;
+#pragma unroll
+        for (int j = j0; j < j1; j++) areg[j] = *(const u32x4*)(ak + aoff[j]);
+    };
+    auto load_b = [&](typename Producer::Raw& r, uint32_t kt, int half) {
+        prod.load(kt0 + (kt < ktiles ? kt : ktiles - 1), r, half);
+    };
+    const uint32_t a_st = gm_swz(a_row, a_chunk);
+    auto store_a = [&](unsigned char* st, int j0, int j1) {
+#pragma unroll
+        for (int j = j0; j < j1; j++) *(u32x4*)(st + a_st + 4096 * j) = areg[j];
+    };
+    // fragment addresses: row (lane & 31) of each 32-row piece, chunks 4 kk + 2 (lane >> 5) and the next one
+    const uint32_t fr = lane & 31, fc = lane >> 5;
+    uint32_t foff[2][2];
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) foff[kk][h] = gm_swz(fr, 4 * kk + 2 * fc + h);
+    const uint32_t fa_base = wm * 128 * 128, fb_base = GM_A_BYTES + wn * 128 * 128;
+    gm_i32x8 fa[2][4], fb[2][4];
+    auto read_one = [&](const unsigned char* p, int kk) {
+        u32x4 lo = *(const u32x4*)(p + foff[kk][0]), hi = *(const u32x4*)(p + foff[kk][1]);
+        return (gm_i32x8){(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+    };
+    auto read_frags = [&](int set, const unsigned char* st, int kk) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) fa[set][i] = read_one(st + fa_base + 4096 * i, kk);
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[set][j] = read_one(st + fb_base + 4096 * j, kk);
+    };
+    auto mfmas = [&](int set, int i0, int i1) {
+#pragma unroll
+        for (int i = i0; i < i1; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)  // formats 0, 0: e4m3 x e4m3; zero scale operands select the unscaled instruction
+                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    };
+
+    typename Producer::Raw braw;
+    load_b(braw, 0, 0);
+    load_b(braw, 0, 1);
+    load_a(0, 0, 8);
+#pragma unroll
+    for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
+    store_a(lds, 0, 8);
+    load_b(braw, 1, 0);
+    load_b(braw, 1, 1);
+    load_a(1, 0, 8);
+    __syncthreads();
+    read_frags(0, lds, 0);
+
+    // One k tile = two MFMA steps of 64 (16 MFMAs of 64 cycles each). Step 0: the weights of tile kt + 1 go to the other
+    // stage and are reloaded with tile kt + 2; step 1: the activations go out under its first 8 MFMAs, the barrier, then
+    // the first fragments of tile kt + 1 and the reload of the activation registers under the last 8.
+    for (uint32_t kt = 0; kt < ktiles; kt++) {
+        const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
+        unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
+        read_frags(1, cur, 1);
+        prod.store(braw, nxt + GM_A_BYTES, 0);
+        prod.store(braw, nxt + GM_A_BYTES, 1);
+        load_b(braw, kt + 2, 0);
+        load_b(braw, kt + 2, 1);
+        mfmas(0, 0, 4);
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        store_a(nxt, 0, 8);
+        mfmas(1, 0, 2);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        __syncthreads();
+        read_frags(0, nxt, 0);
+        load_a(kt + 2, 0, 8);
+        mfmas(1, 2, 4);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();  // the LDS tiles are free for the epilogue
+}
+
 // Hands the wavefront's 128 x 128 accumulators out row by row: 32 rows at a time pass through the wavefront's own LDS
 // slab (GM_EPI_SLAB bytes at lds + wave * GM_EPI_SLAB) so that 32 consecutive lanes hold 128 consecutive columns of one
 // row, 4 a lane. Both halves of the wavefront work on a row of their own. Four row pairs are in flight together:

@@ -460,6 +460,71 @@ extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8(uint16_t* c, co
     fp_gemm_body<Fp8Producer, false>(prod, out, aq, alpha, 1.0f, m, n, k, wk, part);
 }
 
+// The same linear on the 8-bit matrix instruction: activations are the quantizer's e4m3 codes [M][K], weights stay codes
+// in LDS, a k tile is 128 wide (two of the 64-wide weight tiles of the layout above). Same products (an e4m3 x e4m3
+// product is exact in f32) and f32 sums as fe_gemm_fp8, at twice the MFMA rate and half the LDS bytes per flop.
+struct Fp8CodeProducer {
+    const uint8_t* w[2];  // the two 128-row weight tiles + this thread's (row, chunk) offset
+    uint32_t w_skt, w_sr, st;
+    struct Raw {
+        u32x4 c[2][4];
+    };
+    static constexpr int kStoreValu = 0;
+    // thread t: 16-byte chunk t & 7 of rows (t >> 3) + 32 j of each 128-row half; chunks 0..3 come from 64-wide weight
+    // tile 2 kt, chunks 4..7 from 2 kt + 1
+    __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            if (b != half) continue;
+            const uint8_t* p = w[b] + (size_t)(2 * kt) * w_skt;
+#pragma unroll
+            for (int j = 0; j < 4; j++) r.c[b][j] = *(const u32x4*)(p + (size_t)(32 * j) * w_sr);
+        }
+    }
+    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
+#pragma unroll
+        for (int b = 0; b < 2; b++) {
+            if (b != part) continue;
+#pragma unroll
+            for (int j = 0; j < 4; j++) *(u32x4*)(Bs + 16384 * b + st + 4096 * j) = r.c[b][j];
+        }
+    }
+};
+
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_codes(uint16_t* c, const uint8_t* aq, const uint8_t* w,
+                                                                       const float* alpha, const uint16_t* res, uint32_t m,
+                                                                       uint32_t n, uint32_t k, uint32_t ldc, uint32_t group_m,
+                                                                       uint32_t w_snt, uint32_t w_skt, uint32_t w_sr,
+                                                                       uint32_t full_tiles, uint32_t splits, float* part) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t nts = n / 128, tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / 128, full_tiles, splits);
+    const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
+    Fp8CodeProducer prod;
+    const uint32_t chunk = tid & 7, row = tid >> 3;
+#pragma unroll
+    for (int b = 0; b < 2; b++) {
+        uint32_t nt = 2 * wk.tn + b;
+        nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program copies its first tile twice
+        prod.w[b] = w + (size_t)nt * w_snt + (size_t)(chunk >> 2) * w_skt + (size_t)row * w_sr + (chunk & 3) * 16;
+    }
+    prod.w_skt = w_skt, prod.w_sr = w_sr, prod.st = gm_swz(row, chunk);
+    f32x16 acc[4][4];
+    gemm_mainloop_f8(aq, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
+    if (wk.partial) {
+        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
+        return;
+    }
+    const uint32_t colb = n0 + wn * 128;
+    if (colb >= n) return;
+    const uint32_t col = colb + 4 * (tid & 31);
+    const f32x4 al = *(const f32x4*)(alpha + col);
+    FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
+    gemm_epilogue(
+        acc, lds, [](float (&)[4][4], uint32_t) {},
+        [&](uint32_t r, uint32_t l32, float (&v)[4]) { fp_store_piece<false>(out, v, al, l32, m0 + wm * 128 + r, m, col, n); });
+}
+
 // ---- GEMV (1..16 rows) -------------------------------------------------------------------------------------------------
 
 #define FP4_GEMV_RG 8  // 16-row groups of a 128-row weight tile
