@@ -293,6 +293,10 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_fp4_linear_gemm", "operand of 4 GB or more");
     const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
     uint32_t group = kern->group_m == 0 || kern->group_m > tiles_m ? tiles_m : kern->group_m;  // lib.rs:148-151
+    // FP8 codes: the weights are the larger operand from n >= m on, and at the 8-bit instruction's rate their traffic
+    // shows: column tiles are dealt to the XCDs (gemm_raster with group 0), each weight panel through one L2
+    if (l->fp8 && n >= m) group = 0;
+    if (const char *e = getenv("FE_FP4_XCD")) group = atoi(e) ? 0 : group ? group : tiles_m;
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
     // FP8 runs on the 8-bit matrix instruction over the codes of both operands, k tiles of 128 (FE_FP8_F16=1: the fp16

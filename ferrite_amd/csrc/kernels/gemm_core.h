@@ -284,18 +284,24 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
         u32x4 lo = *(const u32x4*)(p + foff[kk][0]), hi = *(const u32x4*)(p + foff[kk][1]);
         return (gm_i32x8){(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
     };
-    auto read_frags = [&](int set, const unsigned char* st, int kk) {
+    auto read_a = [&](int set, const unsigned char* st, int i0, int i1) {  // step kk = set
 #pragma unroll
-        for (int i = 0; i < 4; i++) fa[set][i] = read_one(st + fa_base + 4096 * i, kk);
-#pragma unroll
-        for (int j = 0; j < 4; j++) fb[set][j] = read_one(st + fb_base + 4096 * j, kk);
+        for (int i = i0; i < i1; i++) fa[set][i] = read_one(st + fa_base + 4096 * i, set);
     };
-    auto mfmas = [&](int set, int i0, int i1) {
+    auto read_b = [&](int set, const unsigned char* st, int j0, int j1) {
 #pragma unroll
-        for (int i = i0; i < i1; i++)
+        for (int j = j0; j < j1; j++) fb[set][j] = read_one(st + fb_base + 4096 * j, set);
+    };
+    // 8 MFMAs: rows i0, i0 + 1 of the wavefront's 4 x 4 pieces, first against columns 0, 1, then 2, 3 (whose weights
+    // fragments may still be on their way when the first four issue)
+    auto mfmas = [&](int set, int i0) {
 #pragma unroll
-            for (int j = 0; j < 4; j++)  // formats 0, 0: e4m3 x e4m3; zero scale operands select the unscaled instruction
-                acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0, 0, 0, 0);
+        for (int jh = 0; jh < 2; jh++)
+#pragma unroll
+            for (int i = i0; i < i0 + 2; i++)
+#pragma unroll
+                for (int j = 2 * jh; j < 2 * jh + 2; j++)  // formats 0, 0: e4m3 x e4m3; zero scale operands select the unscaled instruction
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0, 0, 0, 0);
     };
 
     typename Producer::Raw braw;
@@ -309,44 +315,65 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
     load_b(braw, 1, 1);
     load_a(1, 0, 8);
     __syncthreads();
-    read_frags(0, lds, 0);
+    read_a(0, lds, 0, 2);
+    read_b(0, lds, 0, 2);
 
-    // One k tile = two MFMA steps of 64 (16 MFMAs of 64 cycles each). Step 0: the weights of tile kt + 1 go to the other
-    // stage and are reloaded with tile kt + 2; step 1: the activations go out under its first 8 MFMAs, the barrier, then
-    // the first fragments of tile kt + 1 and the reload of the activation registers under the last 8.
+    // One k tile = two MFMA steps of 64, four slices of 8 MFMAs (64 cycles each), shaped like gemm_mainloop's: every
+    // slice reads 8 chunks of fragments for the MFMAs half a slice to one slice ahead; the weights of tile kt + 1 go to
+    // the other stage in slices 0 and 1 and are reloaded with tile kt + 2; the activations go out in slice 2, before the
+    // barrier; slice 3 starts on the fragments of tile kt + 1 and reloads the activation registers.
     for (uint32_t kt = 0; kt < ktiles; kt++) {
         const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
         unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
-        read_frags(1, cur, 1);
+        // slice 0: step 0, rows 0, 1
+        read_b(0, cur, 2, 4);
+        read_a(0, cur, 2, 4);
         prod.store(braw, nxt + GM_A_BYTES, 0);
+        mfmas(0, 0);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // slice 1: step 0, rows 2, 3
+        read_a(1, cur, 0, 2);
+        read_b(1, cur, 0, 2);
         prod.store(braw, nxt + GM_A_BYTES, 1);
         load_b(braw, kt + 2, 0);
         load_b(braw, kt + 2, 1);
-        mfmas(0, 0, 4);
+        mfmas(0, 2);
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
+        for (int i = 0; i < 8; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
+        // slice 2: step 1, rows 0, 1
+        read_b(1, cur, 2, 4);
+        read_a(1, cur, 2, 4);
         store_a(nxt, 0, 8);
-        mfmas(1, 0, 2);
+        mfmas(1, 0);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
-        read_frags(0, nxt, 0);
+        // slice 3: step 1, rows 2, 3, with the first fragments of tile kt + 1
+        read_a(0, nxt, 0, 2);
+        read_b(0, nxt, 0, 2);
         load_a(kt + 2, 0, 8);
-        mfmas(1, 2, 4);
+        mfmas(1, 2);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
