@@ -300,6 +300,18 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     rot_ms = ev.ms(a2, b2) / reps
     res["exl3_b4_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                                  "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "rot_in_ms": round(rot_ms, 4)}
+    # the same with the weights decoded once and kept with the linear (2 bytes a weight): no decode launch per call
+    lin.keep_decoded()
+    lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
+    a3, b3 = ev.new(), ev.new()
+    ev.record(a3, stream)
+    for _ in range(reps):
+        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
+    ev.record(b3, stream)
+    ms = ev.ms(a3, b3) / reps
+    res["exl3_b4_5120x17408_decoded_kept"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                                              "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                                              "kept_bytes": ((n // 128 + 1) // 2) * 256 * k * 2}
     del lin, ws, y
     # NVFP4
     fk = fp4.Kernels.load()

@@ -57,6 +57,7 @@ struct fe_exl3_linear {
     uint32_t programs = 0;  // grid of the streamed GEMV (plan.ver == 2)
     fe_exl3_view view{};
     FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
+    FeBuf hat;                // decoded fp16 tiles kept with the linear (fe_exl3_linear_keep_decoded), else empty
     const fe_exl3_kernels *kern = nullptr;
 };
 
@@ -340,6 +341,18 @@ int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *
     return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
 }
 
+// trellis -> fp16 tiles (exl3_hat_tiles_b*) into `hat`, hat_bytes(l) bytes
+static int launch_decode(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t hat) {
+    const fe_exl3_kernels *kern = l->kern;
+    uint32_t k = l->k, stride_k, stride_nb;
+    view_strides(l->view, &stride_k, &stride_nb);
+    const uint32_t ktiles = k / 64, nbs = l->n / 128;
+    const uint32_t gy = std::min(ktiles, std::max(1u, (8 * std::max(kern->cus, 1u) + nbs - 1) / nbs));
+    fe_devptr_t tr = l->view.trellis;
+    void *dargs[] = {&tr, &hat, &k, &stride_k, &stride_nb};
+    return fe_hip_launch(kern->hat_tiles[bits_slot(l->bits)], nbs, gy, 1, 256, 1, 1, 0, s, dargs);
+}
+
 static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
                        const fe_exl3_workspace *ws) {
     const fe_exl3_kernels *kern = l->kern;
@@ -352,12 +365,10 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = g.full, splits = g.splits;
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
-    if (rows >= hat_rows() && ws->hat.bytes >= hat_bytes(l)) {
-        fe_devptr_t hat = ws->hat.p;
-        const uint32_t ktiles = k / 64, nbs = n / 128;
-        const uint32_t gy = std::min(ktiles, std::max(1u, (8 * std::max(kern->cus, 1u) + nbs - 1) / nbs));
-        void *dargs[] = {&tr, &hat, &k, &stride_k, &stride_nb};
-        FE_TRY(fe_hip_launch(kern->hat_tiles[bits_slot(l->bits)], nbs, gy, 1, 256, 1, 1, 0, s, dargs));
+    const bool kept = l->hat.bytes != 0;  // decoded once and kept: any row count above the GEMV's runs over it
+    if (kept || (rows >= hat_rows() && ws->hat.bytes >= hat_bytes(l))) {
+        fe_devptr_t hat = kept ? l->hat.p : ws->hat.p;
+        if (!kept) FE_TRY(launch_decode(l, s, hat));
         group = 0;  // the raster that deals column tiles to the XCDs: each decoded weight panel goes through one L2
         void *args[] = {&xh, &hat, &svh, &y, &n, &k, &rows, &mode, &group, &full, &splits, &part};
         FE_TRY(fe_hip_launch(kern->gemm_hat, g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
@@ -436,6 +447,19 @@ static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     fe_devptr_t suh = l->view.suh;
     void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk, &x, &x_f32, &suh, &xh};
     return fe_hip_launch(l->kern->gemv[bits_slot(l->bits)][rg - 1], n / 128 * sk, 1, 1, 256, 1, 1, lds, s, args);
+}
+
+int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on) {
+    if (!l) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_keep_decoded", "null linear");
+    if (!on) {
+        l->hat.release();
+        return 0;
+    }
+    if (l->hat.bytes) return 0;
+    FE_TRY(l->hat.zeroed(hat_bytes(l)));  // zeroed: the unused half of the last tile of an odd count of column blocks is read
+    int c = launch_decode(l, s, l->hat.p);
+    if (c) l->hat.release();
+    return c;
 }
 
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }

@@ -262,6 +262,11 @@ class Linear:
         check(_lib.lib().fe_exl3_linear_forward(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), y.data_ptr(),
                                                 int(y_dtype), rows, ws.h))
 
+    def keep_decoded(self, on: bool = True, stream=None):
+        """Decode the trellis once into fp16 tiles kept with the linear (2 bytes a weight): calls with more than 64 rows
+        then run the GEMM over them without decoding."""
+        check(_lib.lib().fe_exl3_linear_keep_decoded(self.h, _stream(stream), int(on)))
+
     def forward_is_one_launch(self, rows: int) -> bool:
         """Whether forward() with this many rows is the decode GEMV alone, rotating its own input."""
         return bool(_lib.lib().fe_exl3_linear_forward_is_one_launch(self.h, rows))

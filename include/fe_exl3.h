@@ -81,6 +81,12 @@ int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t 
  * The workspace's xh holds the rotated input afterwards, as after rotate_input. */
 int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
                            fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws);
+/* Prefill over weights decoded once: decodes the trellis into fp16 tiles (2 bytes a weight, in the rotated basis) that
+ * stay with the linear, and from then on every call with more than 64 rows runs the GEMM over them without decoding
+ * (same bits as the decoding GEMM for whole tiles). The role of the reference's dequantized prompt weights
+ * (reconstruct_bf16 into Linear.w, crates/fe-model/src/model.rs:262-266), for callers that have the memory: 178 MB for
+ * 5120 x 17408. on == 0 frees them. Stream-ordered; the first GEMM may follow on the same stream. */
+int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on);
 /* 1 if forward() with this many rows is a single launch (the decode GEMV rotates its own input: every program's K range
  * is whole 128-element Hadamard blocks), 0 if it is rotate_input followed by gemv_rotated. Same bits either way. */
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows);

@@ -421,3 +421,36 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     o = to_oracle(oracle, t)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
+
+
+def test_prefill_over_kept_decoded_weights(env, oracle, monkeypatch):
+    """keep_decoded: the fp16 tiles stay with the linear, every call above 64 rows runs the GEMM over them (no decode
+    launch, any workspace). Whole tiles have the bits of the decoding GEMM; decode-sized calls are untouched."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    m = 300
+    t = synth.exl3_tensor(1024, 384, 4, 123)
+    xd = dev_u16(torch, synth.activations(m, t.k, 4, outliers=True))
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 256)
+    ws = exl3.Workspace([lin], m)  # not created for the decoded form
+
+    def run(rows):
+        y = torch.full((m + 1, t.n), float("nan"), dtype=torch.float32, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, rows, ws)
+        torch.cuda.synchronize()
+        out = y.cpu().numpy()
+        assert np.isnan(out[rows:]).all()
+        return out[:rows]
+
+    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    before = {rows: run(rows) for rows in (1, 16, 64, 65, 300)}
+    lin.keep_decoded()
+    lin.keep_decoded()  # a second call keeps what is there
+    for rows, want in before.items():
+        assert np.array_equal(run(rows).view(np.uint32), want.view(np.uint32)), rows
+    monkeypatch.delenv("FE_GEMM_SPLITS")
+    cut = run(300)  # a last round cut along K: other tiles are the cut ones, sums in another order
+    rms = np.sqrt((before[300].astype(np.float64) ** 2).mean())
+    assert np.abs(cut.astype(np.float64) - before[300]).max() / rms < 1e-4
+    lin.keep_decoded(False)
+    assert np.array_equal(run(300).view(np.uint32), run(300).view(np.uint32))
