@@ -223,6 +223,7 @@ def main():
     }
 
     out["graph_replay"] = graph_replay(lib, _lib.check, ev, exl3, linears, ws, total_bytes, args.steps, args.warmup)
+    out["rows_sweep_b4"] = rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears)
     if not args.no_prefill:
         out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
     print(json.dumps(out))
@@ -248,6 +249,32 @@ def traffic_pass(torch, np, exl3, synth):
     torch.cuda.synchronize()
     print(json.dumps({"exl3_probe_v4_reads_KiB": lin.weight_bytes() / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
                       "roofline_kernel": "exl3_gemv_b4_r1", "algorithmic_KiB": lin.weight_bytes() / 1024}))
+
+
+def rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears, reps=20):
+    """The 4-bit linears at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts): microseconds per forward,
+    launched back to back, cycling gate, up, down so that no weight is served from cache. Not part of `value`."""
+    four = [(name, lin) for name, bits, lin, x, y in linears if bits == 4]
+    res = {}
+    for m in (1, 4, 8, 16):
+        ws = exl3.Workspace([lin for _, lin in four], m)
+        io = []
+        for name, lin in four:
+            x = torch.from_numpy(synth.activations(m, lin.k, SEED).view(np.int16)).cuda()
+            io.append((lin, x, torch.zeros((m, lin.n), dtype=torch.bfloat16, device="cuda")))
+        for lin, x, y in io:
+            lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, ws, stream=stream)
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        for _ in range(reps):
+            for lin, x, y in io:
+                lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, ws, stream=stream)
+        ev.record(b, stream)
+        us = ev.ms(a, b) * 1e3 / (reps * len(io))
+        nbytes = sum(lin.weight_bytes() for lin, _, _ in io) / len(io)
+        res[f"m{m}"] = {"us_per_forward": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                        "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+    return res
 
 
 def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):

@@ -335,16 +335,18 @@ def test_tuner_returns_a_fitting_plan(env):
 @pytest.mark.parametrize("k,sk,fits", [(1024, 1, True), (1024, 4, True), (2048, 16, True), (1024, 8, True), (1024, 16, False),
                                        (1280, 2, True), (1280, 4, False)])
 def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, monkeypatch):
-    """forward() for up to 64 rows is one launch when every program's K range is whole 128-element blocks (the GEMV
-    rotates its own input and leaves it in the workspace), two launches otherwise. Both give the same bits, in y and in
-    the workspace's rotated input, for bf16 and f32 inputs."""
+    """forward() for few rows is one launch when every program's K range is whole 128-element blocks (the GEMV rotates
+    its own input and leaves it in the workspace), two launches otherwise. Both give the same bits, in y and in the
+    workspace's rotated input, for bf16 and f32 inputs."""
     torch, exl3, kern = env
     from ferrite_amd import _lib, synth
     from ferrite_amd._lib import check
     assert ((k // 64 // sk) % 2 == 0) == fits
     t = synth.exl3_tensor(k, 384, 4, 70 + sk)
     lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(sk=sk, wk=1, ver=1, occ=2))
-    assert lin.forward_is_one_launch(1) == fits and lin.forward_is_one_launch(64) == fits and not lin.forward_is_one_launch(65)
+    # one launch when the K ranges fit and a program's share of the rotation stays small (rows x 128-blocks <= 32)
+    for rows in (1, 4, 7, 16, 33, 64, 65):
+        assert lin.forward_is_one_launch(rows) == (fits and rows <= 64 and rows * (k // 128 // sk) <= 32), rows
     ws = exl3.Workspace([lin], 64)
     xb = synth.activations(64, k, 8, outliers=True)
     xd = dev_u16(torch, xb)
