@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <string>
 #include <vector>
 
@@ -16,6 +17,8 @@ namespace {
 constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
 constexpr uint32_t kHatRows = 513;          // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
 constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
+constexpr uint32_t kGroupMax = 4;           // FE_EXL3_GROUP_MAX: linears of one grouped launch
+constexpr uint32_t kGroupRows = 16;         // rows of a grouped launch (one row group)
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
@@ -38,10 +41,11 @@ int bits_slot(uint32_t bits) {
 struct fe_exl3_kernels {
     fe_module_t module = nullptr;
     fe_function_t recon_hat_f32 = nullptr, recon_hat_f16 = nullptr, had_rows = nullptr, had_cols_bf16 = nullptr;
-    fe_function_t rot_in = nullptr, probe_v4 = nullptr;
+    fe_function_t rot_in = nullptr, rot_in_group = nullptr, probe_v4 = nullptr;
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
     fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
+    fe_function_t gemv_group[6] = {};                             // 1..16 rows, several linears of one input
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     fe_function_t gemm_reduce = nullptr;
@@ -100,6 +104,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     get(&k->had_rows, "exl3_had_rows");
     get(&k->had_cols_bf16, "exl3_had_cols_bf16");
     get(&k->rot_in, "exl3_rot_in");
+    get(&k->rot_in_group, "exl3_rot_in_group");
     get(&k->probe_v4, "exl3_probe_v4");
     for (int b = 3; b <= 5; b++) {
         char nm[64];
@@ -115,6 +120,9 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         }
         snprintf(nm, sizeof nm, "exl3_gemv_stream_b%d", kBits[i]);
         get(&k->gemv_stream[i], nm);
+        snprintf(nm, sizeof nm, "exl3_gemv_group_b%d", kBits[i]);
+        get(&k->gemv_group[i], nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv_group[i], 64 * 1024);
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
@@ -284,8 +292,11 @@ static size_t hat_bytes(const fe_exl3_linear *l) { return (size_t)((l->n / 128 +
 int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows) {
     if (!out || (count && !linears) || !max_rows) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_create", "bad argument");
     size_t max_k = 128, max_z = 0, max_zs = 0, max_nb = 1, max_hat = 0;
+    std::vector<size_t> zs, nbs;  // per linear, for the grouped launch: room for the kGroupMax largest together
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
+        zs.push_back(l->plan.ver == 2 ? 0 : (size_t)l->plan.sk * l->n);
+        nbs.push_back(l->n / 128);
         max_hat = std::max(max_hat, hat_bytes(l));
         max_k = std::max<size_t>(max_k, l->k);
         if (l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
@@ -294,9 +305,18 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     }
     auto *ws = new fe_exl3_workspace;
     ws->max_rows = max_rows, ws->max_k = (uint32_t)max_k;
+    auto top = [](std::vector<size_t> &v) {
+        std::sort(v.begin(), v.end(), std::greater<size_t>());
+        size_t t = 0;
+        for (size_t i = 0; i < v.size() && i < kGroupMax; i++) t += v[i];
+        return t;
+    };
+    const size_t group_z = top(zs), group_nb = top(nbs);
     ws->z_len = std::max<size_t>(std::max(max_z * std::min(max_rows, kMaxRowsPerPass), max_zs * std::min(max_rows, kStreamRows)), 4);
-    ws->counters_len = (size_t)((max_rows + 7) / 8) * max_nb;
-    int c = ws->xh.alloc((size_t)max_rows * max_k * 2);
+    ws->z_len = std::max(ws->z_len, group_z * std::min(max_rows, kGroupRows));
+    ws->counters_len = std::max((size_t)((max_rows + 7) / 8) * max_nb, group_nb);
+    // (rotated inputs: one linear's at max_rows, or a group's at up to kGroupRows rows each)
+    int c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * std::min(max_rows, kGroupRows)) * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
     int cus = 0;
@@ -385,6 +405,7 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
 // fused_rotation_fits first); otherwise it reads xh.
 static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
                        const fe_exl3_workspace *ws, fe_devptr_t x, uint32_t x_f32);
+static uint32_t gemv_chunk(uint32_t rows, uint32_t steps);
 
 // The split-K kernel can rotate its own input when every program's K range is whole 128-element blocks.
 static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
@@ -395,7 +416,9 @@ static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
     // every column block repeats the rotation of its K range: (row, 128-block) pairs a program, 8 at a time. Measured on
     // 5120 x 17408 (8 blocks a program): one launch wins up to 4 rows (19.9 against 22.3 us at 1 row), the separate
     // rotation from 8 rows on (25.2 against 23.7 us).
-    return rows * (l->k / 128 / p.sk) <= 32;
+    uint32_t pairs = 32;
+    if (const char *t = getenv("FE_EXL3_FUSED_ROT_PAIRS")) pairs = (uint32_t)atoi(t);
+    return rows * (l->k / 128 / p.sk) <= pairs;
 }
 
 int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
@@ -440,10 +463,7 @@ static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     }
     const uint32_t rg = (rows + 15) / 16;
     const uint32_t steps = l->k / 64 / p.sk;
-    // staged input chunk: as many load steps as the LDS budget holds for `rows` rows, a multiple of 4
-    uint32_t chunk = (kLdsBudget / rows - 16) / 128 / 4 * 4;
-    chunk = std::max(chunk, 4u);
-    chunk = std::min(chunk, (steps + 3) / 4 * 4);
+    uint32_t chunk = gemv_chunk(rows, steps);
     const uint32_t lds = std::max(rows * (chunk * 128 + 16), rows * kRedPitch * 4);
     uint32_t n = l->n, k = l->k, sk = p.sk, mode = (uint32_t)y_dtype, stride_k, stride_nb;
     view_strides(l->view, &stride_k, &stride_nb);
@@ -482,6 +502,96 @@ int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern,
     }
     FE_TRY(fe_exl3_linear_rotate_input(l, kern, s, x, x_dtype, rows, ws));
     return fe_exl3_linear_gemv_rotated(l, s, ws->xh.p, y, y_dtype, rows, ws);
+}
+
+// mirrors GemvGroup of k_exl3.hip
+struct GemvGroupArgs {
+    uint32_t count, first[kGroupMax + 1];
+    struct Member {
+        fe_devptr_t trellis, svh, suh, xh, y, z, counters;
+        uint32_t n, sk, stride_k, stride_nb, chunk, pad;
+    } m[kGroupMax];
+};
+struct RotGroupArgs {  // RotGroup
+    fe_devptr_t suh[kGroupMax], xh[kGroupMax];
+};
+
+static uint32_t gemv_chunk(uint32_t rows, uint32_t steps) {
+    // staged input chunk: as many load steps as the LDS budget holds for `rows` rows, a multiple of 4
+    uint32_t chunk = (kLdsBudget / rows - 16) / 128 / 4 * 4;
+    chunk = std::max(chunk, 4u);
+    return std::min(chunk, (steps + 3) / 4 * 4);
+}
+
+// The grouped launch: the same input, width and kernel, and room in the workspace for every member's partials (and,
+// where the members do not rotate their own input, rotated inputs) side by side. *fused: the GEMV rotates its own input.
+static bool group_fits(const fe_exl3_linear *const *ls, size_t count, uint32_t rows, const fe_exl3_workspace *ws, bool *fused) {
+    const char *e = getenv("FE_EXL3_NO_GROUP");  // read per call: tests compare both paths in one process
+    if (e && atoi(e) != 0) return false;
+    if (!ls || !ws || count < 2 || count > kGroupMax || rows < 1 || rows > kGroupRows || rows > ws->max_rows) return false;
+    size_t z = 0, nb = 0;
+    bool f = true;
+    for (size_t i = 0; i < count; i++) {
+        const fe_exl3_linear *l = ls[i];
+        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.ver == 2) return false;
+        f = f && fused_rotation_fits(l, rows);
+        z += (size_t)l->plan.sk * rows * l->n;
+        nb += l->n / 128;
+    }
+    if (!f && count * (size_t)rows * ls[0]->k * 2 > ws->xh.bytes) return false;
+    if (fused) *fused = f;
+    return z <= ws->z_len && nb <= ws->counters_len && ls[0]->k <= ws->max_k;
+}
+
+int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_t count, uint32_t rows,
+                                          const fe_exl3_workspace *ws) {
+    bool fused = false;
+    if (!group_fits(ls, count, rows, ws, &fused)) return 0;
+    return fused ? 1 : 2;
+}
+
+int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, const fe_exl3_kernels *kern, fe_stream_t s,
+                                 fe_devptr_t x, int x_dtype, const fe_devptr_t *ys, int y_dtype, uint32_t rows,
+                                 const fe_exl3_workspace *ws) {
+    if (!ls || !ys || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null argument");
+    bool fused = false;
+    if (!group_fits(ls, count, rows, ws, &fused)) {  // member by member: the same bits, more launches
+        for (size_t i = 0; i < count; i++) FE_TRY(fe_exl3_linear_forward(ls[i], kern, s, x, x_dtype, ys[i], y_dtype, rows, ws));
+        return 0;
+    }
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "x is bf16 or f32");
+    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "bad y dtype");
+    GemvGroupArgs g{};
+    RotGroupArgs r{};
+    g.count = (uint32_t)count;
+    uint32_t lds = 0, programs = 0;
+    size_t z_at = 0, cnt_at = 0;
+    for (size_t i = 0; i < count; i++) {
+        const fe_exl3_linear *l = ls[i];
+        if (!ys[i]) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null output");
+        GemvGroupArgs::Member &m = g.m[i];
+        m.trellis = l->view.trellis, m.svh = l->view.svh, m.suh = l->view.suh, m.y = ys[i];
+        m.xh = ws->xh.p + i * (size_t)rows * l->k * 2;
+        r.suh[i] = m.suh, r.xh[i] = m.xh;
+        m.z = ws->z.p + z_at * 4, m.counters = ws->counters.p + cnt_at * 4;
+        m.n = l->n, m.sk = l->plan.sk;
+        view_strides(l->view, &m.stride_k, &m.stride_nb);
+        m.chunk = gemv_chunk(rows, l->k / 64 / m.sk);
+        lds = std::max(lds, std::max(rows * (m.chunk * 128 + 16), rows * kRedPitch * 4));
+        g.first[i] = programs;
+        programs += l->n / 128 * m.sk;
+        z_at += (size_t)m.sk * rows * l->n, cnt_at += l->n / 128;
+    }
+    for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
+    uint32_t x_f32 = (uint32_t)x_dtype & 1, k = ls[0]->k, mode = (uint32_t)y_dtype;
+    if (!fused) {  // one launch rotates the input for every member, and the GEMV reads the members' rotated inputs
+        void *rargs[] = {&r, &x, &x_f32, &k};
+        FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
+        x = 0;
+    }
+    void *args[] = {&g, &x, &x_f32, &k, &rows, &mode};
+    return fe_hip_launch(kern->gemv_group[bits_slot(ls[0]->bits)], programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 
 int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out) {

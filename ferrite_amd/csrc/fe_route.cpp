@@ -277,16 +277,35 @@ static int proj_forward(const fe_route_proj *p, const fe_route_ctx *c, uint32_t 
         off = (size_t)m * pn;
         first = p->cover;
     }
-    for (size_t i = first; i < p->lins.size(); i++) {
-        const fe_route_linear *l = p->lins[i].first;
-        const fe_devptr_t y = out + off * 2;
-        FE_TRY(linear_forward(l, c, dec, y, l->n, x, lda, m, 0));
-        uint32_t col = 0;
-        for (uint32_t w : p->lins[i].second) {
-            push(y + (size_t)col * 2, l->n);
-            col += w;
+    for (size_t i = first; i < p->lins.size();) {
+        // Trellis linears of this input, for a batch the GEMV takes whole: one grouped launch for up to four of them
+        // (the bits of each linear's own forward). The reference runs them one after the other (model.rs:384-392).
+        size_t j = i;
+        if (m <= FE_X3_ROWS && c->x3())
+            while (j < p->lins.size() && j - i < 4 && p->lins[j].first->q && p->lins[j].first->k == lda) j++;
+        if (j - i >= 2) {
+            const fe_exl3_linear *qs[4];
+            fe_devptr_t ys[4];
+            size_t o = off;
+            for (size_t t = i; t < j; t++) {
+                qs[t - i] = p->lins[t].first->q, ys[t - i] = out + o * 2;
+                o += (size_t)m * p->lins[t].first->n;
+            }
+            FE_TRY(fe_exl3_linear_forward_group(qs, j - i, c->xk, c->s, x, FE_DTYPE_BF16, ys, FE_DTYPE_BF16, m, c->xws));
+        } else {
+            j = i + 1;
+            FE_TRY(linear_forward(p->lins[i].first, c, dec, out + off * 2, p->lins[i].first->n, x, lda, m, 0));
         }
-        off += (size_t)m * l->n;
+        for (; i < j; i++) {
+            const fe_route_linear *l = p->lins[i].first;
+            const fe_devptr_t y = out + off * 2;
+            uint32_t col = 0;
+            for (uint32_t w : p->lins[i].second) {
+                push(y + (size_t)col * 2, l->n);
+                col += w;
+            }
+            off += (size_t)m * l->n;
+        }
     }
     if (parts_n) *parts_n = np;
     if (np > parts_cap && (part_ptr || part_ld)) return fe_set_error(FE_ERR_ARG, fn, "more parts than the caller made room for");

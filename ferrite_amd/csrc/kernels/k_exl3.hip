@@ -187,8 +187,7 @@ __device__ __forceinline__ u32x2 rot_block(const void* x, uint32_t x_f32, const 
 
 // xh[row][k] = fp16(H(x * suh) / sqrt(128)), x bf16 (x_f32 = 0) or f32. grid (ceil(k / 512), rows), 128 threads: each
 // half wavefront one 128-element block, 4 elements a lane. (kernels/k-exl3/src/gemv.rs:147-170)
-extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_f32, const uint16_t* suh,
-                                                               uint16_t* xh, uint32_t k) {
+__device__ __forceinline__ void rot_in_body(const void* x, uint32_t x_f32, const uint16_t* suh, uint16_t* xh, uint32_t k) {
     uint32_t l32 = threadIdx.x & 31;
     uint32_t blk = blockIdx.x * 4 + threadIdx.x / 32;
     bool live = blk * 128 < k;
@@ -196,6 +195,21 @@ extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uin
     size_t at = (size_t)blockIdx.y * k + c;
     u32x2 o = rot_block(x, x_f32, suh, at, c, l32);
     if (live) *(u32x2*)(xh + at) = o;
+}
+extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_f32, const uint16_t* suh,
+                                                               uint16_t* xh, uint32_t k) {
+    rot_in_body(x, x_f32, suh, xh, k);
+}
+
+#define FE_EXL3_GROUP_MAX 4  // linears of one grouped launch
+
+// The same input rotated for several linears (each by its own suh into its own xh): grid (ceil(k / 512), rows, members).
+struct RotGroup {
+    const uint16_t* suh[FE_EXL3_GROUP_MAX];
+    uint16_t* xh[FE_EXL3_GROUP_MAX];
+};
+extern "C" __global__ __launch_bounds__(128) void exl3_rot_in_group(RotGroup g, const void* x, uint32_t x_f32, uint32_t k) {
+    rot_in_body(x, x_f32, g.suh[blockIdx.z], g.xh[blockIdx.z], k);
 }
 
 // ---- decode GEMV -----------------------------------------------------------------------------------------------------
@@ -349,7 +363,8 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
                                           const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
                                           uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode,
                                           uint32_t stride_k, uint32_t stride_nb, uint32_t chunk, const void* x,
-                                          uint32_t x_f32, const uint16_t* __restrict__ suh, uint16_t* xh_out) {
+                                          uint32_t x_f32, const uint16_t* __restrict__ suh, uint16_t* xh_out,
+                                          uint32_t program) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
     constexpr uint32_t tw = 8 * BITS;
@@ -357,7 +372,7 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     constexpr int GROUP = 16;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
-    const uint32_t nbs = n / 128, nb = blockIdx.x % nbs, split = blockIdx.x / nbs;
+    const uint32_t nbs = n / 128, nb = program % nbs, split = program / nbs;
     const uint32_t per_split = (k / 16) / sk;  // k steps of this program, a multiple of 4
     const uint32_t kt0 = split * per_split;
     const uint32_t col0 = nb * 128;
@@ -424,7 +439,7 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
             while (p < total) {
                 u32x2 o = rot_finish(rot_raw, x_f32, rot_l32);
                 *(u32x2*)(lds + off) = o;
-                if (nb == 0) *(u32x2*)(xh_out + at) = o;
+                if (nb == 0 && xh_out) *(u32x2*)(xh_out + at) = o;
                 p += 8;
                 if (p < total) {
                     rot_at(c0, nblk, p, at, c, off);
@@ -557,15 +572,48 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
         uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb,       \
         uint32_t chunk, const void* x, uint32_t x_f32, const uint16_t* suh, uint16_t* xh_out) {                        \
         gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk, x,     \
-                            x_f32, suh, xh_out);                                                                      \
+                            x_f32, suh, xh_out, blockIdx.x);                                                          \
     }
 #define GEMV_FAMILY(BITS) GEMV_KERNEL(BITS, 1) GEMV_KERNEL(BITS, 2) GEMV_KERNEL(BITS, 3) GEMV_KERNEL(BITS, 4)
+
+// Several linears of one input in one launch (the projections a model applies to the same activations: q, k, v; gate,
+// up): the programs of member i are first[i] .. first[i + 1] - 1, each exactly the program of the member's own launch
+// (same split, same sums, same bits), rotating the input by the member's own suh (x != nullptr) or reading the member's
+// rotated input xh (exl3_rot_in_group). The launches' start-up and tails overlap and the members' programs fill each
+// other's gaps on the CUs. 1..16 rows.
+struct GemvGroup {
+    uint32_t count, first[FE_EXL3_GROUP_MAX + 1];
+    struct Member {
+        const uint32_t* trellis;
+        const uint16_t *svh, *suh, *xh;
+        void* y;
+        float* z;
+        uint32_t* counters;
+        uint32_t n, sk, stride_k, stride_nb, chunk, pad;
+    } m[FE_EXL3_GROUP_MAX];
+};
+#define GEMV_GROUP_KERNEL(BITS)                                                                                        \
+    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_group_b##BITS(GemvGroup g, const void* x,           \
+                                                                               uint32_t x_f32, uint32_t k, uint32_t m, \
+                                                                               uint32_t y_mode) {                      \
+        uint32_t i = 0;                                                                                                \
+        while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) i++;                                                   \
+        const GemvGroup::Member& mb = g.m[i];                                                                          \
+        gemv_body<BITS, 1>(mb.xh, mb.trellis, mb.svh, mb.y, mb.z, mb.counters, mb.n, k, m, mb.sk, y_mode,            \
+                           mb.stride_k, mb.stride_nb, mb.chunk, x, x_f32, mb.suh, nullptr, blockIdx.x - g.first[i]);   \
+    }
 GEMV_FAMILY(2)
 GEMV_FAMILY(3)
 GEMV_FAMILY(4)
 GEMV_FAMILY(5)
 GEMV_FAMILY(6)
 GEMV_FAMILY(8)
+GEMV_GROUP_KERNEL(2)
+GEMV_GROUP_KERNEL(3)
+GEMV_GROUP_KERNEL(4)
+GEMV_GROUP_KERNEL(5)
+GEMV_GROUP_KERNEL(6)
+GEMV_GROUP_KERNEL(8)
 
 // ---- decode GEMV, streamed over the whole tensor (1..16 rows) -------------------------------------------------------------
 //

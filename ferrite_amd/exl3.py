@@ -279,6 +279,25 @@ class Linear:
         check(_lib.lib().fe_exl3_linear_gemv_rotated(self.h, _stream(stream), ptr, y.data_ptr(), int(y_dtype), rows, ws.h))
 
 
+def _group_handles(linears):
+    return (C.c_void_p * len(linears))(*[l.h for l in linears])
+
+
+def forward_group(linears, x, x_dtype: Dtype, ys, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+    """ys[i][rows][n_i] = x[rows][k] @ W_i for linears of one input (q, k, v; gate, up): one GEMV launch for all of them
+    (forward_group_launches: 1 or 2 with the rotation), else one forward per member; the same bits either way."""
+    kern = linears[0].kern
+    ptrs = (C.c_uint64 * len(ys))(*[y.data_ptr() for y in ys])
+    check(_lib.lib().fe_exl3_linear_forward_group(_group_handles(linears), len(linears), kern.h, _stream(stream), x.data_ptr(),
+                                                  int(x_dtype), ptrs, int(y_dtype), rows, ws.h))
+
+
+def forward_group_launches(linears, rows: int, ws: "Workspace") -> int:
+    """Launches of forward_group: 1 (the GEMV rotates its input), 2 (a rotation for all members, then the GEMV), 0 (the
+    members run one after the other)."""
+    return _lib.lib().fe_exl3_linear_forward_group_launches(_group_handles(linears), len(linears), rows, ws.h)
+
+
 class Workspace:
     """Scratch shared by every Linear on one stream (linear.rs:136-161)."""
 

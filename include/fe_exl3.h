@@ -90,6 +90,21 @@ int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on);
 /* 1 if forward() with this many rows is a single launch (the decode GEMV rotates its own input: every program's K range
  * is whole 128-element Hadamard blocks), 0 if it is rotate_input followed by gemv_rotated. Same bits either way. */
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows);
+/* Several linears applied to the same input (the q, k, v or the gate, up projections of a layer), 1..16 rows: one GEMV
+ * launch whose programs are those of the members' own launches, so y[i] has the bits of
+ * fe_exl3_linear_forward(ls[i], ...). The launches' start-up and tails overlap and the members fill each other's gaps
+ * on the CUs. Where forward() of every member rotates its own input the group does too (one launch); otherwise one
+ * launch rotates the input for all members first (two launches). That needs 2..4 members of the same k and bits and a
+ * workspace with room for all members' partial sums and rotated inputs (one created from these linears has it);
+ * otherwise the members run one after the other (FE_EXL3_NO_GROUP=1 forces that). Which member's rotated input is left
+ * in the workspace is unspecified. The reference loops over the linears (Proj::forward,
+ * crates/fe-model/src/model.rs:365-403): this entry point has no counterpart there. */
+int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, const fe_exl3_kernels *kern, fe_stream_t s,
+                                 fe_devptr_t x, int x_dtype, const fe_devptr_t *ys, int y_dtype, uint32_t rows,
+                                 const fe_exl3_workspace *ws);
+/* Launches of that call: 1, 2, or 0 when the members run one after the other. */
+int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_t count, uint32_t rows,
+                                          const fe_exl3_workspace *ws);
 /* Linear::rotate_input (linear.rs:289-298): xh = fp16(H(x * suh) / sqrt(128)) into the workspace. */
 int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
                                 int x_dtype, uint32_t rows, const fe_exl3_workspace *ws);

@@ -373,6 +373,70 @@ def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, 
     assert np.all(np.abs(got - want) <= np.abs(want) / 1024.0 + 1e-5 * np.sqrt((want ** 2).mean()))
 
 
+@pytest.mark.parametrize("bits,k,ns,sks", [(4, 1024, (384, 128, 256), (2, 4, 1)), (3, 1280, (256, 640), (2, 1)),
+                                           (5, 1024, (128, 128, 384, 256), (8, 1, 2, 4)), (4, 2048, (512, 384), (16, 4))])
+def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sks, monkeypatch):
+    """Linears of one input (q, k, v; gate, up) in one GEMV launch: every member's programs are those of its own launch,
+    so each output has the bits of the member's forward(), for every row count, input and output type, with the input
+    rotated inside the GEMV (one launch) or by one launch for all members (two). Groups that cannot share a launch
+    (different bits, a streamed plan, a workspace without the room) run member by member."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    lins = []
+    for i, (n, sk) in enumerate(zip(ns, sks)):
+        t = synth.exl3_tensor(k, n, bits, 300 + 7 * i + bits)
+        lins.append(exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t) if i % 2 == 0 else exl3.DeviceExl3(t, False),
+                                          exl3.Plan(sk=sk, wk=1, ver=1, occ=2)))
+    ws = exl3.Workspace(lins, 16)
+    xb = synth.activations(16, k, 11, outliers=True)
+    xd = dev_u16(torch, xb)
+    xf = xd.view(torch.bfloat16).float().contiguous()
+    seen = set()
+    for rows in (1, 3, 8, 16):
+        launches = exl3.forward_group_launches(lins, rows, ws)
+        assert launches == (1 if all(l.forward_is_one_launch(rows) for l in lins) else 2), rows
+        seen.add(launches)
+        for x, xdt in ((xd, exl3.Dtype.Bf16), (xf, exl3.Dtype.F32)):
+            for ydt, tdt in ((exl3.Dtype.F32, torch.float32), (exl3.Dtype.Bf16, torch.bfloat16), (exl3.Dtype.Bf16Add, torch.bfloat16)):
+                fill = 1.5 if ydt == exl3.Dtype.Bf16Add else float("nan")
+                want = [torch.full((17, n), fill, dtype=tdt, device="cuda") for n in ns]
+                got = [torch.full((17, n), fill, dtype=tdt, device="cuda") for n in ns]
+                for lin, y in zip(lins, want):
+                    lin.forward(x, xdt, y, ydt, rows, ws)
+                exl3.forward_group(lins, x, xdt, got, ydt, rows, ws)
+                torch.cuda.synchronize()
+                for a, b in zip(want, got):
+                    ia, ib = (a.view(torch.int32), b.view(torch.int32)) if tdt == torch.float32 else (a.view(torch.int16), b.view(torch.int16))
+                    assert torch.equal(ia, ib), (rows, xdt, ydt)
+    assert 1 in seen
+    # twice in a row on the same workspace: the arrival counters are back at zero after each launch
+    y1 = [torch.zeros((4, n), dtype=torch.float32, device="cuda") for n in ns]
+    y2 = [torch.zeros((4, n), dtype=torch.float32, device="cuda") for n in ns]
+    exl3.forward_group(lins, xd, exl3.Dtype.Bf16, y1, exl3.Dtype.F32, 4, ws)
+    exl3.forward_group(lins, xd, exl3.Dtype.Bf16, y2, exl3.Dtype.F32, 4, ws)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(y1, y2))
+    # member by member: switched off, one member alone, a member of other bits, a workspace made for one small linear
+    monkeypatch.setenv("FE_EXL3_NO_GROUP", "1")
+    assert exl3.forward_group_launches(lins, 1, ws) == 0
+    y3 = [torch.zeros((4, n), dtype=torch.float32, device="cuda") for n in ns]
+    exl3.forward_group(lins, xd, exl3.Dtype.Bf16, y3, exl3.Dtype.F32, 4, ws)
+    torch.cuda.synchronize()
+    assert all(torch.equal(a, b) for a, b in zip(y1, y3))
+    monkeypatch.delenv("FE_EXL3_NO_GROUP")
+    assert exl3.forward_group_launches(lins[:1], 1, ws) == 0
+    other = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, 128, bits + 1, 5)), exl3.Plan(sk=1, wk=1, ver=1, occ=2))
+    mixed = [lins[0], other]
+    ws_mixed = exl3.Workspace(mixed, 16)
+    assert exl3.forward_group_launches(mixed, 1, ws_mixed) == 0
+    y4 = [torch.zeros((4, ns[0]), dtype=torch.float32, device="cuda"), torch.zeros((4, 128), dtype=torch.float32, device="cuda")]
+    exl3.forward_group(mixed, xd, exl3.Dtype.Bf16, y4, exl3.Dtype.F32, 4, ws_mixed)
+    torch.cuda.synchronize()
+    assert torch.equal(y4[0], y1[0])
+    small = exl3.Workspace([min(lins, key=lambda l: l.n * l.plan.sk)], 16)  # no room for every member's partial sums
+    assert exl3.forward_group_launches(lins, 16, small) == 0
+
+
 @pytest.mark.parametrize("bits,n,strips", [(2, 384, True), (3, 256, False), (4, 640, True), (5, 384, False), (6, 128, True),
                                            (8, 384, True), (4, 2304, True), (3, 4224, False)])
 def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracle, bits, n, strips, monkeypatch):
