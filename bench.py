@@ -1,19 +1,20 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-prefill]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-prefill] [--no-sweep]
 
 Workload (BASELINE.json configs[1]): the EXL3 decode MLP of a Qwen3.8-27B-shaped layer at M = 1, at 3, 4 and 5 bits per
-weight: gate and up are K=5120 N=17408, down is K=17408 N=5120. One step = Linear::forward (input rotation + trellis
-GEMV) through all nine linears on seeded synthetic layers, inputs and weights resident in HBM. `value` is the trellis
-bytes streamed per second (the reference's numerator, crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step,
-launch gaps and input rotations included. The nine weight sets total 401 MB, more than L2 plus the 256 MB Infinity
-Cache, so every step streams its weights from HBM.
+weight: gate and up are K=5120 N=17408, down is K=17408 N=5120. One step = the forward (input rotation + trellis GEMV)
+of all nine linears on seeded synthetic layers, inputs and weights resident in HBM, launched as the MLP block launches
+them: gate and up, two linears of the same input, as one grouped call (fe_exl3_linear_forward_group), down as
+Linear::forward. `value` is the trellis bytes streamed per second (the reference's numerator,
+crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step, launch gaps and input rotations included. The nine
+weight sets total 401 MB, more than L2 plus the 256 MB Infinity Cache, so every step streams its weights from HBM.
 
-`roofline` is the dominant kernel alone (the 4-bit GEMV of the 5120x17408 projections): its trellis bytes over its
-average launch duration, measured with HIP event pairs on the launch stream around its launches inside the timed
-region (the other launches of the timed region carry no events: every record is a packet of its own on the queue; a
-pass after the timed region brackets all nine for `per_linear_gemv`).
+`roofline` is the dominant kernel alone (the grouped 4-bit GEMV of the two 5120x17408 projections): its trellis bytes
+over its average launch duration, measured with HIP event pairs on the launch stream around its launches inside the
+timed region (the other launches of the timed region carry no events: every record is a packet of its own on the queue;
+a pass after the timed region brackets all six launches for `per_launch`).
 `cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host.
 `m2048` reports the prefill GEMMs (EXL3 4-bit and NVFP4, 5120x17408, M = 2048) in TFLOP/s against the bf16/f16 MFMA
 peak; it is measured after the timed region and is not part of `value`.
@@ -32,9 +33,9 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
-# `bench.py --traffic-pass` (profiles/exl3_gemv_b4_r1_m1_hbm_traffic.md): 22363 KiB fetched x 2.0 (the factor that
-# makes the counter read a streaming read and an elementwise update of known size correctly) + 400 KiB written x 1.0
-ROOFLINE_TRAFFIC_BYTES = int((22363 * 2.0 + 400 * 1.0) * 1024)
+# `bench.py --traffic-pass` (profiles/exl3_gemv_group_b4_m1_hbm_traffic.md): 45202 KiB fetched x 2.0 (the factor that
+# makes the counter read a streaming read and an elementwise update of known size correctly) + 799 KiB written x 1.0
+ROOFLINE_TRAFFIC_BYTES = int((45202 * 2.0 + 799 * 1.0) * 1024)
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA peak of MI355X
 SEED = 20251
@@ -97,6 +98,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true", help="leave out the M = 1, 4, 8, 16 sweep (for a kernel trace of the step alone)")
     ap.add_argument("--traffic-pass", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a streaming read and an elementwise update of "
                          "known size (the counters' calibration), then the roofline kernel, caches evicted in between")
@@ -143,34 +145,45 @@ def main():
         rel = float(np.abs(got - y_cpu).max() / np.sqrt((y_cpu ** 2).mean()))
         cpu["gpu_vs_cpu_max_err_over_rms"] = round(rel, 6)
 
+    # The step's launches: per bit width, gate + up of one input as a grouped call, then down. Every argument of the calls
+    # into the C ABI is prepared once.
+    f_group, f_forward, f_rotate, f_rotated, f_record = (lib.fe_exl3_linear_forward_group, lib.fe_exl3_linear_forward,
+                                                        lib.fe_exl3_linear_rotate_input, lib.fe_exl3_linear_gemv_rotated,
+                                                        lib.fe_hip_event_record)
+    bf16 = int(exl3.Dtype.Bf16)
+    by = {(name, bits): (lin, x, y) for name, bits, lin, x, y in linears}
+    launches = []  # (label, bytes, dominant, kernel launches, [(fn, args)...], keepalive)
+    for bits in BITS:
+        (g, xg, yg), (u, _, yu), (d, xd, yd) = by[("gate", bits)], by[("up", bits)], by[("down", bits)]
+        hs = (C.c_void_p * 2)(g.h, u.h)
+        ys = (C.c_uint64 * 2)(yg.data_ptr(), yu.data_ptr())
+        n_launch = exl3.forward_group_launches([g, u], 1, ws)
+        assert n_launch in (1, 2), "gate and up do not share a launch"
+        launches.append((f"gate+up_b{bits}", g.weight_bytes() + u.weight_bytes(), bits == 4, n_launch,
+                         [(f_group, (hs, 2, kern.h, stream, xg.data_ptr(), bf16, ys, bf16, 1, ws.h))], (hs, ys)))
+        if d.forward_is_one_launch(1):  # forward() is the GEMV alone (it rotates its own input)
+            calls = [(f_forward, (d.h, kern.h, stream, xd.data_ptr(), bf16, yd.data_ptr(), bf16, 1, ws.h))]
+        else:
+            calls = [(f_rotate, (d.h, kern.h, stream, xd.data_ptr(), bf16, 1, ws.h)),
+                     (f_rotated, (d.h, stream, ws.xh_ptr, yd.data_ptr(), bf16, 1, ws.h))]
+        launches.append((f"down_b{bits}", d.weight_bytes(), False, len(calls), calls, None))
+
     # Event pairs on the launch stream. In the timed region only the dominant kernel's launches carry them (each record is
     # a packet of its own on the queue and costs a few microseconds of the step); one more pass after the timed region
-    # brackets every linear for the per-linear table.
-    one_launch = [l[2].forward_is_one_launch(1) for l in linears]
-    dominant = [bits == 4 and lin.k == 5120 for name, bits, lin, x, y in linears]
-    events = [[(ev.new(), ev.new()) if dominant[li] else None for li in range(len(linears))] for _ in range(args.steps)]
-    table_events = [(ev.new(), ev.new()) for _ in linears]
-
-    # The step's calls into the C ABI, with every argument prepared once.
-    f_forward, f_rotate, f_rotated, f_record = (lib.fe_exl3_linear_forward, lib.fe_exl3_linear_rotate_input,
-                                                lib.fe_exl3_linear_gemv_rotated, lib.fe_hip_event_record)
-    bf16 = int(exl3.Dtype.Bf16)
-    calls = []
-    for li, (name, bits, lin, x, y) in enumerate(linears):
-        if one_launch[li]:  # forward() is the GEMV alone (it rotates its own input): the pair brackets that launch
-            calls.append((None, (f_forward, (lin.h, kern.h, stream, x.data_ptr(), bf16, y.data_ptr(), bf16, 1, ws.h))))
-        else:
-            calls.append(((f_rotate, (lin.h, kern.h, stream, x.data_ptr(), bf16, 1, ws.h)),
-                          (f_rotated, (lin.h, stream, ws.xh_ptr, y.data_ptr(), bf16, 1, ws.h))))
+    # brackets every launch for the per-launch table. The pair brackets the last call of a launch (the GEMV).
+    events = [[(ev.new(), ev.new()) if la[2] else None for la in launches] for _ in range(args.steps)]
+    table_events = [(ev.new(), ev.new()) for _ in launches]
 
     def step(pairs=None):
         rc = 0
-        for li, (pre, (fn, a)) in enumerate(calls):
-            if pre is not None:
-                rc |= pre[0](*pre[1])
+        for li, la in enumerate(launches):
+            calls = la[4]
+            for fn, a in calls[:-1]:
+                rc |= fn(*a)
             pair = pairs[li] if pairs is not None else None
             if pair is not None:
                 rc |= f_record(pair[0], stream)
+            fn, a = calls[-1]
             rc |= fn(*a)
             if pair is not None:
                 rc |= f_record(pair[1], stream)
@@ -188,24 +201,23 @@ def main():
     value = total_bytes / (dt / args.steps) / 1e9
 
     dom_ms = []
-    for li, (name, bits, lin, x, y) in enumerate(linears):
-        if dominant[li]:
+    for li, la in enumerate(launches):
+        if la[2]:
             dom_ms += [ev.ms(*events[i][li]) for i in range(args.steps)]
-            dom_bytes = lin.weight_bytes()
-            dom_kernel = "exl3_gemv_stream_b4" if lin.plan.ver == 2 else "exl3_gemv_b4_r1"
+            dom_bytes = la[1]
+            dom_kernel = "exl3_gemv_group_b4"
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
 
     per, reps = {}, max(args.steps, 5)
-    acc = [0.0] * len(linears)
-    for _ in range(reps):  # after the timed region: every linear bracketed
+    acc = [0.0] * len(launches)
+    for _ in range(reps):  # after the timed region: every launch bracketed
         step(table_events)
-        for li in range(len(linears)):
+        for li in range(len(launches)):
             acc[li] += ev.ms(*table_events[li])
-    for li, (name, bits, lin, x, y) in enumerate(linears):
+    for li, la in enumerate(launches):
         us = acc[li] / reps * 1e3
-        per[f"{name}_b{bits}"] = {"us": round(us, 2), "GB/s": round(lin.weight_bytes() / us / 1e3, 1), "plan": [lin.plan.sk, lin.plan.ver, lin.plan.occ],
-                                   "launches": 1 if one_launch[li] else 2}
+        per[la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
 
     out = {
         "metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048",
@@ -215,15 +227,16 @@ def main():
         "config": {"workload": "EXL3 decode MLP, Qwen3.8-27B-shaped layer, M=1, 3/4/5 bpw (gate, up 5120x17408; down 17408x5120)",
                    "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
-        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (5120x17408, M=1)", "achieved": round(achieved, 2),
+        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (gate + up, 5120x17408 each, M=1)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ROOFLINE_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms)},
         "cpu_baseline": cpu,
-        "per_linear_gemv": per,
+        "per_launch": per,
     }
 
-    out["graph_replay"] = graph_replay(lib, _lib.check, ev, exl3, linears, ws, total_bytes, args.steps, args.warmup)
-    out["rows_sweep_b4"] = rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears)
+    out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup)
+    if not args.no_sweep:
+        out["rows_sweep_b4"] = rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears)
     if not args.no_prefill:
         out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
     print(json.dumps(out))
@@ -234,57 +247,66 @@ def traffic_pass(torch, np, exl3, synth):
     exactly the roofline kernel's algorithmic bytes, evict, the roofline kernel. Prints the known sizes."""
     kern = exl3.Kernels.load()
     k, n = 5120, 17408
-    t = synth.exl3_tensor(k, n, 4, SEED, "gate")
-    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), exl3.default_blocks(exl3.cu_count()))
-    ws = exl3.Workspace([lin], 1)
+    blocks = exl3.default_blocks(exl3.cu_count())
+    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, n, 4, SEED, name)), blocks) for name in ("gate", "up")]
+    ws = exl3.Workspace(lins, 1)
     x = torch.from_numpy(synth.activations(1, k, SEED).view(np.int16)).cuda()
-    y = torch.zeros((1, n), dtype=torch.bfloat16, device="cuda")
-    buf = torch.zeros(lin.weight_bytes(), dtype=torch.uint8, device="cuda")
+    ys = [torch.zeros((1, n), dtype=torch.bfloat16, device="cuda") for _ in lins]
+    nbytes = sum(l.weight_bytes() for l in lins)
+    buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
     big = torch.zeros(600 << 20, dtype=torch.uint8, device="cuda")
+    assert exl3.forward_group_launches(lins, 1, ws) == 1
     for _ in range(3):
         big.add_(1)
         kern.probe_stream_read(buf, 1024, 1)
         big.add_(1)
-        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws)
+        exl3.forward_group(lins, x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, 1, ws)
     torch.cuda.synchronize()
-    print(json.dumps({"exl3_probe_v4_reads_KiB": lin.weight_bytes() / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
-                      "roofline_kernel": "exl3_gemv_b4_r1", "algorithmic_KiB": lin.weight_bytes() / 1024}))
+    print(json.dumps({"exl3_probe_v4_reads_KiB": nbytes / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
+                      "roofline_kernel": "exl3_gemv_group_b4", "algorithmic_KiB": nbytes / 1024}))
 
 
 def rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears, reps=20):
-    """The 4-bit linears at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts): microseconds per forward,
-    launched back to back, cycling gate, up, down so that no weight is served from cache. Not part of `value`."""
-    four = [(name, lin) for name, bits, lin, x, y in linears if bits == 4]
+    """The 4-bit MLP at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts): microseconds per linear,
+    launched back to back as the step launches them (gate + up grouped, then down), so that no weight is served from
+    cache. Not part of `value`."""
+    four = {name: lin for name, bits, lin, x, y in linears if bits == 4}
+    g, u, d = four["gate"], four["up"], four["down"]
     res = {}
     for m in (1, 4, 8, 16):
-        ws = exl3.Workspace([lin for _, lin in four], m)
-        io = []
-        for name, lin in four:
-            x = torch.from_numpy(synth.activations(m, lin.k, SEED).view(np.int16)).cuda()
-            io.append((lin, x, torch.zeros((m, lin.n), dtype=torch.bfloat16, device="cuda")))
-        for lin, x, y in io:
-            lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, ws, stream=stream)
+        ws = exl3.Workspace([g, u, d], m)
+        x = torch.from_numpy(synth.activations(m, g.k, SEED).view(np.int16)).cuda()
+        xd = torch.from_numpy(synth.activations(m, d.k, SEED).view(np.int16)).cuda()
+        yg, yu = (torch.zeros((m, g.n), dtype=torch.bfloat16, device="cuda") for _ in range(2))
+        yd = torch.zeros((m, d.n), dtype=torch.bfloat16, device="cuda")
+
+        def mlp():
+            exl3.forward_group([g, u], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=stream)
+            d.forward(xd, exl3.Dtype.Bf16, yd, exl3.Dtype.Bf16, m, ws, stream=stream)
+
+        mlp()
         a, b = ev.new(), ev.new()
         ev.record(a, stream)
         for _ in range(reps):
-            for lin, x, y in io:
-                lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, ws, stream=stream)
+            mlp()
         ev.record(b, stream)
-        us = ev.ms(a, b) * 1e3 / (reps * len(io))
-        nbytes = sum(lin.weight_bytes() for lin, _, _ in io) / len(io)
-        res[f"m{m}"] = {"us_per_forward": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
-                        "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        us = ev.ms(a, b) * 1e3 / (reps * 3)
+        nbytes = (g.weight_bytes() + u.weight_bytes() + d.weight_bytes()) / 3
+        res[f"m{m}"] = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
+                        "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                        "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
     return res
 
 
-def graph_replay(lib, check, ev, exl3, linears, ws, total_bytes, steps, warmup):
+def graph_replay(lib, check, ev, launches, stream, total_bytes, steps, warmup):
     """The same step captured once into a HIP graph on a stream of its own and replayed: what the step costs when the
-    host does not launch 18 kernels one by one. Reported beside `value`, which stays the eagerly launched step."""
+    host does not launch its kernels one by one. Reported beside `value`, which stays the eagerly launched step."""
     s = C.c_void_p()
     check(lib.fe_hip_stream_create(C.byref(s)))
     check(lib.fe_hip_graph_begin(s))
-    for name, bits, lin, x, y in linears:
-        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, 1, ws, stream=s)
+    for la in launches:
+        for fn, a in la[4]:
+            check(fn(*[s if v is stream else v for v in a]))  # the prepared calls, on the capturing stream
     g = C.c_void_p()
     check(lib.fe_hip_graph_end(s, C.byref(g)))
     for _ in range(max(warmup, 2)):
