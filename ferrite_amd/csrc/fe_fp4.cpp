@@ -20,7 +20,7 @@ constexpr uint32_t kTileN = 256;                        // GM_BN
 
 struct fe_fp4_kernels {
     fe_module_t module = nullptr;
-    fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4 = nullptr;
+    fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4[3] = {nullptr, nullptr, nullptr};
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
     uint32_t cus = 0;
@@ -41,8 +41,8 @@ struct fe_fp4_workspace {
     uint32_t max_rows = 0, max_k = 0;
     FeBuf codes, sf, aq, part, counters;  // part: partial sums of the GEMM (one slot a CU) or of the GEMV's splits
 };
-constexpr uint32_t kGemvRows = 16;      // rows of one fe_gemv_nvfp4 pass
-constexpr uint32_t kGemvMaxRows = 64;   // up to here the GEMV runs in passes; above, the GEMM
+constexpr uint32_t kGemvRows = 48;      // rows of one fe_gemv_nvfp4 pass (three groups of 16)
+constexpr uint32_t kGemvMaxRows = 64;   // up to here the GEMV runs (two passes above 48 rows); above, the GEMM
 constexpr uint32_t kGemvCounters = 8192;  // arrival counters: weight tiles of 128 rows (n <= 1 M)
 
 extern "C" {
@@ -55,7 +55,11 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->gemm4, k->module, "fe_gemm_nvfp4");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm4, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->reduce4, k->module, "fe_gemm_nvfp4_reduce");
-    if (!c) c = fe_hip_module_get_function(&k->gemv4, k->module, "fe_gemv_nvfp4");
+    for (int xr = 1; xr <= 3 && !c; xr++) {
+        char nm[32];
+        snprintf(nm, sizeof nm, "fe_gemv_nvfp4_x%d", xr);
+        c = fe_hip_module_get_function(&k->gemv4[xr - 1], k->module, nm);
+    }
     if (!c) c = fe_hip_module_get_function(&k->quant8, k->module, "fe_fp8_quant");
     if (!c) c = fe_hip_module_get_function(&k->gemm8, k->module, "fe_gemm_fp8");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
@@ -270,8 +274,8 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
     if (!l->fp8 && m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
-        // decode-sized: the weight-read-bound GEMV, 16 rows a pass. Two programs fit a CU: as many programs as run at
-        // once, not more (a second round of short programs costs more than idle CUs in the first).
+        // decode-sized: the weight-read-bound GEMV, up to 48 rows a pass. Two programs fit a CU: as many programs as run
+        // at once, not more (a second round of short programs costs more than idle CUs in the first).
         const uint32_t nts = n / kTile, kts = k / 64;
         uint32_t sk = 2 * kern->cus / nts;
         if (const char *e = getenv("FE_FP4_GEMV_SK")) sk = (uint32_t)atoi(e);
@@ -285,7 +289,7 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
             uint32_t rows = m - r0 < kGemvRows ? m - r0 : kGemvRows;
             fe_devptr_t yy = y + (size_t)r0 * ldy * 2, aq = ws->aq.p + (size_t)r0 * k * 2, rr = res ? res + (size_t)r0 * ldy * 2 : 0;
             void *args[] = {&yy, &aq, &w, &sw, &alpha, &rr, &z, &cnt, &rows, &n, &k, &ldy, &sk, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr};
-            FE_TRY(fe_hip_launch(kern->gemv4, nts * sk, 1, 1, 256, 1, 1, 0, s, args));
+            FE_TRY(fe_hip_launch(kern->gemv4[(rows + 15) / 16 - 1], nts * sk, 1, 1, 256, 1, 1, 0, s, args));
         }
         return 0;
     }

@@ -525,33 +525,36 @@ extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_codes(uint16_t*
         [&](uint32_t r, uint32_t l32, float (&v)[4]) { fp_store_piece<false>(out, v, al, l32, m0 + wm * 128 + r, m, col, n); });
 }
 
-// ---- GEMV (1..16 rows) -------------------------------------------------------------------------------------------------
+// ---- GEMV (1..48 rows) -------------------------------------------------------------------------------------------------
 
 #define FP4_GEMV_RG 8  // 16-row groups of a 128-row weight tile
 
 // One k tile of one 128-row weight tile as a wavefront reads it: lane L = 16 g + r takes, of row 16 rg + r, the 16 codes
-// k = 16 g .. 16 g + 15 (8 bytes) and the row's four scale bytes (it uses byte g), and of activation row r the same 16
-// values. The k index inside an MFMA is only a summation index, so the A operand (weights) and the B operand
-// (activations) merely have to agree: MFMA j of a row group multiplies k = 16 g + 8 j .. + 7 of lane group g.
+// k = 16 g .. 16 g + 15 (8 bytes) and the row's four scale bytes (it uses byte g), and of activation rows r, 16 + r, ...
+// (XR groups of 16) the same 16 values. The k index inside an MFMA is only a summation index, so the A operand (weights)
+// and the B operand (activations) merely have to agree: MFMA j of a row group multiplies k = 16 g + 8 j .. + 7 of lane
+// group g.
+template <int XR>
 struct Fp4GemvStage {
     u32x2 cw[FP4_GEMV_RG];
     uint32_t sc[FP4_GEMV_RG];
-    f16x8 x[2];
+    f16x8 x[XR][2];
 };
 
-// c[m][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res) for m <= 16 rows: the decode-sized form of fe_gemm_nvfp4, bound by
-// the read of the weights. grid (n / 128) * sk, 256 threads: a program takes one 128-row weight tile and one of sk runs
-// of k tiles, its four wavefronts alternate k tiles. Each wavefront expands its codes in registers straight into the
-// A operand of v_mfma_f32_16x16x32_f16 (rows = weight rows, columns = activation rows); the wavefronts' sums meet in
-// LDS. With sk > 1 the splits leave f32 partials in z[split][16][n]; the last to arrive (counters[tile]) adds them in
-// split order, finishes the tile and re-arms the counter, so the result does not depend on timing. Weight addressing as
-// in fe_gemm_nvfp4.
-extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
-                                                                   const uint8_t* sw, const float* alpha, const uint16_t* res,
-                                                                   float* z, uint32_t* counters, uint32_t m, uint32_t n,
-                                                                   uint32_t k, uint32_t ldc, uint32_t sk, uint32_t w_snt,
-                                                                   uint32_t w_skt, uint32_t w_sr, uint32_t s_snt,
-                                                                   uint32_t s_skt, uint32_t s_sr) {
+// c[m][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res) for m <= 16 XR rows: the decode-sized form of fe_gemm_nvfp4, bound
+// by the read of the weights, which every row count reads once. grid (n / 128) * sk, 256 threads: a program takes one
+// 128-row weight tile and one of sk runs of k tiles, its four wavefronts alternate k tiles. Each wavefront expands its
+// codes in registers straight into the A operand of v_mfma_f32_16x16x32_f16 (rows = weight rows, columns = activation
+// rows; one expansion serves all XR groups of activation rows); the wavefronts' sums meet in LDS. With sk > 1 the
+// splits leave f32 partials in z[split][m][n]; the last to arrive (counters[tile]) adds them in split order, finishes
+// the tile and re-arms the counter, so the result does not depend on timing. A row's sums do not depend on XR. Weight
+// addressing as in fe_gemm_nvfp4.
+template <int XR>
+__device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw,
+                                                const float* alpha, const uint16_t* res, float* z, uint32_t* counters,
+                                                uint32_t m, uint32_t n, uint32_t k, uint32_t ldc, uint32_t sk,
+                                                uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt,
+                                                uint32_t s_skt, uint32_t s_sr) {
     __shared__ f32x4 red[4][FP4_GEMV_RG][64];
     __shared__ uint32_t last_flag;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
@@ -559,9 +562,11 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
     const uint32_t ktiles = k / 64, kt_begin = split * ktiles / sk, kt_end = (split + 1) * ktiles / sk;
     const uint8_t* wp = w + (size_t)nt * w_snt + (size_t)r * w_sr + 8 * g;
     const uint8_t* sp = sw + (size_t)nt * s_snt + (size_t)r * s_sr;
-    const _Float16* xp = aq + (size_t)(r < m ? r : m - 1) * k + 16 * g;
+    const _Float16* xp[XR];
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++) xp[xr] = aq + (size_t)(16 * xr + r < m ? 16 * xr + r : m - 1) * k + 16 * g;
 
-    auto load = [&](Fp4GemvStage& st, uint32_t kt) {
+    auto load = [&](Fp4GemvStage<XR>& st, uint32_t kt) {
         const uint8_t* wk = wp + (size_t)kt * w_skt;
         const uint8_t* sk_ = sp + (size_t)kt * s_skt;
 #pragma unroll
@@ -569,26 +574,33 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
             st.cw[rg] = __builtin_nontemporal_load((const u32x2*)(wk + (size_t)(16 * rg) * w_sr));
             st.sc[rg] = __builtin_nontemporal_load((const uint32_t*)(sk_ + (size_t)(16 * rg) * s_sr));
         }
-        st.x[0] = *(const f16x8*)(xp + kt * 64);
-        st.x[1] = *(const f16x8*)(xp + kt * 64 + 8);
-    };
-    f32x4 acc[FP4_GEMV_RG];
 #pragma unroll
-    for (int rg = 0; rg < FP4_GEMV_RG; rg++) acc[rg] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    auto compute = [&](const Fp4GemvStage& st) {
+        for (int xr = 0; xr < XR; xr++) {
+            st.x[xr][0] = *(const f16x8*)(xp[xr] + kt * 64);
+            st.x[xr][1] = *(const f16x8*)(xp[xr] + kt * 64 + 8);
+        }
+    };
+    f32x4 acc[XR][FP4_GEMV_RG];
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++)
+#pragma unroll
+        for (int rg = 0; rg < FP4_GEMV_RG; rg++) acc[xr][rg] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const Fp4GemvStage<XR>& st) {
 #pragma unroll
         for (int rg = 0; rg < FP4_GEMV_RG; rg++) {
             Fp4Scale s = fp4_scale((st.sc[rg] >> (8 * g)) & 0xff);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 u32x4 a = fp4x8_to_f16(st.cw[rg][j], s);
-                acc[rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), st.x[j], acc[rg], 0, 0, 0);
+#pragma unroll
+                for (int xr = 0; xr < XR; xr++)
+                    acc[xr][rg] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), st.x[xr][j], acc[xr][rg], 0, 0, 0);
             }
         }
     };
     // Two k tiles in flight per wavefront. Loads past the end re-read the last k tile of the run (never used), which
     // keeps the loop free of branches around memory instructions.
-    Fp4GemvStage s0, s1;
+    Fp4GemvStage<XR> s0, s1;
     const uint32_t last = kt_end - 1;
     auto clamp = [&](uint32_t t) { return t < last ? t : last; };
     uint32_t kt = kt_begin + wave;
@@ -607,37 +619,47 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
         __builtin_amdgcn_sched_barrier(0);
     }
     if (kt < kt_end) compute(s0);
-    // the four wavefronts' sums meet in LDS; wavefront v finishes row groups 2 v and 2 v + 1
-#pragma unroll
-    for (int rg = 0; rg < FP4_GEMV_RG; rg++) red[wave][rg][lane] = acc[rg];
-    __syncthreads();
-    f32x4 sum[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        sum[h] = red[0][2 * wave + h][lane];
-#pragma unroll
-        for (int v = 1; v < 4; v++) sum[h] += red[v][2 * wave + h][lane];
-    }
-    // lane (r, g) holds, for row group rg, output row m = r, columns n0 + 16 rg + 4 g .. + 3
+    // The four wavefronts' sums meet in LDS, one group of activation rows at a time; wavefront v finishes weight row
+    // groups 2 v and 2 v + 1. Lane (r, g) then holds, for weight row group rg, output row 16 xr + r, columns
+    // n0 + 16 rg + 4 g .. + 3.
     const uint32_t col = nt * 128 + 32 * wave + 4 * g;  // + 16 h
-    auto finish = [&](const f32x4 (&v)[2]) {
-        if (r >= m) return;
+    f32x4 sum[XR][2];
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++) {
+        if (xr) __syncthreads();
+#pragma unroll
+        for (int rg = 0; rg < FP4_GEMV_RG; rg++) red[wave][rg][lane] = acc[xr][rg];
+        __syncthreads();
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            sum[xr][h] = red[0][2 * wave + h][lane];
+#pragma unroll
+            for (int v = 1; v < 4; v++) sum[xr][h] += red[v][2 * wave + h][lane];
+        }
+    }
+    auto finish = [&](uint32_t row, const f32x4 (&v)[2]) {
+        if (row >= m) return;
 #pragma unroll
         for (int h = 0; h < 2; h++) {
             uint32_t cc = col + 16 * h;
             float o[4] = {v[h][0], v[h][1], v[h][2], v[h][3]};
-            fp4_store4(c, res, (size_t)r * ldc + cc, o, *(const f32x4*)(alpha + cc) * FP4_OPERAND_SCALE);
+            fp4_store4(c, res, (size_t)row * ldc + cc, o, *(const f32x4*)(alpha + cc) * FP4_OPERAND_SCALE);
         }
     };
     if (sk == 1) {
-        finish(sum);
+#pragma unroll
+        for (int xr = 0; xr < XR; xr++) finish(16 * xr + r, sum[xr]);
         return;
     }
     // Partials cross to another program, possibly on another XCD with its own L2: agent-scope accesses, ordered by the
     // barriers around the arrival counter.
-    if (r < m) {
 #pragma unroll
-        for (int h = 0; h < 2; h++) store_agent_f32x4(z + ((size_t)split * 16 + r) * n + col + 16 * h, sum[h]);
+    for (int xr = 0; xr < XR; xr++) {
+        const uint32_t row = 16 * xr + r;
+        if (row < m) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) store_agent_f32x4(z + ((size_t)split * m + row) * n + col + 16 * h, sum[xr][h]);
+        }
     }
     __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's stores are acknowledged at agent scope
     __syncthreads();
@@ -648,24 +670,40 @@ extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4(uint16_t* c, 
     __syncthreads();
     if (!last_flag) return;
     if (tid == 0) __hip_atomic_store(&counters[nt], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (r >= m) return;
     // the loads of 8 splits are in flight together (an agent-scope load takes a trip to memory); sums in split order
-    f32x4 tot[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    for (uint32_t s0 = 0; s0 < sk; s0 += 8) {
-        f32x4 t[16];
 #pragma unroll
-        for (int b = 0; b < 8; b++) {
-            const uint32_t sp = s0 + b < sk ? s0 + b : sk - 1;
+    for (int xr = 0; xr < XR; xr++) {
+        const uint32_t row = 16 * xr + r;
+        if (row >= m) continue;
+        f32x4 tot[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        for (uint32_t s0 = 0; s0 < sk; s0 += 8) {
+            f32x4 t[16];
 #pragma unroll
-            for (int h = 0; h < 2; h++) t[2 * b + h] = load_agent_f32x4(z + ((size_t)sp * 16 + r) * n + col + 16 * h);
-        }
-        agent_loads_wait(t);
+            for (int b = 0; b < 8; b++) {
+                const uint32_t sp = s0 + b < sk ? s0 + b : sk - 1;
 #pragma unroll
-        for (int b = 0; b < 8; b++)
-            if (s0 + b < sk) {
-#pragma unroll
-                for (int h = 0; h < 2; h++) tot[h] += t[2 * b + h];
+                for (int h = 0; h < 2; h++) t[2 * b + h] = load_agent_f32x4(z + ((size_t)sp * m + row) * n + col + 16 * h);
             }
+            agent_loads_wait(t);
+#pragma unroll
+            for (int b = 0; b < 8; b++)
+                if (s0 + b < sk) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) tot[h] += t[2 * b + h];
+                }
+        }
+        finish(row, tot);
     }
-    finish(tot);
 }
+
+#define FP4_GEMV_KERNEL(XR)                                                                                            \
+    extern "C" __global__ __launch_bounds__(256, 2) void fe_gemv_nvfp4_x##XR(                                          \
+        uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw, const float* alpha, const uint16_t* res, \
+        float* z, uint32_t* counters, uint32_t m, uint32_t n, uint32_t k, uint32_t ldc, uint32_t sk, uint32_t w_snt,   \
+        uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt, uint32_t s_sr) {                                \
+        gemv_nvfp4_body<XR>(c, aq, w, sw, alpha, res, z, counters, m, n, k, ldc, sk, w_snt, w_skt, w_sr, s_snt, s_skt, \
+                            s_sr);                                                                                     \
+    }
+FP4_GEMV_KERNEL(1)
+FP4_GEMV_KERNEL(2)
+FP4_GEMV_KERNEL(3)  // (four groups of rows would not fit the registers of two programs a CU)

@@ -150,8 +150,9 @@ def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
 
 
 def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
-    """Up to 64 rows run the weight-read-bound GEMV (16 rows a pass, K cut over several programs); FE_FP4_NO_GEMV sends
-    the same rows through the GEMM. Both sum the same exact products in f32, in different orders."""
+    """Up to 64 rows run the weight-read-bound GEMV (up to 48 rows a pass, K cut over several programs); FE_FP4_NO_GEMV
+    sends the same rows through the GEMM. Both sum the same exact products in f32, in different orders; within the GEMV a
+    row's bits do not depend on the rows around it."""
     torch, fp4, kern = env
     from ferrite_amd import synth
     n, k = 384, 2048
@@ -160,7 +161,7 @@ def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
     lin = host.upload()
     view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), torch.from_numpy(host.sf).cuda(),
                                       torch.from_numpy(host.alpha).cuda(), host.g)
-    for m in (1, 3, 16, 17, 64):
+    for m in (1, 3, 16, 17, 48, 64):
         ws = fp4.Workspace(m, k)
         xd = dev_u16(torch, fp4_check_activations(m, k, lin.g, 40 + m))
         res = dev_u16(torch, bf16_bits(np.random.default_rng(m).normal(size=(m + 1, n)).astype(np.float32)))
@@ -182,6 +183,18 @@ def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
         monkeypatch.delenv("FE_FP4_NO_GEMV")
         a, b = bf16_to_f32(gemv).astype(np.float64), bf16_to_f32(gemm).astype(np.float64)
         assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all()
+    # the same rows alone, in a pass of 16, 32 or 48 rows, and as the second pass of 64
+    ws = fp4.Workspace(64, k)
+    x64 = dev_u16(torch, fp4_check_activations(64, k, lin.g, 77))
+    outs = {}
+    for m, r0 in ((5, 0), (16, 0), (30, 0), (48, 0), (64, 0), (7, 48), (16, 48)):
+        y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        lin.forward(kern, ws, y, n, x64[r0:], k, m)
+        torch.cuda.synchronize()
+        outs[(m, r0)] = y.view(torch.int16).cpu().numpy().view(np.uint16)
+    for m in (16, 30, 48, 64):
+        assert np.array_equal(outs[(m, 0)][:5], outs[(5, 0)])
+    assert np.array_equal(outs[(64, 0)][48:55], outs[(7, 48)]) and np.array_equal(outs[(64, 0)][48:], outs[(16, 48)])
 
 
 def test_fp4_argument_errors(env):
