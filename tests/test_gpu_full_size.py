@@ -112,6 +112,30 @@ def test_exl3_decode_rows_at_full_size(env, oracle, shape, bits):
                 assert np.array_equal(y1.cpu().numpy()[0].astype(np.float64), got[r])
 
 
+@pytest.mark.parametrize("shapes,bits", [(("gate_up", "gate_up"), 4), (("qo", "kv", "kv"), 4), (("gate_up", "gate_up"), 3)])
+def test_exl3_grouped_projections_at_full_size(env, shapes, bits):
+    """The projections of one input (gate, up; q, k, v) as one grouped launch at the benchmark's sizes: every member's
+    output has the bits of the member's own forward (checked against the reference above), at 1..16 rows."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    k = SHAPES[shapes[0]][0]
+    blocks = exl3.default_blocks(exl3.cu_count())
+    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, SHAPES[s][1], bits, 900 + i)), blocks)
+            for i, s in enumerate(shapes)]
+    ws = exl3.Workspace(lins, 16)
+    xd = dev_u16(torch, synth.activations(16, k, 3, outliers=True))
+    for m in (1, 4, 8, 16):
+        assert exl3.forward_group_launches(lins, m, ws) in (1, 2)
+        want = [torch.zeros((m, l.n), dtype=torch.bfloat16, device="cuda") for l in lins]
+        got = [torch.ones((m, l.n), dtype=torch.bfloat16, device="cuda") for l in lins]
+        for l, y in zip(lins, want):
+            l.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, ws)
+        exl3.forward_group(lins, xd, exl3.Dtype.Bf16, got, exl3.Dtype.Bf16, m, ws)
+        torch.cuda.synchronize()
+        for a, b in zip(want, got):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16)), m
+
+
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
 def test_exl3_prefill_at_full_size(env, oracle, shape):
     """M = 2048, 1 % outlier channels x20: the MFMA GEMM, including the tiles cut along K and the reduce kernel."""

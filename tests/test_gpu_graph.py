@@ -23,8 +23,12 @@ def test_forward_calls_replay_from_a_graph():
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 64)  # few programs per block: the K range is split
     streamed = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(4, 4, 2, 2))
     flin = synth.fp4_linear(384, 1024, 6).upload()
+    # two more linears of the same input: with `lin` a grouped launch (the argument block is copied at capture)
+    pair = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, n, 4, 30 + n)), 64) for n in (256, 128)]
+    group = [lin] + pair
     rows = [1, 16, 40, 300]
-    ws = exl3.Workspace([lin, streamed], max(rows))
+    ws = exl3.Workspace([lin, streamed] + pair, max(rows))
+    assert exl3.forward_group_launches(group, 1, ws) in (1, 2) and exl3.forward_group_launches(group, 16, ws) in (1, 2)
     fws = fp4.Workspace(max(rows), 1024)
     xs = {m: dev_u16(torch, synth.activations(m, 1024, m)) for m in rows}
 
@@ -33,17 +37,23 @@ def test_forward_calls_replay_from_a_graph():
             lin.forward(xs[m], exl3.Dtype.Bf16, outs[("e", m)], exl3.Dtype.F32, m, ws, stream=stream)
             flin.forward(fk, fws, outs[("f", m)], 384, xs[m], 1024, m, stream=stream)
         streamed.forward(xs[16], exl3.Dtype.Bf16, outs[("s", 16)], exl3.Dtype.F32, 16, ws, stream=stream)
+        for m in (1, 16):
+            exl3.forward_group(group, xs[m], exl3.Dtype.Bf16, [outs[("g", m, i)] for i in range(3)], exl3.Dtype.F32, m, ws, stream=stream)
 
     def fresh():
         o = {("e", m): torch.zeros((m, 384), dtype=torch.float32, device="cuda") for m in rows}
         o.update({("f", m): torch.zeros((m, 384), dtype=torch.bfloat16, device="cuda") for m in rows})
         o[("s", 16)] = torch.zeros((16, 384), dtype=torch.float32, device="cuda")
+        for m in (1, 16):
+            for i, l in enumerate(group):
+                o[("g", m, i)] = torch.zeros((m, l.n), dtype=torch.float32, device="cuda")
         return o
 
     eager = fresh()
     calls(None, eager)
     torch.cuda.synchronize()
     want = {k: v.clone() for k, v in eager.items()}
+    assert torch.equal(want[("g", 16, 0)], want[("e", 16)])  # a member of a group has the bits of its own forward
 
     s = C.c_void_p()
     check(lib.fe_hip_stream_create(C.byref(s)))
