@@ -295,6 +295,30 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears, reps=20):
         res[f"m{m}"] = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                         "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                         "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
+    # the attention projections of the same layer (40 heads of 128, 8 KV heads): q, k, v of one input grouped, then o
+    blocks = exl3.default_blocks(exl3.cu_count())
+    q, kk, v, o = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, n, 4, SEED, name)), blocks)
+                   for name, n in (("q", 5120), ("k", 1024), ("v", 1024), ("o", 5120)))
+    abytes = sum(l.weight_bytes() for l in (q, kk, v, o))
+    for m in (1, 4, 8, 16):
+        ws = exl3.Workspace([q, kk, v, o], m)
+        x = torch.from_numpy(synth.activations(m, 5120, SEED).view(np.int16)).cuda()
+        ys = [torch.zeros((m, l.n), dtype=torch.bfloat16, device="cuda") for l in (q, kk, v)]
+        yo = torch.zeros((m, 5120), dtype=torch.bfloat16, device="cuda")
+
+        def attn():
+            exl3.forward_group([q, kk, v], x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, m, ws, stream=stream)
+            o.forward(x, exl3.Dtype.Bf16, yo, exl3.Dtype.Bf16, m, ws, stream=stream)
+
+        attn()
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        for _ in range(reps):
+            attn()
+        ev.record(b, stream)
+        us = ev.ms(a, b) * 1e3 / reps
+        res[f"m{m}"]["attn_qkv_o_us"] = round(us, 2)
+        res[f"m{m}"]["attn_GB/s"] = round(abytes / us / 1e3, 1)
     return res
 
 
@@ -397,6 +421,35 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     res["nvfp4_5120x17408_m1"] = {"gemv_us": round(us, 2), "GB/s": round(wbytes / us / 1e3, 1),
                                   "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
     del flin, yf
+    # the layer's other prefill shape, down (17408 x 5120): the same two GEMMs
+    kd, nd = n, k
+    flops_d = 2.0 * m * nd * kd
+
+    def timed(fn):
+        fn()
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        for _ in range(10):
+            fn()
+        ev.record(b, stream)
+        return ev.ms(a, b) / 10
+
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(kd, nd, 4, SEED, "down")), 1024)
+    ws = exl3.Workspace([lin], m)
+    x = torch.from_numpy(synth.activations(m, kd, SEED, outliers=True).view(np.int16)).cuda()
+    y = torch.zeros((m, nd), dtype=torch.bfloat16, device="cuda")
+    lin.rotate_input(x, exl3.Dtype.Bf16, m, ws)
+    ms = timed(lambda: lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws))
+    res["exl3_b4_17408x5120"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops_d / ms / 1e9, 1),
+                                 "frac_mfma_peak": round(flops_d / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    del lin, ws
+    flin_d = synth.fp4_linear(nd, kd, SEED, input_scale=1.0).upload()
+    fws_d = fp4.Workspace(m, kd)
+    flin_d.quantize(fk, fws_d, x, kd, m)
+    ms = timed(lambda: flin_d.gemm(fk, fws_d, y, nd, m))
+    res["nvfp4_17408x5120"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops_d / ms / 1e9, 1),
+                               "frac_mfma_peak": round(flops_d / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    del flin_d, fws_d, x, y
     # the two neighbours of that GEMM in the prompt path: the fused gate|up front (SwiGLU + NVFP4 re-quantization in the
     # epilogue, 2 x 17408 output columns) and an FP8 linear of the same shape
     reps = 5

@@ -321,7 +321,7 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
     int cus = 0;
     if (!c && max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
-    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
+    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes);
     // zeroed once: the unused half of the last tile of an odd count of column blocks is read (and its sums discarded)
     if (!c && max_rows >= hat_rows() && max_hat) c = ws->hat.zeroed(max_hat);
     if (c) {
@@ -382,7 +382,7 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear_gemv_rotated", "rotated input of 4 GB or more");
     const uint32_t tiles_m = (rows + 255) / 256, tiles_n = (n / 128 + 1) / 2;
     if (group == 0 || group > tiles_m) group = tiles_m;
-    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = g.full, splits = g.splits;
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
     const bool kept = l->hat.bytes != 0;  // decoded once and kept: any row count above the GEMV's runs over it

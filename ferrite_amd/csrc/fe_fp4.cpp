@@ -211,7 +211,7 @@ int fe_fp4_workspace_create(fe_fp4_workspace **out, uint32_t max_rows, uint32_t 
     if (!c) c = ws->aq.alloc(rp * max_k * 2);
     int cus = 0;
     if (!c) c = fe_hip_cu_count(&cus);
-    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmPartBytes);
+    if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes);
     if (!c) c = ws->counters.zeroed(kGemvCounters * 4);
     if (c) {
         delete ws;
@@ -307,7 +307,7 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     // expansion on the 16-bit instruction, k tiles of 64; same products, another order of the f32 sums)
     const char *f16env = getenv("FE_FP8_F16");
     const bool codes8 = l->fp8 && !(f16env && atoi(f16env) != 0);
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = ws->part.p;
     float scale = l->fp8 ? 1.0f : 0.0625f;  // what the fp16 expansions of the two operands carry (FP4_OPERAND_SCALE)
@@ -356,7 +356,7 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p, part = ws->part.p;
     fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
     uint32_t full = gs.full, splits = gs.splits;
     void *args[] = {&aq,    &w,     &sw,   &alpha, &m,    &n,      &k,    &group,   &w_snt, &w_skt, &w_sr,
                     &s_snt, &s_skt, &s_sr, &full,  &splits, &part, &q_codes, &q_sf, &q_aq,  &down_g};

@@ -1,5 +1,6 @@
 // Shared by the host-side sources of libferrite_amd: error plumbing, device buffers, embedded code objects.
 #pragma once
+#include <algorithm>
 #include <cstddef>
 #include <cstdint>
 #include <cstdlib>
@@ -75,19 +76,28 @@ struct FeGemmSplit {
     uint32_t cut() const { return tiles - full; }
 };
 constexpr size_t kFeGemmPartBytes = 256 * 256 * 4;  // one partial slot
-// at most `cus` slots are ever used
-inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus) {
+constexpr uint32_t kFeGemmSlotsPerCu = 2;           // slots a workspace holds per CU
+// The cut that finishes the last round soonest: s pieces a tile take ceil(rem s / cus) rounds of 1 / s of a tile's time;
+// every piece also writes its 256 KB partial and the reduce kernel reads it back (about 2 % of a tile's time a piece).
+// At most `slots` pieces.
+inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus, uint32_t slots) {
     FeGemmSplit g;
     g.tiles = g.full = tiles;
-    if (!cus) return g;
-    uint32_t rem = tiles % cus;
-    if (rem == 0 || rem * 2 > cus) return g;  // a last round that is at least half full runs as it is
-    uint32_t splits = cus / rem, cap = 8;
+    if (!cus || !slots) return g;
+    const uint32_t rem = tiles % cus;
+    if (rem == 0) return g;
+    uint32_t cap = 8;
     if (const char *e = getenv("FE_GEMM_SPLITS")) cap = (uint32_t)atoi(e);  // 1: never cut
-    if (splits > cap) splits = cap;
-    if (splits > ktiles / 4) splits = ktiles / 4;  // at least 4 k tiles a program
-    if (splits < 2) return g;
+    cap = std::min(cap, ktiles / 4);                                        // at least 4 k tiles a program
+    cap = std::min(cap, slots / rem);
+    uint32_t best = 1;
+    float best_cost = 1.0f;
+    for (uint32_t sp = 2; sp <= cap; sp++) {
+        const float cost = (float)((rem * sp + cus - 1) / cus) / (float)sp + 0.02f * (float)sp;
+        if (cost < best_cost - 1e-6f) best = sp, best_cost = cost;
+    }
+    if (best < 2) return g;
     g.full = tiles - rem;
-    g.splits = splits;
+    g.splits = best;
     return g;
 }
