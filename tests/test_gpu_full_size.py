@@ -136,6 +136,41 @@ def test_exl3_grouped_projections_at_full_size(env, shapes, bits):
             assert torch.equal(a.view(torch.int16), b.view(torch.int16)), m
 
 
+def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
+    """The decode MLP's launches (gate + up grouped, then down) 240 times back to back on one workspace without a
+    synchronization in between, the row count changing from call to call (the role of
+    crates/fe-exl3/src/bin/exl3-stress.rs): partial sums and arrival counters of one launch must never leak into the
+    next, so every call has the bits of the first call with its row count."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    blocks = exl3.default_blocks(exl3.cu_count())
+    g, u = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, 17408, 4, 40 + i)), blocks) for i in range(2))
+    d = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(17408, 5120, 4, 42)), blocks)
+    ws = exl3.Workspace([g, u, d], 16)
+    x = dev_u16(torch, synth.activations(16, 5120, 5))
+    xd = dev_u16(torch, synth.activations(16, 17408, 6))
+    rows_list = (1, 16, 4, 8, 2, 13)
+    outs = []
+    for it in range(240):
+        m = rows_list[it % len(rows_list)]
+        ys = [torch.empty((m, 17408), dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+        yd = torch.empty((m, 5120), dtype=torch.bfloat16, device="cuda")
+        exl3.forward_group([g, u], x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, m, ws)
+        d.forward(xd, exl3.Dtype.Bf16, yd, exl3.Dtype.Bf16, m, ws)
+        outs.append((m, ys[0], ys[1], yd))
+    torch.cuda.synchronize()
+    first = {}
+    for it, (m, a, b, c) in enumerate(outs):
+        if m not in first:
+            first[m] = (a, b, c)
+            continue
+        for want, got in zip(first[m], (a, b, c)):
+            assert torch.equal(want.view(torch.int16), got.view(torch.int16)), (it, m)
+    # rows of a batch have the bits of the same rows in a smaller batch
+    assert torch.equal(first[16][0][:4].view(torch.int16), first[4][0].view(torch.int16))
+    assert torch.equal(first[16][2][:1].view(torch.int16), first[1][2].view(torch.int16))
+
+
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
 def test_exl3_prefill_at_full_size(env, oracle, shape):
     """M = 2048, 1 % outlier channels x20: the MFMA GEMM, including the tiles cut along K and the reduce kernel."""
