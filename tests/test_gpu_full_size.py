@@ -16,7 +16,8 @@ import pytest
 
 pytestmark = pytest.mark.gpu
 
-SHAPES = {"qo": (5120, 5120), "kv": (5120, 1024), "gate_up": (5120, 17408), "down": (17408, 5120)}
+SHAPES = {"qo": (5120, 5120), "kv": (5120, 1024), "gate_up": (5120, 17408), "down": (17408, 5120),
+          "lm_head": (5120, 151936)}  # the largest linear of a decode step: 1187 column blocks
 
 
 @pytest.fixture(scope="module")
@@ -95,7 +96,8 @@ def check(got, got_bf16, ref, f32_bound):
     assert (np.abs(got_bf16 - ref) / np.maximum(np.abs(ref), rms)).max() < 1e-2
 
 
-@pytest.mark.parametrize("shape,bits", [("qo", 4), ("kv", 4), ("gate_up", 3), ("gate_up", 4), ("gate_up", 5), ("down", 4)])
+@pytest.mark.parametrize("shape,bits", [("qo", 4), ("kv", 4), ("gate_up", 3), ("gate_up", 4), ("gate_up", 5), ("down", 4),
+                                        ("lm_head", 6)])
 def test_exl3_decode_rows_at_full_size(env, oracle, shape, bits):
     torch, exl3, kern = env
     k, n = SHAPES[shape]
