@@ -80,6 +80,7 @@ SYMBOLS = {
     "fe_exl3_linear_forward": (I, [P, P, P, U64, I, U64, I, U32, P]),
     "fe_exl3_linear_forward_is_one_launch": (I, [P, U32]),
     "fe_exl3_linear_keep_decoded": (I, [P, P, I]),
+    "fe_exl3_linear_forward_swiglu": (I, [P, P, P, U64, U64, U32, U64, I, U32, P]),
     "fe_exl3_linear_forward_group": (I, [PP, SZ, P, P, U64, I, C.POINTER(U64), I, U32, P]),
     "fe_exl3_linear_forward_group_launches": (I, [PP, SZ, U32, P]),
     "fe_exl3_linear_rotate_input": (I, [P, P, P, U64, I, U32, P]),

@@ -345,20 +345,34 @@ int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t 
     return 0;
 }
 
-int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
-                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
-    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "null argument");
+// The input of a rotation: bf16 (mode 0) or f32 (mode 1) rows of stride ld, or (mode 2) SwiGLU of two bf16 arrays,
+// x = gate and x2 = up, taken on the way in (RotSrc of k_exl3.hip).
+struct RotInput {
+    fe_devptr_t x = 0, x2 = 0;
+    uint32_t mode = 0, ld = 0;
+};
+
+static int launch_rot(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, const RotInput &in, uint32_t rows,
+                      const fe_exl3_workspace *ws, const char *fn) {
     if (rows == 0 || rows > ws->max_rows || l->k > ws->max_k) {
         char msg[160];
         snprintf(msg, sizeof msg, "%s: rows %u (workspace %u x %u)", l->name.c_str(), rows, ws->max_rows, ws->max_k);
-        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_rotate_input", msg);
+        return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
     }
+    uint32_t mode = in.mode, k = l->k, ld = in.ld;
+    fe_devptr_t x = in.x, x2 = in.x2, suh = l->view.suh, xh = ws->xh.p;
+    void *args[] = {&x, &mode, &suh, &xh, &k, &x2, &ld};
+    return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
+}
+
+int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
+                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "null argument");
     if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
         return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "x is bf16 or f32");
-    uint32_t x_f32 = (uint32_t)x_dtype & 1, k = l->k;
-    fe_devptr_t suh = l->view.suh, xh = ws->xh.p;
-    void *args[] = {&x, &x_f32, &suh, &xh, &k};
-    return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
+    RotInput in;
+    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
+    return launch_rot(l, kern, s, in, rows, ws, "fe_exl3_linear_rotate_input");
 }
 
 // trellis -> fp16 tiles (exl3_hat_tiles_b*) into `hat`, hat_bytes(l) bytes
@@ -401,10 +415,10 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
-// Decode-sized rows. With x != 0 the split-K kernel rotates x itself and leaves the rotated rows in xh (callers check
-// fused_rotation_fits first); otherwise it reads xh.
+// Decode-sized rows. With in.x != 0 the split-K kernel rotates that input itself and leaves the rotated rows in xh
+// (callers check fused_rotation_fits first); otherwise it reads xh.
 static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
-                       const fe_exl3_workspace *ws, fe_devptr_t x, uint32_t x_f32);
+                       const fe_exl3_workspace *ws, const RotInput &in);
 static uint32_t gemv_chunk(uint32_t rows, uint32_t steps);
 
 // The split-K kernel can rotate its own input when every program's K range is whole 128-element blocks.
@@ -423,11 +437,11 @@ static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
 
 int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
                                 uint32_t rows, const fe_exl3_workspace *ws) {
-    return launch_rows(l, s, xh, y, y_dtype, rows, ws, 0, 0);
+    return launch_rows(l, s, xh, y, y_dtype, rows, ws, RotInput{});
 }
 
 static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
-                       const fe_exl3_workspace *ws, fe_devptr_t x, uint32_t x_f32) {
+                       const fe_exl3_workspace *ws, const RotInput &in) {
     if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "null argument");
     if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "bad y dtype");
     const fe_exl3_plan &p = l->plan;
@@ -468,8 +482,9 @@ static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     uint32_t n = l->n, k = l->k, sk = p.sk, mode = (uint32_t)y_dtype, stride_k, stride_nb;
     view_strides(l->view, &stride_k, &stride_nb);
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
-    fe_devptr_t suh = l->view.suh;
-    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk, &x, &x_f32, &suh, &xh};
+    fe_devptr_t suh = l->view.suh, x = in.x, x2 = in.x2;
+    uint32_t x_mode = in.mode, ldx = in.ld;
+    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk, &x, &x_mode, &suh, &xh, &x2, &ldx};
     return fe_hip_launch(l->kern->gemv[bits_slot(l->bits)][rg - 1], n / 128 * sk, 1, 1, 256, 1, 1, lds, s, args);
 }
 
@@ -488,20 +503,40 @@ int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on) {
 
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }
 
-int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
-                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
-    if (l && kern && ws && x && fused_rotation_fits(l, rows)) {  // one launch: the GEMV rotates its own input
+// forward() on a described input: one launch where the GEMV rotates its own input, else the rotation and the linear.
+static int forward_from(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, const RotInput &in, fe_devptr_t y,
+                        int y_dtype, uint32_t rows, const fe_exl3_workspace *ws, const char *fn) {
+    if (fused_rotation_fits(l, rows)) {
         if (rows > ws->max_rows || l->k > ws->max_k) {
             char msg[160];
             snprintf(msg, sizeof msg, "%s: rows %u (workspace %u x %u)", l->name.c_str(), rows, ws->max_rows, ws->max_k);
-            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_forward", msg);
+            return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
         }
-        if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
-            return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "x is bf16 or f32");
-        return launch_rows(l, s, ws->xh.p, y, y_dtype, rows, ws, x, (uint32_t)x_dtype & 1);
+        return launch_rows(l, s, ws->xh.p, y, y_dtype, rows, ws, in);
     }
-    FE_TRY(fe_exl3_linear_rotate_input(l, kern, s, x, x_dtype, rows, ws));
+    FE_TRY(launch_rot(l, kern, s, in, rows, ws, fn));
     return fe_exl3_linear_gemv_rotated(l, s, ws->xh.p, y, y_dtype, rows, ws);
+}
+
+int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "null argument");
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "x is bf16 or f32");
+    RotInput in;
+    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
+    return forward_from(l, kern, s, in, y, y_dtype, rows, ws, "fe_exl3_linear_forward");
+}
+
+int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t gate,
+                                  fe_devptr_t up, uint32_t ld, fe_devptr_t y, int y_dtype, uint32_t rows,
+                                  const fe_exl3_workspace *ws) {
+    const char *fn = "fe_exl3_linear_forward_swiglu";
+    if (!l || !kern || !ws || !gate || !up) return fe_set_error(FE_ERR_ARG, fn, "null argument");
+    if (ld < l->k || ld % 4 || gate % 8 || up % 8) return fe_set_error(FE_ERR_ARG, fn, "gate / up: rows of at least k elements, 8-byte aligned");
+    RotInput in;
+    in.x = gate, in.x2 = up, in.mode = 2, in.ld = ld;
+    return forward_from(l, kern, s, in, y, y_dtype, rows, ws, fn);
 }
 
 // mirrors GemvGroup of k_exl3.hip
@@ -584,13 +619,13 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
         z_at += (size_t)m.sk * rows * l->n, cnt_at += l->n / 128;
     }
     for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
-    uint32_t x_f32 = (uint32_t)x_dtype & 1, k = ls[0]->k, mode = (uint32_t)y_dtype;
+    uint32_t x_mode = (uint32_t)x_dtype & 1, k = ls[0]->k, mode = (uint32_t)y_dtype;
     if (!fused) {  // one launch rotates the input for every member, and the GEMV reads the members' rotated inputs
-        void *rargs[] = {&r, &x, &x_f32, &k};
+        void *rargs[] = {&r, &x, &x_mode, &k};
         FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
         x = 0;
     }
-    void *args[] = {&g, &x, &x_f32, &k, &rows, &mode};
+    void *args[] = {&g, &x, &x_mode, &k, &rows, &mode};
     return fe_hip_launch(kern->gemv_group[bits_slot(ls[0]->bits)], programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 

@@ -347,8 +347,14 @@ int fe_route_mlp_forward(const fe_route_ctx *c, const fe_route_proj *gate_up, co
         FE_TRY(proj_forward(gate_up, c, d, big, xn, hidden, n_rest, ptr, ld, 8, &parts));
         if (parts < 2) return fe_set_error(FE_ERR_SHAPE, fn, "gate_up has fewer than two parts");
         if (ld[0] != ld[1]) return fe_set_error(FE_ERR_SHAPE, fn, "gate/up strides differ");
-        FE_TRY(fe_route_silu_mul(c->s, act, ptr[0], ptr[1], ld[0], inter, n_rest));
-        FE_TRY(linear_forward(down, c, d, x, hidden, act, inter, n_rest, x));
+        if (down->q && c->x3() && n_rest <= FE_X3_PASS && (n_rest <= FE_X3_ROWS || d >= n_rest)) {
+            // every row through down's trellis GEMV in one pass: SwiGLU is applied as the GEMV's input rotation reads
+            // gate and up (the bits of fe_silu_mul followed by the linear; the reference launches both, model.rs:3184-3199)
+            FE_TRY(fe_exl3_linear_forward_swiglu(down->q, c->xk, c->s, ptr[0], ptr[1], ld[0], x, FE_DTYPE_BF16_ADD, n_rest, c->xws));
+        } else {
+            FE_TRY(fe_route_silu_mul(c->s, act, ptr[0], ptr[1], ld[0], inter, n_rest));
+            FE_TRY(linear_forward(down, c, d, x, hidden, act, inter, n_rest, x));
+        }
     }
     return 0;
 }

@@ -151,54 +151,59 @@ extern "C" __global__ __launch_bounds__(128) void exl3_had_cols_bf16(const float
 
 // ---- input rotation ------------------------------------------------------------------------------------------------
 
-// One 128-element block of a row: fp16(H(x * suh) / sqrt(128)), 4 elements a lane of a half wavefront. `at` indexes x
-// (bf16, or f32 with x_f32), `c` the block's channel of this lane. Split in two so that a caller can issue the loads
-// early; all 32 lanes of the half wavefront take part in rot_finish.
+// One 128-element block of a row: fp16(H(x * suh) / sqrt(128)), 4 elements a lane of a half wavefront. The input is
+// bf16 (mode 0) or f32 (mode 1) rows, or (mode 2) SwiGLU of two bf16 arrays, x = gate and x2 = up, taken on the way in:
+// bf16(bf16(silu(gate)) * up), the bits fe_silu_mul would have left in memory. `xat` indexes the input (row * ld + c),
+// `c` is the block's channel of this lane. Split in two so that a caller can issue the loads early; all 32 lanes of the
+// half wavefront take part in rot_finish.
+struct RotSrc {
+    const void *x, *x2;
+    uint32_t mode, ld;  // ld: elements between input rows
+};
 struct RotRaw {
     f32x4 xf;
-    u32x2 xb, s;
+    u32x2 xb, ub, s;
 };
-__device__ __forceinline__ RotRaw rot_load(const void* x, uint32_t x_f32, const uint16_t* suh, size_t at, uint32_t c) {
+__device__ __forceinline__ RotRaw rot_load(const RotSrc& src, const uint16_t* suh, size_t xat, uint32_t c) {
     RotRaw r;
-    if (x_f32)
-        r.xf = *(const f32x4*)((const float*)x + at);
-    else
-        r.xb = *(const u32x2*)((const uint16_t*)x + at);
+    if (src.mode == 1) {
+        r.xf = *(const f32x4*)((const float*)src.x + xat);
+    } else {
+        r.xb = *(const u32x2*)((const uint16_t*)src.x + xat);
+        if (src.mode == 2) r.ub = *(const u32x2*)((const uint16_t*)src.x2 + xat);
+    }
     r.s = *(const u32x2*)(suh + c);
     return r;
 }
-__device__ __forceinline__ u32x2 rot_finish(const RotRaw& r, uint32_t x_f32, uint32_t l32) {
+__device__ __forceinline__ u32x2 rot_finish(const RotRaw& r, uint32_t mode, uint32_t l32) {
     float v[4];
-    if (x_f32) {
+    if (mode == 1) {
         v[0] = r.xf[0], v[1] = r.xf[1], v[2] = r.xf[2], v[3] = r.xf[3];
     } else {
-        v[0] = __uint_as_float(r.xb[0] << 16), v[1] = __uint_as_float(r.xb[0] & 0xffff0000u);
-        v[2] = __uint_as_float(r.xb[1] << 16), v[3] = __uint_as_float(r.xb[1] & 0xffff0000u);
+        u32x2 xb = r.xb;
+        if (mode == 2) xb = (u32x2){silu_mul_bf16x2(r.xb[0], r.ub[0]), silu_mul_bf16x2(r.xb[1], r.ub[1])};
+        v[0] = __uint_as_float(xb[0] << 16), v[1] = __uint_as_float(xb[0] & 0xffff0000u);
+        v[2] = __uint_as_float(xb[1] << 16), v[3] = __uint_as_float(xb[1] & 0xffff0000u);
     }
     v[0] *= f16_bits_to_f32(r.s[0] & 0xffff), v[1] *= f16_bits_to_f32(r.s[0] >> 16);
     v[2] *= f16_bits_to_f32(r.s[1] & 0xffff), v[3] *= f16_bits_to_f32(r.s[1] >> 16);
     fwht128_half_wave(v, l32);
     return (u32x2){pack_f16x2(v[0] * FE_HAD_SCALE, v[1] * FE_HAD_SCALE), pack_f16x2(v[2] * FE_HAD_SCALE, v[3] * FE_HAD_SCALE)};
 }
-__device__ __forceinline__ u32x2 rot_block(const void* x, uint32_t x_f32, const uint16_t* suh, size_t at, uint32_t c,
-                                           uint32_t l32) {
-    return rot_finish(rot_load(x, x_f32, suh, at, c), x_f32, l32);
-}
 
-// xh[row][k] = fp16(H(x * suh) / sqrt(128)), x bf16 (x_f32 = 0) or f32. grid (ceil(k / 512), rows), 128 threads: each
-// half wavefront one 128-element block, 4 elements a lane. (kernels/k-exl3/src/gemv.rs:147-170)
-__device__ __forceinline__ void rot_in_body(const void* x, uint32_t x_f32, const uint16_t* suh, uint16_t* xh, uint32_t k) {
+// xh[row][k] = fp16(H(x * suh) / sqrt(128)). grid (ceil(k / 512), rows), 128 threads: each half wavefront one
+// 128-element block, 4 elements a lane. (kernels/k-exl3/src/gemv.rs:147-170)
+__device__ __forceinline__ void rot_in_body(const RotSrc& src, const uint16_t* suh, uint16_t* xh, uint32_t k) {
     uint32_t l32 = threadIdx.x & 31;
     uint32_t blk = blockIdx.x * 4 + threadIdx.x / 32;
     bool live = blk * 128 < k;
     uint32_t c = (live ? blk : 0) * 128 + 4 * l32;
-    size_t at = (size_t)blockIdx.y * k + c;
-    u32x2 o = rot_block(x, x_f32, suh, at, c, l32);
-    if (live) *(u32x2*)(xh + at) = o;
+    u32x2 o = rot_finish(rot_load(src, suh, (size_t)blockIdx.y * src.ld + c, c), src.mode, l32);
+    if (live) *(u32x2*)(xh + (size_t)blockIdx.y * k + c) = o;
 }
-extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_f32, const uint16_t* suh,
-                                                               uint16_t* xh, uint32_t k) {
-    rot_in_body(x, x_f32, suh, xh, k);
+extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uint32_t x_mode, const uint16_t* suh,
+                                                               uint16_t* xh, uint32_t k, const void* x2, uint32_t ldx) {
+    rot_in_body(RotSrc{x, x2, x_mode, ldx}, suh, xh, k);
 }
 
 #define FE_EXL3_GROUP_MAX 4  // linears of one grouped launch
@@ -208,8 +213,8 @@ struct RotGroup {
     const uint16_t* suh[FE_EXL3_GROUP_MAX];
     uint16_t* xh[FE_EXL3_GROUP_MAX];
 };
-extern "C" __global__ __launch_bounds__(128) void exl3_rot_in_group(RotGroup g, const void* x, uint32_t x_f32, uint32_t k) {
-    rot_in_body(x, x_f32, g.suh[blockIdx.z], g.xh[blockIdx.z], k);
+extern "C" __global__ __launch_bounds__(128) void exl3_rot_in_group(RotGroup g, const void* x, uint32_t x_mode, uint32_t k) {
+    rot_in_body(RotSrc{x, nullptr, x_mode, k}, g.suh[blockIdx.z], g.xh[blockIdx.z], k);
 }
 
 // ---- decode GEMV -----------------------------------------------------------------------------------------------------
@@ -355,16 +360,15 @@ __device__ __forceinline__ f32x4 row_scales(const uint16_t* svh, uint32_t col) {
 // inputs of the program's K range pass through LDS in chunks of `chunk` load steps (a multiple of 4): dynamic LDS
 // max(m * (chunk * 128 + 16), m * GEMV_RED_PITCH * 4) bytes. With sk > 1 the splits leave f32 partials in
 // z[split][m][n]; the last to arrive (counters[column block]) adds them in split order, finishes the block and re-arms
-// the counter. With x != nullptr the kernel rotates its own inputs from x (as exl3_rot_in does, bit for bit) instead of
+// the counter. With src.x != nullptr the kernel rotates its own inputs from src (as exl3_rot_in does, bit for bit) instead of
 // reading xh, and leaves them in xh_out: one launch for the whole linear. That needs every staged K range to be whole
 // 128-element blocks: k / 64 / sk and chunk even. (kernels/k-exl3/src/gemv.rs:412-587)
 template <int BITS, int RG>
 __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
                                           const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
                                           uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode,
-                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk, const void* x,
-                                          uint32_t x_f32, const uint16_t* __restrict__ suh, uint16_t* xh_out,
-                                          uint32_t program) {
+                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk, const RotSrc src,
+                                          const uint16_t* __restrict__ suh, uint16_t* xh_out, uint32_t program) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
     constexpr uint32_t tw = 8 * BITS;
@@ -398,20 +402,22 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     // Rotating here: the first block's loads go out ahead of the trellis loads (loads return in order), so that the
     // rotation runs while the first trellis words are still on their way.
     const uint32_t rot_hw = tid >> 5, rot_l32 = tid & 31;
-    auto rot_at = [&](uint32_t c0, uint32_t nblk, uint32_t p, size_t& at, uint32_t& c, uint32_t& off) {
+    const void* x = src.x;
+    auto rot_at = [&](uint32_t c0, uint32_t nblk, uint32_t p, size_t& at, size_t& xat, uint32_t& c, uint32_t& off) {
         uint32_t row = p / nblk, b = p - row * nblk;
         c = (kt0 + 4 * c0) * 16 + b * 128 + 4 * rot_l32;
         at = (size_t)row * k + c;
+        xat = (size_t)row * src.ld + c;
         off = row * xpitch + b * 256 + 8 * rot_l32;
     };
     RotRaw rot_raw = {};
     if (x) {
         const uint32_t nblk = (steps < chunk ? steps : chunk) / 2;
         if (rot_hw < m * nblk) {
-            size_t at;
+            size_t at, xat;
             uint32_t c, off;
-            rot_at(0, nblk, rot_hw, at, c, off);
-            rot_raw = rot_load(x, x_f32, suh, at, c);
+            rot_at(0, nblk, rot_hw, at, xat, c, off);
+            rot_raw = rot_load(src, suh, xat, c);
         }
     }
 
@@ -431,19 +437,19 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
             // (the launcher's condition for passing x).
             const uint32_t nblk = cs / 2, total = m * nblk;
             uint32_t p = rot_hw, c = 0, off = 0;
-            size_t at = 0;
+            size_t at = 0, xat = 0;
             if (p < total) {
-                rot_at(c0, nblk, p, at, c, off);
-                if (c0) rot_raw = rot_load(x, x_f32, suh, at, c);
+                rot_at(c0, nblk, p, at, xat, c, off);
+                if (c0) rot_raw = rot_load(src, suh, xat, c);
             }
             while (p < total) {
-                u32x2 o = rot_finish(rot_raw, x_f32, rot_l32);
+                u32x2 o = rot_finish(rot_raw, src.mode, rot_l32);
                 *(u32x2*)(lds + off) = o;
                 if (nb == 0 && xh_out) *(u32x2*)(xh_out + at) = o;
                 p += 8;
                 if (p < total) {
-                    rot_at(c0, nblk, p, at, c, off);
-                    rot_raw = rot_load(x, x_f32, suh, at, c);
+                    rot_at(c0, nblk, p, at, xat, c, off);
+                    rot_raw = rot_load(src, suh, xat, c);
                 }
             }
         } else {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
@@ -570,9 +576,10 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_b##BITS##_r##RG(                                      \
         const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,       \
         uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb,       \
-        uint32_t chunk, const void* x, uint32_t x_f32, const uint16_t* suh, uint16_t* xh_out) {                        \
-        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk, x,     \
-                            x_f32, suh, xh_out, blockIdx.x);                                                          \
+        uint32_t chunk, const void* x, uint32_t x_mode, const uint16_t* suh, uint16_t* xh_out, const void* x2,         \
+        uint32_t ldx) {                                                                                               \
+        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk,        \
+                            RotSrc{x, x2, x_mode, ldx}, suh, xh_out, blockIdx.x);                                     \
     }
 #define GEMV_FAMILY(BITS) GEMV_KERNEL(BITS, 1) GEMV_KERNEL(BITS, 2) GEMV_KERNEL(BITS, 3) GEMV_KERNEL(BITS, 4)
 
@@ -594,13 +601,14 @@ struct GemvGroup {
 };
 #define GEMV_GROUP_KERNEL(BITS)                                                                                        \
     extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_group_b##BITS(GemvGroup g, const void* x,           \
-                                                                               uint32_t x_f32, uint32_t k, uint32_t m, \
+                                                                               uint32_t x_mode, uint32_t k, uint32_t m, \
                                                                                uint32_t y_mode) {                      \
         uint32_t i = 0;                                                                                                \
         while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) i++;                                                   \
         const GemvGroup::Member& mb = g.m[i];                                                                          \
         gemv_body<BITS, 1>(mb.xh, mb.trellis, mb.svh, mb.y, mb.z, mb.counters, mb.n, k, m, mb.sk, y_mode,            \
-                           mb.stride_k, mb.stride_nb, mb.chunk, x, x_f32, mb.suh, nullptr, blockIdx.x - g.first[i]);   \
+                           mb.stride_k, mb.stride_nb, mb.chunk, RotSrc{x, nullptr, x_mode, k}, mb.suh, nullptr,        \
+                           blockIdx.x - g.first[i]);                                                                   \
     }
 GEMV_FAMILY(2)
 GEMV_FAMILY(3)

@@ -9,14 +9,7 @@ extern "C" __global__ __launch_bounds__(256) void fe_silu_mul(uint16_t* out, con
     const uint32_t r = blockIdx.y, c = (blockIdx.x * 256 + threadIdx.x) * 2;
     if (c >= inter) return;
     const uint32_t g = *(const uint32_t*)(gate + (size_t)r * ld + c), u = *(const uint32_t*)(up + (size_t)r * ld + c);
-    float v[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        float gv = bf16_bits_to_f32((g >> (16 * i)) & 0xffff), uv = bf16_bits_to_f32((u >> (16 * i)) & 0xffff);
-        float s = gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv));
-        v[i] = bf16_bits_to_f32(f32_to_bf16_bits(s)) * uv;
-    }
-    *(uint32_t*)(out + (size_t)r * inter + c) = pack_bf16x2(v[0], v[1]);
+    *(uint32_t*)(out + (size_t)r * inter + c) = silu_mul_bf16x2(g, u);
 }
 
 // dst[r][c .. c + 1] = src[r][c .. c + 1]. grid (rows, ceil(cols / 2 / 256)), 256 threads.

@@ -125,6 +125,19 @@ __device__ __forceinline__ void fwht128_half_wave_rows(float (&v)[R][4], uint32_
         for (int q = 0; q < 4; q++) v[r][q] = x[4 * r + q];
 }
 
+// Two elements of SwiGLU on bf16 pairs: bf16(bf16(silu(g)) * u), silu(g) = g / (1 + exp(-g)) in f32
+// (kernels/k-core/src/misc.rs:58-71). One definition, so that every kernel that applies it rounds alike.
+__device__ __forceinline__ uint32_t silu_mul_bf16x2(uint32_t g, uint32_t u) {
+    float v[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        float gv = bf16_bits_to_f32((g >> (16 * i)) & 0xffff), uv = bf16_bits_to_f32((u >> (16 * i)) & 0xffff);
+        float s = gv * __builtin_amdgcn_rcpf(1.0f + __expf(-gv));
+        v[i] = bf16_bits_to_f32(f32_to_bf16_bits(s)) * uv;
+    }
+    return pack_bf16x2(v[0], v[1]);
+}
+
 // 16 bytes at agent scope: partial sums that one program leaves for another, possibly on another XCD with its own L2.
 // The store goes through to memory, the load reads past this XCD's L2 (the sc1 forms that clang emits for 4-byte
 // agent-scope atomics; it has no 16-byte ones). The compiler does not count these loads: agent_loads_wait must come

@@ -262,6 +262,14 @@ class Linear:
         check(_lib.lib().fe_exl3_linear_forward(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), y.data_ptr(),
                                                 int(y_dtype), rows, ws.h))
 
+    def forward_swiglu(self, gate, up, ld: int, y, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+        """y[rows][n] = SwiGLU(gate, up)[rows][k] @ W with bf16 gate / up of row stride ld (pointers or tensors): the
+        activation bf16(bf16(silu(gate)) * up) is formed as the input rotation reads it."""
+        gp = gate if isinstance(gate, int) else gate.data_ptr()
+        up_ = up if isinstance(up, int) else up.data_ptr()
+        check(_lib.lib().fe_exl3_linear_forward_swiglu(self.h, self.kern.h, _stream(stream), gp, up_, ld, y.data_ptr(), int(y_dtype),
+                                                       rows, ws.h))
+
     def keep_decoded(self, on: bool = True, stream=None):
         """Decode the trellis once into fp16 tiles kept with the linear (2 bytes a weight): calls with more than 64 rows
         then run the GEMM over them without decoding."""

@@ -90,6 +90,15 @@ int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on);
 /* 1 if forward() with this many rows is a single launch (the decode GEMV rotates its own input: every program's K range
  * is whole 128-element Hadamard blocks), 0 if it is rotate_input followed by gemv_rotated. Same bits either way. */
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows);
+/* forward() on SwiGLU(gate, up) without the activation ever being stored: y = act @ W with
+ * act[r][c] = bf16(bf16(silu(gate[r][c])) * up[r][c]) (the arithmetic of fe_silu_mul, kernels/k-core/src/misc.rs:58-71),
+ * computed as the input rotation reads it, inside the GEMV for few rows. gate and up are bf16 [rows][>= k] with row
+ * stride ld elements, 8-byte aligned, ld % 4 == 0. Same bits as fe_silu_mul into a buffer followed by
+ * fe_exl3_linear_forward on it. This is the down projection of the MLP block (crates/fe-model/src/model.rs:3184-3199),
+ * where the reference launches fe_silu_mul and Linear::forward one after the other. */
+int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t gate,
+                                  fe_devptr_t up, uint32_t ld, fe_devptr_t y, int y_dtype, uint32_t rows,
+                                  const fe_exl3_workspace *ws);
 /* Several linears applied to the same input (the q, k, v or the gate, up projections of a layer), 1..16 rows: one GEMV
  * launch whose programs are those of the members' own launches, so y[i] has the bits of
  * fe_exl3_linear_forward(ls[i], ...). The launches' start-up and tails overlap and the members fill each other's gaps

@@ -78,7 +78,9 @@ int fe_route_copy2d(fe_stream_t s, fe_devptr_t dst, uint32_t ldd, fe_devptr_t sr
  * Prompt rows [d, rows) with more than FE_X3_ROWS of them take the fused front when swiglu (gate|up interleaved by 8,
  * NVFP4), down's prompt form and act_ws (a prompt workspace for [rows][inter]) are given: forward_swiglu, then down's
  * GEMM on the quantized activation with the residual in place. The other rows: gate_up, fe_silu_mul, down with the
- * residual. big: scratch for gate_up's outputs ([rows][total n]); act: scratch [rows][inter]. */
+ * residual; where all of them go through down's trellis GEMV in one pass, SwiGLU is applied as that GEMV's input
+ * rotation reads gate and up (fe_exl3_linear_forward_swiglu: the same bits, act is not written).
+ * big: scratch for gate_up's outputs ([rows][total n]); act: scratch [rows][inter]. */
 int fe_route_mlp_forward(const fe_route_ctx *c, const fe_route_proj *gate_up, const fe_route_linear *down,
                          const fe_fp4_linear *swiglu, const fe_fp4_workspace *act_ws, fe_devptr_t x, fe_devptr_t xn,
                          fe_devptr_t big, fe_devptr_t act, uint32_t rows, uint32_t hidden, uint32_t inter);

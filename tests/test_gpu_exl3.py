@@ -373,6 +373,45 @@ def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, 
     assert np.all(np.abs(got - want) <= np.abs(want) / 1024.0 + 1e-5 * np.sqrt((want ** 2).mean()))
 
 
+@pytest.mark.parametrize("k,sk", [(1024, 2), (1280, 2), (2048, 16)])
+def test_forward_on_swiglu_of_gate_and_up(env, k, sk):
+    """The down projection of the MLP block takes SwiGLU(gate, up) as its input without the activation being stored:
+    the bits of fe_silu_mul into a buffer followed by forward() on it, for every row count (inside the GEMV, in the
+    rotation kernel in front of the GEMV, in front of the GEMM) and output mode, gate and up being column ranges of one
+    wider array."""
+    torch, exl3, kern = env
+    from ferrite_amd import route, synth
+    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, 384, 4, 90 + sk)), exl3.Plan(sk=sk, wk=1, ver=1, occ=2))
+    mr = 130
+    ws = exl3.Workspace([lin], mr)
+    ld = 2 * k + 8
+    gu = dev_u16(torch, synth.activations(mr, ld, 21, outliers=True))  # [gate | up | 8 unused columns]
+    gate_ptr, up_ptr = gu.data_ptr(), gu.data_ptr() + 2 * k
+    seen = set()
+    for rows in (1, 3, 16, 40, 64, 65, 130):
+        act = torch.zeros((rows, k), dtype=torch.bfloat16, device="cuda")
+        route.silu_mul(act, gate_ptr, up_ptr, ld, k, rows)
+        seen.add(lin.forward_is_one_launch(rows))
+        for ydt, tdt in ((exl3.Dtype.F32, torch.float32), (exl3.Dtype.Bf16Add, torch.bfloat16)):
+            want = torch.full((rows + 1, 384), 0.5, dtype=tdt, device="cuda")
+            got = torch.full((rows + 1, 384), 0.5, dtype=tdt, device="cuda")
+            lin.forward(act.view(torch.int16), exl3.Dtype.Bf16, want, ydt, rows, ws)
+            torch.cuda.synchronize()
+            xh_want = ws.xh(rows, k).copy()
+            lin.forward_swiglu(gate_ptr, up_ptr, ld, got, ydt, rows, ws)
+            torch.cuda.synchronize()
+            assert np.array_equal(ws.xh(rows, k), xh_want), rows
+            a, b = want.view(torch.int32 if tdt == torch.float32 else torch.int16), got.view(torch.int32 if tdt == torch.float32 else torch.int16)
+            assert torch.equal(a, b), (rows, ydt)
+            assert float(got[rows].float().abs().max()) == 0.5  # the row after the batch is untouched
+    assert seen == {True, False}
+    from ferrite_amd._lib import FeError
+    with pytest.raises(FeError):
+        lin.forward_swiglu(gate_ptr, up_ptr, k - 4, got, exl3.Dtype.F32, 1, ws)
+    with pytest.raises(FeError):
+        lin.forward_swiglu(gate_ptr + 2, up_ptr, ld, got, exl3.Dtype.F32, 1, ws)
+
+
 @pytest.mark.parametrize("bits,k,ns,sks", [(4, 1024, (384, 128, 256), (2, 4, 1)), (3, 1280, (256, 640), (2, 1)),
                                            (5, 1024, (128, 128, 384, 256), (8, 1, 2, 4)), (4, 2048, (512, 384), (16, 4))])
 def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sks, monkeypatch):
