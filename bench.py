@@ -295,6 +295,21 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears, reps=20):
         res[f"m{m}"] = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
                         "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
                         "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
+        # the MLP block as the model runs it: down reads SwiGLU(gate, up) of the grouped launch's outputs and adds
+        # into the residual stream
+        resid = torch.zeros((m, d.n), dtype=torch.bfloat16, device="cuda")
+
+        def block():
+            exl3.forward_group([g, u], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=stream)
+            d.forward_swiglu(yg, yu, g.n, resid, exl3.Dtype.Bf16Add, m, ws, stream=stream)
+
+        block()
+        a, b = ev.new(), ev.new()
+        ev.record(a, stream)
+        for _ in range(reps):
+            block()
+        ev.record(b, stream)
+        res[f"m{m}"]["mlp_block_us"] = round(ev.ms(a, b) * 1e3 / reps, 2)
     # the attention projections of the same layer (40 heads of 128, 8 KV heads): q, k, v of one input grouped, then o
     blocks = exl3.default_blocks(exl3.cu_count())
     q, kk, v, o = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, n, 4, SEED, name)), blocks)
