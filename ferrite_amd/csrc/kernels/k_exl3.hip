@@ -551,22 +551,37 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
     }
     __syncthreads();
     if (last_flag) {
-        for (uint32_t row = hw; row < m; row += 8) {
-            size_t at = (size_t)row * n + col0 + 4 * l32;
-            float v[4] = {0.f, 0.f, 0.f, 0.f};
-            for (uint32_t sp0 = 0; sp0 < sk; sp0 += 8) {  // 8 splits' loads in flight, summed in split order
-                f32x4 t[8];
+        // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB splits each, so that 16 loads are
+        // in flight (an agent-scope load takes a trip to memory); every row's partials are added in split order.
+        constexpr int RB = RG == 1 ? 2 : 4, SB = 16 / RB;
+        for (uint32_t row0 = hw; row0 < m; row0 += 8 * RB) {
+            float v[RB][4];
 #pragma unroll
-                for (int b = 0; b < 8; b++) t[b] = load_agent_f32x4(z + (size_t)(sp0 + b < sk ? sp0 + b : sk - 1) * m * n + at);
+            for (int j = 0; j < RB; j++) v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.f;
+            for (uint32_t sp0 = 0; sp0 < sk; sp0 += SB) {
+                f32x4 t[RB * SB];
+#pragma unroll
+                for (int j = 0; j < RB; j++) {
+                    const uint32_t row = row0 + 8 * j < m ? row0 + 8 * j : row0;
+#pragma unroll
+                    for (int b = 0; b < SB; b++)
+                        t[j * SB + b] = load_agent_f32x4(z + ((size_t)(sp0 + b < sk ? sp0 + b : sk - 1) * m + row) * n + col0 + 4 * l32);
+                }
                 agent_loads_wait(t);
 #pragma unroll
-                for (int b = 0; b < 8; b++)
-                    if (sp0 + b < sk) {
+                for (int j = 0; j < RB; j++)
 #pragma unroll
-                        for (int e = 0; e < 4; e++) v[e] += t[b][e];
-                    }
+                    for (int b = 0; b < SB; b++)
+                        if (sp0 + b < sk) {
+#pragma unroll
+                            for (int e = 0; e < 4; e++) v[j][e] += t[j * SB + b][e];
+                        }
             }
-            finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, at);
+#pragma unroll
+            for (int j = 0; j < RB; j++) {
+                const uint32_t row = row0 + 8 * j;
+                if (row < m) finish_row(v[j], l32, svh, col0 + 4 * l32, y, y_mode, (size_t)row * n + col0 + 4 * l32);
+            }
         }
         if (tid == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
