@@ -292,8 +292,7 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
 #pragma unroll
         for (int j = j0; j < j1; j++) fb[set][j] = read_one(st + fb_base + 4096 * j, set);
     };
-    // 8 MFMAs: rows i0, i0 + 1 of the wavefront's 4 x 4 pieces, first against columns 0, 1, then 2, 3 (whose weights
-    // fragments may still be on their way when the first four issue)
+    // 8 MFMAs: rows i0, i0 + 1 of the wavefront's 4 x 4 pieces, first against columns 0, 1, then 2, 3
     auto mfmas = [&](int set, int i0) {
 #pragma unroll
         for (int jh = 0; jh < 2; jh++)
@@ -316,19 +315,24 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
     load_a(1, 0, 8);
     __syncthreads();
     read_a(0, lds, 0, 2);
-    read_b(0, lds, 0, 2);
+    read_b(0, lds, 0, 4);
 
-    // One k tile = two MFMA steps of 64, four slices of 8 MFMAs (64 cycles each), shaped like gemm_mainloop's: every
-    // slice reads 8 chunks of fragments for the MFMAs half a slice to one slice ahead; the weights of tile kt + 1 go to
-    // the other stage in slices 0 and 1 and are reloaded with tile kt + 2; the activations go out in slice 2, before the
-    // barrier; slice 3 starts on the fragments of tile kt + 1 and reloads the activation registers.
+    // One k tile = two MFMA steps of 64, four slices of 8 MFMAs (64 cycles each). Every fragment is read a whole slice
+    // before its first use (with four wavefronts queueing reads and writes the LDS answers hundreds of cycles late):
+    // the slices that work on rows 0, 1 of a step read rows 2, 3 of it (4 reads) and carry the LDS writes of tile
+    // kt + 1 (weights in the first, activations in the third); the slices on rows 2, 3 read the next step's rows 0, 1
+    // and all its weight fragments (12 reads) and reload the registers just written out (issuing those loads right after
+    // the writes, a slice earlier, made the writing slices longer by more than the loads' earlier arrival saved). The
+    // barrier sits before the last slice, which starts on the fragments of tile kt + 1. Cycle stamps per k tile (2048
+    // cycles of MFMAs): 705 / 508 / 555 / 494 and 137 at the barrier; the two slices that write LDS are bound by it
+    // (8 writes and 4 reads a wavefront are 618 cycles of the LDS pipe for the four of them).
     for (uint32_t kt = 0; kt < ktiles; kt++) {
         const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
         unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
         // slice 0: step 0, rows 0, 1
-        read_b(0, cur, 2, 4);
         read_a(0, cur, 2, 4);
         prod.store(braw, nxt + GM_A_BYTES, 0);
+        prod.store(braw, nxt + GM_A_BYTES, 1);
         mfmas(0, 0);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -339,21 +343,18 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
         __builtin_amdgcn_sched_barrier(0);
         // slice 1: step 0, rows 2, 3
         read_a(1, cur, 0, 2);
-        read_b(1, cur, 0, 2);
-        prod.store(braw, nxt + GM_A_BYTES, 1);
+        read_b(1, cur, 0, 4);
         load_b(braw, kt + 2, 0);
         load_b(braw, kt + 2, 1);
         mfmas(0, 2);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         // slice 2: step 1, rows 0, 1
-        read_b(1, cur, 2, 4);
         read_a(1, cur, 2, 4);
         store_a(nxt, 0, 8);
         mfmas(1, 0);
@@ -367,13 +368,13 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
         __syncthreads();
         // slice 3: step 1, rows 2, 3, with the first fragments of tile kt + 1
         read_a(0, nxt, 0, 2);
-        read_b(0, nxt, 0, 2);
+        read_b(0, nxt, 0, 4);
         load_a(kt + 2, 0, 8);
         mfmas(1, 2);
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
         }
