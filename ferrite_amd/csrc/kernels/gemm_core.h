@@ -165,7 +165,7 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
     read_frags(0, lds, 0);
 
     // One k tile: writes tile kt + 1 into the other LDS stage (weights from braw, half in each of the first two slices,
-    // activations from areg in the third) and reloads the registers with tile kt + 2 in the slice after they are
+    // activations from areg, a quarter in the second and the rest in the third) and reloads the registers with tile kt + 2 in the slice after they are
     // written out, so that every slice carries a similar share of the memory instructions. The
     // sched_group_barrier sequences ask for one MFMA, then a few of the other instructions, and so on, so that memory
     // instructions are issued while the matrix pipe works instead of in bursts that hold back the next MFMA.
@@ -188,6 +188,7 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         // slice 1
         read_frags(0, cur, 2);
         prod.store(braw, nxt + GM_A_BYTES, 1);
+        store_a(nxt, 0, 2);  // a quarter of the activations' LDS writes here: slice 2 is the one bound by the LDS
         load_b(braw, kt + 2, 0);
         load_b(braw, kt + 2, 1);
         mfmas(1);
@@ -202,7 +203,7 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         __builtin_amdgcn_sched_barrier(0);
         // slice 2
         read_frags(1, cur, 3);
-        store_a(nxt, 0, 8);
+        store_a(nxt, 2, 8);
         mfmas(0);
 #pragma unroll
         for (int i = 0; i < 16; i++) {
