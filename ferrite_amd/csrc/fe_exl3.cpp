@@ -18,7 +18,7 @@ constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
 constexpr uint32_t kHatRows = 513;          // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
 constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
 constexpr uint32_t kGroupMax = 4;           // FE_EXL3_GROUP_MAX: linears of one grouped launch
-constexpr uint32_t kGroupRows = 16;         // rows of a grouped launch (one row group)
+constexpr uint32_t kGroupRows = 64;         // rows of a grouped launch (one GEMV pass)
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
@@ -45,7 +45,7 @@ struct fe_exl3_kernels {
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
     fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
-    fe_function_t gemv_group[6] = {};                             // 1..16 rows, several linears of one input
+    fe_function_t gemv_group[6][4] = {};                          // several linears of one input, [bits slot][row groups - 1]
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     fe_function_t gemm_reduce = nullptr;
@@ -120,9 +120,14 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         }
         snprintf(nm, sizeof nm, "exl3_gemv_stream_b%d", kBits[i]);
         get(&k->gemv_stream[i], nm);
-        snprintf(nm, sizeof nm, "exl3_gemv_group_b%d", kBits[i]);
-        get(&k->gemv_group[i], nm);
-        if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv_group[i], 64 * 1024);
+        for (int rg = 1; rg <= 4; rg++) {
+            if (rg == 1)
+                snprintf(nm, sizeof nm, "exl3_gemv_group_b%d", kBits[i]);
+            else
+                snprintf(nm, sizeof nm, "exl3_gemv_group_b%d_r%d", kBits[i], rg);
+            get(&k->gemv_group[i][rg - 1], nm);
+            if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv_group[i][rg - 1], 64 * 1024);
+        }
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
@@ -628,7 +633,7 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
         x = 0;
     }
     void *args[] = {&g, &x, &x_mode, &k, &rows, &mode};
-    return fe_hip_launch(kern->gemv_group[bits_slot(ls[0]->bits)], programs, 1, 1, 256, 1, 1, lds, s, args);
+    return fe_hip_launch(kern->gemv_group[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 
 int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out) {

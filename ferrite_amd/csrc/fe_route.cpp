@@ -278,10 +278,10 @@ static int proj_forward(const fe_route_proj *p, const fe_route_ctx *c, uint32_t 
         first = p->cover;
     }
     for (size_t i = first; i < p->lins.size();) {
-        // Trellis linears of this input, for a batch the GEMV takes whole: one grouped launch for up to four of them
+        // Trellis linears of this input, for a batch the GEMV takes whole in one pass: one grouped launch for up to four of them
         // (the bits of each linear's own forward). The reference runs them one after the other (model.rs:384-392).
         size_t j = i;
-        if (m <= FE_X3_ROWS && c->x3())
+        if ((m <= FE_X3_ROWS || (dec >= m && m <= FE_X3_PASS)) && c->x3())
             while (j < p->lins.size() && j - i < 4 && p->lins[j].first->q && p->lins[j].first->k == lda) j++;
         if (j - i >= 2) {
             const fe_exl3_linear *qs[4];

@@ -602,7 +602,7 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
 // up): the programs of member i are first[i] .. first[i + 1] - 1, each exactly the program of the member's own launch
 // (same split, same sums, same bits), rotating the input by the member's own suh (x != nullptr) or reading the member's
 // rotated input xh (exl3_rot_in_group). The launches' start-up and tails overlap and the members' programs fill each
-// other's gaps on the CUs. 1..16 rows.
+// other's gaps on the CUs. 1..64 rows (16 RG).
 struct GemvGroup {
     uint32_t count, first[FE_EXL3_GROUP_MAX + 1];
     struct Member {
@@ -614,29 +614,33 @@ struct GemvGroup {
         uint32_t n, sk, stride_k, stride_nb, chunk, pad;
     } m[FE_EXL3_GROUP_MAX];
 };
-#define GEMV_GROUP_KERNEL(BITS)                                                                                        \
-    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_group_b##BITS(GemvGroup g, const void* x,           \
-                                                                               uint32_t x_mode, uint32_t k, uint32_t m, \
-                                                                               uint32_t y_mode) {                      \
+#define GEMV_GROUP_KERNEL(BITS, RG, NAME)                                                                              \
+    extern "C" __global__ __launch_bounds__(256, 2) void NAME(GemvGroup g, const void* x, uint32_t x_mode, uint32_t k, \
+                                                              uint32_t m, uint32_t y_mode) {                           \
         uint32_t i = 0;                                                                                                \
         while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) i++;                                                   \
         const GemvGroup::Member& mb = g.m[i];                                                                          \
-        gemv_body<BITS, 1>(mb.xh, mb.trellis, mb.svh, mb.y, mb.z, mb.counters, mb.n, k, m, mb.sk, y_mode,            \
-                           mb.stride_k, mb.stride_nb, mb.chunk, RotSrc{x, nullptr, x_mode, k}, mb.suh, nullptr,        \
-                           blockIdx.x - g.first[i]);                                                                   \
+        gemv_body<BITS, RG>(mb.xh, mb.trellis, mb.svh, mb.y, mb.z, mb.counters, mb.n, k, m, mb.sk, y_mode,             \
+                            mb.stride_k, mb.stride_nb, mb.chunk, RotSrc{x, nullptr, x_mode, k}, mb.suh, nullptr,       \
+                            blockIdx.x - g.first[i]);                                                                  \
     }
+#define GEMV_GROUP_FAMILY(BITS)                                 \
+    GEMV_GROUP_KERNEL(BITS, 1, exl3_gemv_group_b##BITS)         \
+    GEMV_GROUP_KERNEL(BITS, 2, exl3_gemv_group_b##BITS##_r2)    \
+    GEMV_GROUP_KERNEL(BITS, 3, exl3_gemv_group_b##BITS##_r3)    \
+    GEMV_GROUP_KERNEL(BITS, 4, exl3_gemv_group_b##BITS##_r4)
 GEMV_FAMILY(2)
 GEMV_FAMILY(3)
 GEMV_FAMILY(4)
 GEMV_FAMILY(5)
 GEMV_FAMILY(6)
 GEMV_FAMILY(8)
-GEMV_GROUP_KERNEL(2)
-GEMV_GROUP_KERNEL(3)
-GEMV_GROUP_KERNEL(4)
-GEMV_GROUP_KERNEL(5)
-GEMV_GROUP_KERNEL(6)
-GEMV_GROUP_KERNEL(8)
+GEMV_GROUP_FAMILY(2)
+GEMV_GROUP_FAMILY(3)
+GEMV_GROUP_FAMILY(4)
+GEMV_GROUP_FAMILY(5)
+GEMV_GROUP_FAMILY(6)
+GEMV_GROUP_FAMILY(8)
 
 // ---- decode GEMV, streamed over the whole tensor (1..16 rows) -------------------------------------------------------------
 //

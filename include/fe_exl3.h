@@ -99,7 +99,7 @@ int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows)
 int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t gate,
                                   fe_devptr_t up, uint32_t ld, fe_devptr_t y, int y_dtype, uint32_t rows,
                                   const fe_exl3_workspace *ws);
-/* Several linears applied to the same input (the q, k, v or the gate, up projections of a layer), 1..16 rows: one GEMV
+/* Several linears applied to the same input (the q, k, v or the gate, up projections of a layer), 1..64 rows: one GEMV
  * launch whose programs are those of the members' own launches, so y[i] has the bits of
  * fe_exl3_linear_forward(ls[i], ...). The launches' start-up and tails overlap and the members fill each other's gaps
  * on the CUs. Where forward() of every member rotates its own input the group does too (one launch); otherwise one

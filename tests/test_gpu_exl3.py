@@ -426,20 +426,21 @@ def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sk
         t = synth.exl3_tensor(k, n, bits, 300 + 7 * i + bits)
         lins.append(exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t) if i % 2 == 0 else exl3.DeviceExl3(t, False),
                                           exl3.Plan(sk=sk, wk=1, ver=1, occ=2)))
-    ws = exl3.Workspace(lins, 16)
-    xb = synth.activations(16, k, 11, outliers=True)
+    ws = exl3.Workspace(lins, 64)
+    xb = synth.activations(64, k, 11, outliers=True)
     xd = dev_u16(torch, xb)
     xf = xd.view(torch.bfloat16).float().contiguous()
     seen = set()
-    for rows in (1, 3, 8, 16):
+    assert exl3.forward_group_launches(lins, 65, exl3.Workspace(lins, 65)) == 0  # more than a GEMV pass: member by member
+    for rows in (1, 3, 8, 16, 17, 40, 64):
         launches = exl3.forward_group_launches(lins, rows, ws)
         assert launches == (1 if all(l.forward_is_one_launch(rows) for l in lins) else 2), rows
         seen.add(launches)
         for x, xdt in ((xd, exl3.Dtype.Bf16), (xf, exl3.Dtype.F32)):
             for ydt, tdt in ((exl3.Dtype.F32, torch.float32), (exl3.Dtype.Bf16, torch.bfloat16), (exl3.Dtype.Bf16Add, torch.bfloat16)):
                 fill = 1.5 if ydt == exl3.Dtype.Bf16Add else float("nan")
-                want = [torch.full((17, n), fill, dtype=tdt, device="cuda") for n in ns]
-                got = [torch.full((17, n), fill, dtype=tdt, device="cuda") for n in ns]
+                want = [torch.full((65, n), fill, dtype=tdt, device="cuda") for n in ns]
+                got = [torch.full((65, n), fill, dtype=tdt, device="cuda") for n in ns]
                 for lin, y in zip(lins, want):
                     lin.forward(x, xdt, y, ydt, rows, ws)
                 exl3.forward_group(lins, x, xdt, got, ydt, rows, ws)
