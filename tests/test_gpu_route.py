@@ -196,6 +196,18 @@ def test_proj_places_parts_as_the_reference(env):
     got = bits(out)
     assert np.array_equal(got[:6, :INTER], want_g[:6]) and np.array_equal(got[:6, INTER:], want_u[:6])
     assert np.array_equal(got[6:], bits(yp)[6:])
+
+    # no fused prompt linear, 40 rows that are all decode / verify rows: one GEMV pass, the two linears as one grouped
+    # launch, each writing its own [m][n] block
+    plain = route.Proj([(g, [INTER]), (u, [INTER])])
+    c.dec = 40
+    out = torch.zeros((40, 2 * INTER), dtype=torch.bfloat16, device="cuda")
+    parts = plain.forward(c, out, x, HIDDEN, 40)
+    torch.cuda.synchronize()
+    assert parts == [(out.data_ptr(), INTER), (out.data_ptr() + 40 * INTER * 2, INTER)]
+    flat = bits(out).reshape(-1)
+    assert np.array_equal(flat[:40 * INTER].reshape(40, INTER), want_g[:40])
+    assert np.array_equal(flat[40 * INTER:].reshape(40, INTER), want_u[:40])
     c.dec = 0
 
 
