@@ -200,6 +200,7 @@ def test_proj_places_parts_as_the_reference(env):
     # no fused prompt linear, 40 rows that are all decode / verify rows: one GEMV pass, the two linears as one grouped
     # launch, each writing its own [m][n] block
     plain = route.Proj([(g, [INTER]), (u, [INTER])])
+    assert e.exl3.forward_group_launches([e.q_gate, e.q_up], 40, e.xws) in (1, 2)
     c.dec = 40
     out = torch.zeros((40, 2 * INTER), dtype=torch.bfloat16, device="cuda")
     parts = plain.forward(c, out, x, HIDDEN, 40)
