@@ -354,6 +354,9 @@ __device__ __forceinline__ f32x4 row_scales(const uint16_t* svh, uint32_t col) {
     return (f32x4){f16_bits_to_f32(s[0] & 0xffff), f16_bits_to_f32(s[0] >> 16), f16_bits_to_f32(s[1] & 0xffff),
                    f16_bits_to_f32(s[1] >> 16)};
 }
+#ifndef FE_STAGE_NB1
+#define FE_STAGE_NB1 4
+#endif
 #define GEMV_RED_PITCH 132  // floats a row of the 128-column partial sums (16-byte aligned, banks spread)
 
 // y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for m <= 16 RG rows. grid (n / 128 * sk), 256 threads. The rotated
@@ -453,11 +456,24 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
                 }
             }
         } else {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
-            const uint32_t chunks16 = cs * 8;  // 16-byte pieces a row
-            for (uint32_t i = tid; i < m * chunks16; i += 256) {
-                uint32_t row = i / chunks16, c = i - row * chunks16;
-                u32x4 v = *(const u32x4*)(xh + (size_t)row * k + (size_t)(kt0 + 4 * c0) * 16 + c * 8);
-                *(u32x4*)(lds + row * xpitch + c * 16) = v;
+            // (NB loads in flight a thread: one after the other they cost a trip to L2 each, 8 per chunk at 64 rows;
+            // fewer for one row group, whose kernels would lose a resident wavefront to the registers)
+            constexpr int NB = RG == 1 ? FE_STAGE_NB1 : 8;
+            const uint32_t chunks16 = cs * 8, total = m * chunks16;  // 16-byte pieces a row, pieces in all
+            const uint16_t* xsrc = xh + (size_t)(kt0 + 4 * c0) * 16;
+            for (uint32_t i0 = tid; i0 < total; i0 += 256 * NB) {
+                u32x4 v[NB];
+                uint32_t off[NB];
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const uint32_t i = i0 + 256 * j < total ? i0 + 256 * j : i0;  // past the end: a piece again, not stored
+                    const uint32_t row = i / chunks16, c = i - row * chunks16;
+                    v[j] = *(const u32x4*)(xsrc + (size_t)row * k + c * 8);
+                    off[j] = row * xpitch + c * 16;
+                }
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    if (i0 + 256 * j < total) *(u32x4*)(lds + off[j]) = v[j];
             }
         }
         __syncthreads();
