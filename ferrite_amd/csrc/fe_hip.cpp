@@ -210,7 +210,7 @@ int fe_hip_graph_end(fe_stream_t s, fe_graph_t *out) {
     int c = fe_check_hip((int)hipStreamEndCapture((hipStream_t)s, &g->g), "hipStreamEndCapture");
     if (!c) c = fe_check_hip((int)hipGraphInstantiate(&g->e, g->g, nullptr, nullptr, 0), "hipGraphInstantiate");
     if (c) {
-        if (g->g) hipGraphDestroy(g->g);
+        if (g->g) (void)hipGraphDestroy(g->g);
         delete g;
         return c;
     }
@@ -227,8 +227,8 @@ int fe_hip_graph_launch(fe_graph_t g, fe_stream_t s) {
 int fe_hip_graph_destroy(fe_graph_t g) {
     if (!g) return 0;
     fe_graph *p = (fe_graph *)g;
-    hipGraphExecDestroy(p->e);
-    hipGraphDestroy(p->g);
+    (void)hipGraphExecDestroy(p->e);
+    (void)hipGraphDestroy(p->g);
     delete p;
     return 0;
 }

@@ -778,7 +778,7 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh
         if (old == 3) {
             uint32_t g_old = 0;
             if (lane == 0) g_old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            finisher = __builtin_amdgcn_readfirstlane(g_old) == last_prog - first_prog;
+            finisher = (uint32_t)__builtin_amdgcn_readfirstlane(g_old) == last_prog - first_prog;
         }
         if (finisher) {
             // add the segments in program order, rotate, scale, store; two rows at a time, 8 segments' loads in flight
