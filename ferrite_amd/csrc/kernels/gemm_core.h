@@ -4,8 +4,9 @@
 // SIMD). The large tile is what keeps the kernel off the memory system: a k tile of 64 brings 32 KB of activations and
 // the packed weights of 256 columns from L2 for 64 MFMAs a wavefront (half the bytes per flop of a 256 x 128 tile), and
 // moves 64 KB into and 128 KB out of LDS in the time of 2048 MFMA cycles. LDS holds two k tiles (one barrier per
-// k tile). Rows of an LDS tile are 64 f16 = 8 chunks of 16 bytes, chunk c of row r stored at position c ^ (r & 7), so
-// the lanes that read one chunk column of 8 consecutive rows hit 8 different bank groups (measured conflict-free).
+// k tile). Rows of an LDS tile are 64 f16 = 8 chunks of 16 bytes, chunk c of row r stored at position
+// c ^ (r & 7) ^ ((r >> 3) & 1) (gm_swz below), which leaves neither the tile writes nor the fragment reads a bank
+// conflict (SQ_LDS_BANK_CONFLICT reads 0 for every GEMM kernel).
 #pragma once
 #include "kcommon.h"
 

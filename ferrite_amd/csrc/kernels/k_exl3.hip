@@ -962,8 +962,8 @@ __device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, 
 // ---- prefill over decoded weights -----------------------------------------------------------------------------------
 //
 // For many rows the trellis is decoded once per call into `hat`, fp16, as the very images the GEMM keeps in LDS: block
-// (tn, kt) of 32 KB = rows n = 256 tn .. + 255 of k tile kt, 128 bytes a row, 16-byte chunk c of row r at position
-// c ^ (r & 7). The GEMM over it then copies blocks instead of decoding, with the same fragments, the same MFMA order and
+// (tn, kt) of 32 KB = rows n = 256 tn .. + 255 of k tile kt, 128 bytes a row, 16-byte chunk c of row r at the position gm_swz
+// gives it. The GEMM over it then copies blocks instead of decoding, with the same fragments, the same MFMA order and
 // so the same bits as exl3_gemm_b*.
 
 // grid (n / 128, gy), 256 threads; program (nb, j) decodes k tiles j, j + gy, ... of column block nb with the lane
