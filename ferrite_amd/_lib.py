@@ -111,6 +111,14 @@ SYMBOLS = {
     "fe_route_ctx_destroy": (I, [P]),
     "fe_route_ctx_set_dec": (I, [P, U32]),
     "fe_route_ctx_set_x3_gemm": (I, [P, I]),
+    "fe_route_ctx_set_bf16": (I, [P, P]),
+    "fe_route_linear_set_bf16": (I, [P, U64]),
+    # fe_bf16.h
+    "fe_bf16_kernels_load": (I, [PP]),
+    "fe_bf16_kernels_destroy": (I, [P]),
+    "fe_bf16_gemv": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
+    "fe_bf16_gemm": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
+    "fe_bf16_linear_forward": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32, U32]),
     "fe_route_linear_create": (I, [PP, C.c_char_p, U32, U32, P, P]),
     "fe_route_linear_destroy": (I, [P]),
     "fe_route_linear_forward": (I, [P, P, U64, U32, U64, U32, U32, U64]),

@@ -19,8 +19,8 @@ HIPCC = os.path.join(ROCM, "bin", "hipcc")
 # -packed-fp32-ops off: the compiler must not form v_pk_*_f32 from the float code in these kernels
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-mcode-object-version=5",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-KERNELS = ["k_exl3", "k_fp4", "k_route"]
-HOST = ["fe_hip.cpp", "fe_exl3.cpp", "fe_fp4.cpp", "fe_route.cpp"]
+KERNELS = ["k_exl3", "k_fp4", "k_route", "k_bf16"]
+HOST = ["fe_hip.cpp", "fe_exl3.cpp", "fe_fp4.cpp", "fe_bf16.cpp", "fe_route.cpp"]
 
 
 def _run(cmd, **kw):

@@ -1,0 +1,130 @@
+// fe_bf16: host side of the plain bf16 linear (see include/fe_bf16.h). Follows crates/fe-model/src/model.rs:310-345;
+// the kernels are ferrite_amd/csrc/kernels/k_bf16.hip.
+#include "fe_bf16.h"
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "fe_exl3.h"  // error codes
+#include "fe_internal.h"
+
+namespace {
+constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // GM_LDS_TILES
+constexpr uint32_t kTileM = 256, kTileN = 256;           // GM_BM, GM_BN
+constexpr uint32_t kGemvRows = 8;                        // rows of one GEMV pass (model.rs:326)
+constexpr uint32_t kSmallBatch = 16;                     // X3_ROWS: batches up to here are decode rows (model.rs:172)
+}  // namespace
+
+struct fe_bf16_kernels {
+    fe_module_t module = nullptr;
+    fe_function_t gemm = nullptr, reduce = nullptr, gemv[4] = {}, gemv_kw[4] = {};  // GEMV forms for 1, 2, 4, 8 rows
+    uint32_t cus = 0;
+    FeBuf part;
+};
+
+static int check(const char *fn, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda, fe_devptr_t w, fe_devptr_t res,
+                 uint32_t n, uint32_t k) {
+    if (!y || !x || !w) return fe_set_error(FE_ERR_ARG, fn, "null pointer");
+    if (!n || !k || n % 8 || k % 64) {
+        char msg[120];
+        snprintf(msg, sizeof msg, "bf16 linear n %u k %u (n %% 8 == 0, k %% 64 == 0)", n, k);
+        return fe_set_error(FE_ERR_SHAPE, fn, msg);
+    }
+    if (lda % 8 || lda < k || x % 16 || w % 16) return fe_set_error(FE_ERR_ARG, fn, "x / w rows must be 16-byte aligned, lda >= k");
+    if (ldy % 4 || ldy < n || y % 8 || (res && res % 8)) return fe_set_error(FE_ERR_ARG, fn, "y / res rows must be 8-byte aligned, ldy >= n");
+    return 0;
+}
+
+extern "C" {
+
+int fe_bf16_kernels_load(fe_bf16_kernels **out) {
+    if (!out) return fe_set_error(FE_ERR_ARG, "fe_bf16_kernels_load", "null out");
+    auto *k = new fe_bf16_kernels;
+    int c = fe_load_module(&k->module, "FE_BF16_HSACO", fe_k_bf16_hsaco, fe_k_bf16_hsaco_end);
+    if (!c) c = fe_hip_module_get_function(&k->gemm, k->module, "fe_gemm_bf16");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->reduce, k->module, "fe_gemm_bf16_reduce");
+    for (int i = 0; i < 4 && !c; i++) {
+        char nm[32];
+        snprintf(nm, sizeof nm, "fe_gemv_bf16_r%d", 1 << i);
+        c = fe_hip_module_get_function(&k->gemv[i], k->module, nm);
+        snprintf(nm, sizeof nm, "fe_gemv_bf16_kw_r%d", 1 << i);
+        if (!c) c = fe_hip_module_get_function(&k->gemv_kw[i], k->module, nm);
+    }
+    int cus = 0;
+    if (!c) c = fe_hip_cu_count(&cus);
+    k->cus = (uint32_t)cus;
+    if (!c) c = k->part.alloc((size_t)kFeGemmSlotsPerCu * k->cus * kFeGemmPartBytes);
+    if (c) {
+        fe_bf16_kernels_destroy(k);
+        return c;
+    }
+    *out = k;
+    return 0;
+}
+
+int fe_bf16_kernels_destroy(fe_bf16_kernels *k) {
+    if (!k) return 0;
+    k->part.release();
+    if (k->module) fe_hip_module_unload(k->module);
+    delete k;
+    return 0;
+}
+
+int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda,
+                 fe_devptr_t w, fe_devptr_t res, uint32_t m, uint32_t n, uint32_t k) {
+    const char *fn = "fe_bf16_gemv";
+    if (!kern) return fe_set_error(FE_ERR_ARG, fn, "null kernels");
+    if (m == 0) return 0;
+    if (m > kGemvRows) return fe_set_error(FE_ERR_ARG, fn, "at most 8 rows a call");
+    FE_TRY(check(fn, y, ldy, x, lda, w, res, n, k));
+    const int form = m <= 1 ? 0 : m <= 2 ? 1 : m <= 4 ? 2 : 3;
+    const bool narrow = n <= 512;  // model.rs:319 (k % 64 == 0 holds for every k this library takes)
+    void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy};
+    return fe_hip_launch(narrow ? kern->gemv_kw[form] : kern->gemv[form], narrow ? n : (n + 15) / 16, 1, 1, 256, 1, 1, 0, s, args);
+}
+
+int fe_bf16_gemm(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda,
+                 fe_devptr_t w, fe_devptr_t res, uint32_t m, uint32_t n, uint32_t k) {
+    const char *fn = "fe_bf16_gemm";
+    if (!kern) return fe_set_error(FE_ERR_ARG, fn, "null kernels");
+    if (m == 0) return 0;
+    FE_TRY(check(fn, y, ldy, x, lda, w, res, n, k));
+    if ((uint64_t)m * lda * 2 >= (1ull << 32) || (uint64_t)n * k * 2 >= (1ull << 32))
+        return fe_set_error(FE_ERR_UNSUPPORTED, fn, "operand of 4 GB or more");
+    const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
+    // weights at least as large as the activations: column tiles are dealt to the XCDs, each weight panel through one L2
+    // (gemm_raster with group 0); else row tiles in groups of 8
+    uint32_t group = n >= m ? 0 : tiles_m < 8 ? tiles_m : 8;
+    if (const char *e = getenv("FE_BF16_GROUP")) group = (uint32_t)atoi(e);
+    if (group > tiles_m) group = tiles_m;
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes));
+    uint32_t full = gs.full, splits = gs.splits;
+    fe_devptr_t part = kern->part.p;
+    void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy, &group, &full, &splits, &part};
+    FE_TRY(fe_hip_launch(kern->gemm, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (!gs.cut()) return 0;
+    void *rargs[] = {&y, &part, &res, &m, &n, &ldy, &group, &full, &splits};
+    return fe_hip_launch(kern->reduce, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
+}
+
+int fe_bf16_linear_forward(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x,
+                           uint32_t lda, fe_devptr_t w, fe_devptr_t res, uint32_t m, uint32_t n, uint32_t k, uint32_t dec) {
+    const char *fn = "fe_bf16_linear_forward";
+    if (!kern) return fe_set_error(FE_ERR_ARG, fn, "null kernels");
+    if (m == 0) return 0;
+    FE_TRY(check(fn, y, ldy, x, lda, w, res, n, k));
+    // decode / verify rows: the GEMV in passes of up to 8 rows, so that a row's bits do not depend on the batch
+    uint32_t d = m <= kSmallBatch ? m : (dec < m ? dec : m);
+    if (k % 256) d = 0;
+    for (uint32_t r = 0; r < d; r += kGemvRows) {
+        const uint32_t mr = d - r < kGemvRows ? d - r : kGemvRows;
+        FE_TRY(fe_bf16_gemv(kern, s, y + (size_t)r * ldy * 2, ldy, x + (size_t)r * lda * 2, lda, w,
+                            res ? res + (size_t)r * ldy * 2 : 0, mr, n, k));
+    }
+    if (d == m) return 0;
+    return fe_bf16_gemm(kern, s, y + (size_t)d * ldy * 2, ldy, x + (size_t)d * lda * 2, lda, w,
+                        res ? res + (size_t)d * ldy * 2 : 0, m - d, n, k);
+}
+
+}  // extern "C"

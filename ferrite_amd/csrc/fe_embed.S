@@ -19,4 +19,10 @@ fe_k_route_hsaco:
     .incbin "k_route.hsaco"
     .global fe_k_route_hsaco_end
 fe_k_route_hsaco_end:
+    .balign 4096
+    .global fe_k_bf16_hsaco
+fe_k_bf16_hsaco:
+    .incbin "k_bf16.hsaco"
+    .global fe_k_bf16_hsaco_end
+fe_k_bf16_hsaco_end:
     .section .note.GNU-stack,"",@progbits

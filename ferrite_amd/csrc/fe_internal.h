@@ -23,6 +23,8 @@ extern "C" const unsigned char fe_k_fp4_hsaco[];
 extern "C" const unsigned char fe_k_fp4_hsaco_end[];
 extern "C" const unsigned char fe_k_route_hsaco[];
 extern "C" const unsigned char fe_k_route_hsaco_end[];
+extern "C" const unsigned char fe_k_bf16_hsaco[];
+extern "C" const unsigned char fe_k_bf16_hsaco_end[];
 
 // The embedded image, or the file the environment variable names.
 int fe_load_module(fe_module_t *out, const char *env, const unsigned char *begin, const unsigned char *end);

@@ -40,6 +40,7 @@ struct fe_route_ctx {
     const fe_exl3_workspace *xws = nullptr;
     const fe_fp4_kernels *fk = nullptr;
     const fe_fp4_workspace *fws = nullptr;
+    const fe_bf16_kernels *bk = nullptr;
     fe_stream_t s = nullptr;
     FeBuf tmp;  // [FE_DEC_MAX][max_proj] bf16
     uint32_t max_proj = 0, dec = 0;
@@ -53,6 +54,7 @@ struct fe_route_linear {
     uint32_t n = 0, k = 0;
     const fe_exl3_linear *q = nullptr;
     const fe_fp4_linear *p = nullptr;
+    fe_devptr_t w = 0;  // bf16 weights [n][k]
 };
 
 struct fe_route_proj {
@@ -98,9 +100,13 @@ static int linear_forward(const fe_route_linear *l, const fe_route_ctx *c, uint3
         }
         return linear_forward(l, c, m, y, ldy, x, lda, m, res);
     }
-    char msg[200];
-    snprintf(msg, sizeof msg, "%s: no weights for %u rows (bf16 weights are not part of this library)", l->name.c_str(), m);
-    return fe_set_error(FE_ERR_UNSUPPORTED, fn, msg);
+    if (!l->w || !c->bk) {
+        char msg[200];
+        snprintf(msg, sizeof msg, "%s: no bf16 weights for %u rows", l->name.c_str(), m);
+        return fe_set_error(FE_ERR_UNSUPPORTED, fn, msg);
+    }
+    // plain bf16 weights: GEMV passes for the decode rows, the GEMM for the rest (model.rs:310-345)
+    return fe_bf16_linear_forward(c->bk, c->s, y, ldy, x, lda, l->w, res, m, l->n, l->k, dec);
 }
 
 extern "C" {
@@ -133,6 +139,19 @@ int fe_route_ctx_destroy(fe_route_ctx *c) {
 int fe_route_ctx_set_dec(fe_route_ctx *c, uint32_t dec) {
     if (!c) return fe_set_error(FE_ERR_ARG, "fe_route_ctx_set_dec", "null context");
     c->dec = dec;
+    return 0;
+}
+
+int fe_route_ctx_set_bf16(fe_route_ctx *c, const fe_bf16_kernels *bk) {
+    if (!c) return fe_set_error(FE_ERR_ARG, "fe_route_ctx_set_bf16", "null context");
+    c->bk = bk;
+    return 0;
+}
+
+int fe_route_linear_set_bf16(fe_route_linear *l, fe_devptr_t w) {
+    if (!l) return fe_set_error(FE_ERR_ARG, "fe_route_linear_set_bf16", "null linear");
+    if (w % 16) return fe_set_error(FE_ERR_ARG, "fe_route_linear_set_bf16", "weights must be 16-byte aligned");
+    l->w = w;
     return 0;
 }
 

@@ -100,7 +100,8 @@ __device__ __forceinline__ GemmWork gemm_work(uint32_t pid, uint32_t tiles_m, ui
 // the registers that carry a tile from memory to LDS are reloaded with tile kt + 2 right after they are written out; the LDS writes of tile kt + 1 are issued between the MFMAs of tile kt; MFMA fragments are read from LDS one 16-wide k slice ahead. The barrier sits before the last slice, whose
 // fragments are already in registers, so the first fragments of tile kt + 1 load under the last 16 MFMAs of tile kt.
 // Loads past the end re-read the last tile / row and are never used: the loop body has no branches.
-template <class Producer>
+// BF16: the operands are bf16 (v_mfma_f32_32x32x16_bf16) instead of fp16; everything else is bytes and the same.
+template <class Producer, bool BF16 = false>
 __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, uint32_t lda, uint32_t m, uint32_t kt0,
                                               uint32_t ktiles, uint32_t m0, Producer& prod, unsigned char* lds,
                                               f32x16 (&acc)[4][4]) {
@@ -157,7 +158,11 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         for (int i = 0; i < 4; i++)
 #pragma unroll
             for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
+                if constexpr (BF16)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][i]),
+                                                                         __builtin_bit_cast(bf16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
     typename Producer::Raw braw;

@@ -35,6 +35,11 @@ class LinCtx:
         check(_lib.lib().fe_route_ctx_set_dec(self.h, d))
         self._dec = d
 
+    def set_bf16(self, kernels):
+        """LinCtx::k: the plain bf16 kernels (ferrite_amd.bf16.Kernels), or None."""
+        self._bf16 = kernels
+        check(_lib.lib().fe_route_ctx_set_bf16(self.h, kernels.h if kernels is not None else None))
+
     def set_x3_gemm(self, on: bool):
         check(_lib.lib().fe_route_ctx_set_x3_gemm(self.h, int(on)))
 
@@ -45,14 +50,18 @@ class LinCtx:
 
 
 class Linear:
-    """y[M][N] = x[M][K] . W[N][K]^T with q = the EXL3 linear and / or p = the prompt linear (model.rs:260-346)."""
+    """y[M][N] = x[M][K] . W[N][K]^T with q = the EXL3 linear, p = the prompt linear, w = bf16 weights [n][k] (a torch
+    tensor on the device); any of them may be None (model.rs:260-346)."""
 
-    def __init__(self, name: str, n: int, k: int, q=None, p=None):
+    def __init__(self, name: str, n: int, k: int, q=None, p=None, w=None):
         _lib.init()
-        self.name, self.n, self.k, self.q, self.p = name, n, k, q, p
+        self.name, self.n, self.k, self.q, self.p, self.w = name, n, k, q, p, w
         self.h = C.c_void_p()
         check(_lib.lib().fe_route_linear_create(C.byref(self.h), name.encode(), n, k, q.h if q is not None else None,
                                                 p.h if p is not None else None))
+        if w is not None:
+            assert tuple(w.shape) == (n, k) and w.is_contiguous() and w.element_size() == 2
+            check(_lib.lib().fe_route_linear_set_bf16(self.h, w.data_ptr()))
 
     def forward(self, c: LinCtx, y, ldy: int, x, lda: int, m: int, res=None):
         check(_lib.lib().fe_route_linear_forward(self.h, c.h, y.data_ptr(), ldy, x.data_ptr(), lda, m,

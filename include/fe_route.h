@@ -3,15 +3,15 @@
  * them: decode / verify rows through the EXL3 trellis GEMV (whatever the batch size, so a row's bits do not depend on
  * the batch), prompt rows through the NVFP4 / FP8 prompt linear, fused prompt projections, and the MLP block built from
  * them. C ABI of crates/fe-model/src/model.rs:172-203 (constants, LinCtx), :260-346 (Linear::forward), :349-403 (Proj),
- * :3160-3203 (the MLP block). The plain bf16 weight form of the reference's Linear (its own GEMV/GEMM kernels) is not
- * part of this library: a linear with neither a trellis nor a prompt form fails as the reference does for a linear
- * without weights.
+ * :3160-3203 (the MLP block). A linear with none of the three weight forms (trellis, prompt, plain bf16) fails as the
+ * reference does for a linear without weights.
  *
  * All activations are bf16, row-major. Errors are return codes as in fe_exl3.h (fe_hip_last_error() has the text).
  */
 #ifndef FE_ROUTE_H
 #define FE_ROUTE_H
 
+#include "fe_bf16.h"
 #include "fe_exl3.h"
 #include "fe_fp4.h"
 
@@ -24,7 +24,7 @@ extern "C" {
 #define FE_DEC_MAX 64 /* most decode / verify rows of a batch (model.rs:203) */
 
 typedef struct fe_route_ctx fe_route_ctx;       /* LinCtx, model.rs:189-200 */
-typedef struct fe_route_linear fe_route_linear; /* Linear, model.rs:260-273 (q and p forms) */
+typedef struct fe_route_linear fe_route_linear; /* Linear, model.rs:260-273 */
 typedef struct fe_route_proj fe_route_proj;     /* Proj, model.rs:351-359 */
 
 /* LinCtx: the EXL3 kernels + workspace (either may be NULL: no trellis path), the prompt kernels + workspace (NULL: no
@@ -35,6 +35,8 @@ int fe_route_ctx_create(fe_route_ctx **out, const fe_exl3_kernels *xk, const fe_
 int fe_route_ctx_destroy(fe_route_ctx *c);
 /* LinCtx::dec (model.rs:197-199): the first `dec` rows of the next batches are decode / verify rows. */
 int fe_route_ctx_set_dec(fe_route_ctx *c, uint32_t dec);
+/* LinCtx::k (model.rs:191): the plain bf16 kernels, NULL (default) = no bf16 path. Borrowed. */
+int fe_route_ctx_set_bf16(fe_route_ctx *c, const fe_bf16_kernels *bk);
 /* What prompt rows of a linear without prompt weights run on: 1 (default) = one call of the trellis linear with all of
  * them, which above 64 rows is the MFMA GEMM (needs an EXL3 workspace for that many rows); 0 = passes of FE_X3_PASS rows
  * through the GEMV as the reference (model.rs:305-309). No counterpart in the reference, which has no trellis GEMM. */
@@ -44,6 +46,8 @@ int fe_route_ctx_set_x3_gemm(fe_route_ctx *c, int on);
  * Borrowed. */
 int fe_route_linear_create(fe_route_linear **out, const char *name, uint32_t n, uint32_t k, const fe_exl3_linear *q,
                            const fe_fp4_linear *p);
+/* Linear::w (model.rs:265): bf16 weights [n][k] on the device (0 = none), used where neither q nor p applies. Borrowed. */
+int fe_route_linear_set_bf16(fe_route_linear *l, fe_devptr_t w);
 int fe_route_linear_destroy(fe_route_linear *l);
 /* Linear::forward (model.rs:275-346): y (row stride ldy) = x (row stride lda) . W^T for m rows; with res (stride ldy):
  * y = bf16(bf16(x . W) + res). On the trellis path res must be y itself (the add happens in the GEMV's epilogue). */

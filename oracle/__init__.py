@@ -363,6 +363,26 @@ def ref_gemm(a, w, threads=0):
     return y
 
 
+def bf16_linear_ref(x_bits, w_bits, res_bits=None, threads=0):
+    """The plain bf16 linear of the caller (kernels/k-core/src/gemm.rs:128-167): x [m][k], w [n][k] as bf16 bit
+    patterns (uint16) -> (y bits [m][n], the f64-accumulated sums as f32). y = bf16(sum); with res: bf16(bf16(sum) + res),
+    two roundings (gemm.rs:152-158). Pinned in tests/test_oracle_bf16.py by one-hot weights (y == x), all-ones operands
+    (y == k), a brute-force loop on a tiny case and a residual whose two roundings differ from one."""
+    x = (np.ascontiguousarray(x_bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+    w = (np.ascontiguousarray(w_bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+    acc = ref_gemm(x, w, threads)
+
+    def rne(f):
+        b = np.ascontiguousarray(f, np.float32).view(np.uint32)
+        return ((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint16)
+
+    y = rne(acc)
+    if res_bits is not None:
+        r = (np.ascontiguousarray(res_bits, np.uint16).astype(np.uint32) << 16).view(np.float32)
+        y = rne((y.astype(np.uint32) << 16).view(np.float32) + r)
+    return y, acc
+
+
 def select(src, row_len, keep, c0, c1):
     src = _c(src, np.uint8).reshape(-1)
     kp = _c(np.array(keep, dtype=np.uint64).reshape(-1), np.uint64)

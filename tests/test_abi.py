@@ -13,7 +13,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def declared_symbols():
     names = []
-    for h in ("fe_hip.h", "fe_exl3.h", "fe_fp4.h", "fe_route.h"):
+    for h in sorted(os.listdir(os.path.join(ROOT, "include"))):
         text = open(os.path.join(ROOT, "include", h)).read()
         text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
         names += re.findall(r"\b(fe_[a-z0-9_]+)\s*\(", text)
@@ -36,12 +36,12 @@ def test_embedded_code_objects_are_gfx950_elf():
     out = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ROOT, "ferrite_amd", "libferrite_amd.so")],
                          stdout=subprocess.PIPE, text=True).stdout
     # the code objects are private data of the library; check them through the build directory instead
-    for k in ("k_exl3", "k_fp4", "k_route"):
+    for k in ("k_exl3", "k_fp4", "k_route", "k_bf16"):
         p = os.path.join(ROOT, "ferrite_amd", "_build", k + ".hsaco")
         if os.path.exists(p):
             head = open(p, "rb").read(20)
             assert head[:4] == b"\x7fELF" and head[18] == 0xE0  # EM_AMDGPU
-    assert "fe_exl3_linear_forward" in out and "fe_fp4_linear_forward" in out
+    assert "fe_exl3_linear_forward" in out and "fe_fp4_linear_forward" in out and "fe_bf16_linear_forward" in out
 
 
 def synthetic(k, n, bits):
