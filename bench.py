@@ -510,6 +510,29 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     ms = ev.ms(a, b) / reps
     res["fp8_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1), "mfma": "f32_32x32x64_f8f6f4 (e4m3 x e4m3)",
                              "frac_mfma_fp8_peak": round(flops / ms / 1e9 / MFMA_FP8_PEAK_TFLOPS, 4)}
+    del f8, y8
+    # the plain bf16 weight form of the same linear (the caller's third form): GEMM at M = 2048 on the bf16 MFMA, GEMV
+    # at 1 and 8 rows, which reads 2 bytes a weight and nothing else of size; three weight copies in turn, 535 MB, so
+    # that no launch finds its weights in the 256 MB of last-level cache
+    from ferrite_amd import bf16
+    bk = bf16.Kernels.load()
+    gen = torch.Generator(device="cuda").manual_seed(SEED)
+    ws_b = [(torch.randn((n, k), generator=gen, device="cuda") * k ** -0.5).to(torch.bfloat16) for _ in range(3)]
+    yb = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    ms = timed(lambda: bf16.gemm(bk, yb, n, xf, k, ws_b[0], m))
+    res["bf16_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                              "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    for rows in (1, 8):
+        reps = 30
+        pairs = [(ev.new(), ev.new()) for _ in range(reps)]
+        bf16.gemv(bk, yb, n, xf, k, ws_b[0], rows)
+        for i, (a, b) in enumerate(pairs):
+            ev.record(a, stream)
+            bf16.gemv(bk, yb, n, xf, k, ws_b[i % 3], rows)
+            ev.record(b, stream)
+        us = sum(ev.ms(a, b) for a, b in pairs) / reps * 1e3
+        res[f"bf16_5120x17408_m{rows}"] = {"gemv_us": round(us, 2), "GB/s": round(2.0 * n * k / us / 1e3, 1),
+                                          "frac_hbm_peak": round(2.0 * n * k / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res
 
 

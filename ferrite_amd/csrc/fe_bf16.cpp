@@ -17,10 +17,16 @@ constexpr uint32_t kSmallBatch = 16;                     // X3_ROWS: batches up 
 
 struct fe_bf16_kernels {
     fe_module_t module = nullptr;
-    fe_function_t gemm = nullptr, reduce = nullptr, gemv[4] = {}, gemv_kw[4] = {};  // GEMV forms for 1, 2, 4, 8 rows
+    fe_function_t gemm = nullptr, reduce = nullptr;
+    fe_function_t gemv[4][4] = {};  // [rows 1, 2, 4, 8][columns of a program 1, 2, 4, 8]
     uint32_t cus = 0;
     FeBuf part;
 };
+
+// log2 of the columns a GEMV program takes: 4 measured best for 1..8 rows on 5120 x 17408, 17408 x 5120 and
+// 5120 x 5120 (at 8 rows 48 us against 86 us with one column, 51 us with eight); narrow linears take fewer so that the
+// grid still has a few programs a CU
+static int gemv_cols(uint32_t n) { return n >= 4096 ? 2 : n >= 1024 ? 1 : 0; }
 
 static int check(const char *fn, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda, fe_devptr_t w, fe_devptr_t res,
                  uint32_t n, uint32_t k) {
@@ -44,13 +50,12 @@ int fe_bf16_kernels_load(fe_bf16_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->gemm, k->module, "fe_gemm_bf16");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->reduce, k->module, "fe_gemm_bf16_reduce");
-    for (int i = 0; i < 4 && !c; i++) {
-        char nm[32];
-        snprintf(nm, sizeof nm, "fe_gemv_bf16_r%d", 1 << i);
-        c = fe_hip_module_get_function(&k->gemv[i], k->module, nm);
-        snprintf(nm, sizeof nm, "fe_gemv_bf16_kw_r%d", 1 << i);
-        if (!c) c = fe_hip_module_get_function(&k->gemv_kw[i], k->module, nm);
-    }
+    for (int i = 0; i < 4 && !c; i++)
+        for (int j = 0; j < 4 && !c; j++) {
+            char nm[32];
+            snprintf(nm, sizeof nm, "fe_gemv_bf16_r%d_c%d", 1 << i, 1 << j);
+            c = fe_hip_module_get_function(&k->gemv[i][j], k->module, nm);
+        }
     int cus = 0;
     if (!c) c = fe_hip_cu_count(&cus);
     k->cus = (uint32_t)cus;
@@ -79,9 +84,12 @@ int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint
     if (m > kGemvRows) return fe_set_error(FE_ERR_ARG, fn, "at most 8 rows a call");
     FE_TRY(check(fn, y, ldy, x, lda, w, res, n, k));
     const int form = m <= 1 ? 0 : m <= 2 ? 1 : m <= 4 ? 2 : 3;
-    const bool narrow = n <= 512;  // model.rs:319 (k % 64 == 0 holds for every k this library takes)
+    // columns of a program: the results do not depend on it. More columns read x less often (x is read once per program
+    // and step, the weights once in all), fewer give more programs
+    int cols = gemv_cols(n);
+    if (const char *e = getenv("FE_BF16_NC")) cols = atoi(e) >= 8 ? 3 : atoi(e) >= 4 ? 2 : atoi(e) >= 2 ? 1 : 0;
     void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy};
-    return fe_hip_launch(narrow ? kern->gemv_kw[form] : kern->gemv[form], narrow ? n : (n + 15) / 16, 1, 1, 256, 1, 1, 0, s, args);
+    return fe_hip_launch(kern->gemv[form][cols], n >> cols, 1, 1, 256, 1, 1, 0, s, args);
 }
 
 int fe_bf16_gemm(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda,

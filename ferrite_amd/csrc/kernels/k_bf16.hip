@@ -115,11 +115,9 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-#define BF16_GEMV_COLS 4  // output columns of one wavefront
-
-// One wavefront: the sums of x rows 0..MR-1 (rows >= m repeat row m - 1) with NC weight rows over the
-// 16-byte chunks [c0, c1) of K, lane L taking chunks c0 + L, c0 + L + 64, ... A row's sums do not depend on MR or m:
-// a lane adds its chunks in ascending order, one v_dot2 per element pair, then the lanes meet in a butterfly.
+// One wavefront: the sums of x rows 0..MR-1 (rows >= m repeat row m - 1) with NC weight rows over the 16-byte chunks
+// [c0, c1) of K, lane L taking chunks c0 + L, c0 + L + 64, ... in ascending order, one v_dot2 per element pair, then the
+// lanes meet in a butterfly.
 template <int MR, int NC>
 __device__ __forceinline__ void gemv_bf16_sums(const uint16_t* a, const uint16_t* const (&wr)[NC], uint32_t m, uint32_t lda,
                                                uint32_t c0, uint32_t c1, float (&acc)[MR][NC]) {
@@ -149,67 +147,50 @@ __device__ __forceinline__ void gemv_bf16_sums(const uint16_t* a, const uint16_t
         for (int j = 0; j < NC; j++) acc[r][j] = wave_sum(acc[r][j]);
 }
 
-// y[r][n] = bf16(x[r][:] . W[n][:]) (+ res) for r < m <= MR. grid ceil(N / 16), 256 threads: a wavefront takes 4
-// consecutive columns over all of K, so the weights stream in 1 KB runs a column and x is read once per 4 columns.
-// K % 8 == 0, N % 4 == 0, lda % 8 == 0, ldc % 4 == 0. (kernels/k-core/src/gemm.rs:172-208: fe_gemv_bf16, one warp a column)
-template <int MR>
+// y[r][n] = bf16(x[r][:] . W[n][:]) (+ res) for r < m <= MR. grid N / NC, 256 threads: a program takes NC consecutive
+// columns; K is walked in steps of 64 chunks of 16 bytes (a 1 KB run of every weight row a step), wavefront w takes
+// steps [w S / 4, (w + 1) S / 4) of the S steps, and the four sums are added in wavefront order. So a row's bits depend
+// on K only, neither on the other rows nor on NC: the host picks NC by the shape and the row count (more columns a program
+// read x less often, fewer columns give more programs), where the reference picks between two kernels by the shape.
+// K % 8 == 0, N % NC == 0, lda % 8 == 0. (kernels/k-core/src/gemm.rs:172-262: fe_gemv_bf16 and fe_gemv_bf16_kw)
+template <int MR, int NC>
 __device__ __forceinline__ void gemv_bf16_body(uint16_t* c, const uint16_t* a, const uint16_t* w, const uint16_t* res,
                                                uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc) {
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t col = (blockIdx.x * 4 + wave) * BF16_GEMV_COLS;
-    if (col >= n) return;
-    const uint16_t* wr[BF16_GEMV_COLS];
+    __shared__ float red[4][MR][NC];
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = blockIdx.x * NC;
+    const uint16_t* wr[NC];
 #pragma unroll
-    for (int j = 0; j < BF16_GEMV_COLS; j++) wr[j] = w + (size_t)(col + j < n ? col + j : n - 1) * k;
-    float acc[MR][BF16_GEMV_COLS];
-    gemv_bf16_sums<MR, BF16_GEMV_COLS>(a, wr, m, lda, 0, k / 8, acc);
+    for (int j = 0; j < NC; j++) wr[j] = w + (size_t)(col + j) * k;
+    const uint32_t chunks = k / 8, steps = (chunks + 63) / 64;
+    const uint32_t c0 = (wave * steps / 4) * 64, c1 = ((wave + 1) * steps / 4) * 64;
+    float acc[MR][NC];
+    gemv_bf16_sums<MR, NC>(a, wr, m, lda, c0, c1 < chunks ? c1 : chunks, acc);
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < MR; r++)
-            if ((uint32_t)r < m) bf16_store4(c, res, (size_t)r * ldc + col, acc[r]);
-    }
-}
-
-// The same for narrow linears (N <= 512): one program a column, its four wavefronts take a quarter of K each and wavefront
-// 0 adds the four in order, so the grid fills the GPU where fe_gemv_bf16 would run N / 16 programs. grid N, 256 threads.
-// K % 32 == 0. (kernels/k-core/src/gemm.rs:210-262: fe_gemv_bf16_kw)
-template <int MR>
-__device__ __forceinline__ void gemv_bf16_kw_body(uint16_t* c, const uint16_t* a, const uint16_t* w, const uint16_t* res,
-                                                  uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc) {
-    __shared__ float red[4][8];
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = blockIdx.x;
-    if (col >= n) return;
-    const uint16_t* wr[1] = {w + (size_t)col * k};
-    const uint32_t span = k / 32;
-    float acc[MR][1];
-    gemv_bf16_sums<MR, 1>(a, wr, m, lda, wave * span, (wave + 1) * span, acc);
-    if (lane == 0) {
 #pragma unroll
-        for (int r = 0; r < MR; r++) red[wave][r] = acc[r][0];
+            for (int j = 0; j < NC; j++) red[wave][r][j] = acc[r][j];
     }
     __syncthreads();
-    if (threadIdx.x < m) {
-        float y = red[0][threadIdx.x];
-        for (int q = 1; q < 4; q++) y += red[q][threadIdx.x];
-        const size_t at = (size_t)threadIdx.x * ldc + col;
+    const uint32_t r = threadIdx.x / NC, j = threadIdx.x % NC;
+    if (r < m) {
+        float y = red[0][r][j];
+        for (int q = 1; q < 4; q++) y += red[q][r][j];
+        const size_t at = (size_t)r * ldc + col + j;
         if (res) y = bf16_bits_to_f32(f32_to_bf16_bits(y)) + bf16_bits_to_f32(res[at]);
         c[at] = (uint16_t)f32_to_bf16_bits(y);
     }
 }
 
-#define BF16_GEMV_KERNELS(MR)                                                                                              \
-    extern "C" __global__ __launch_bounds__(256) void fe_gemv_bf16_r##MR(uint16_t* c, const uint16_t* a, const uint16_t* w, \
-                                                                         const uint16_t* res, uint32_t m, uint32_t n,     \
-                                                                         uint32_t k, uint32_t lda, uint32_t ldc) {        \
-        gemv_bf16_body<MR>(c, a, w, res, m, n, k, lda, ldc);                                                               \
-    }                                                                                                                      \
-    extern "C" __global__ __launch_bounds__(256) void fe_gemv_bf16_kw_r##MR(uint16_t* c, const uint16_t* a,                \
-                                                                            const uint16_t* w, const uint16_t* res,       \
-                                                                            uint32_t m, uint32_t n, uint32_t k,           \
-                                                                            uint32_t lda, uint32_t ldc) {                 \
-        gemv_bf16_kw_body<MR>(c, a, w, res, m, n, k, lda, ldc);                                                            \
+#define BF16_GEMV_KERNEL(MR, NC)                                                                                           \
+    extern "C" __global__ __launch_bounds__(256) void fe_gemv_bf16_r##MR##_c##NC(uint16_t* c, const uint16_t* a,           \
+                                                                                 const uint16_t* w, const uint16_t* res,  \
+                                                                                 uint32_t m, uint32_t n, uint32_t k,      \
+                                                                                 uint32_t lda, uint32_t ldc) {            \
+        gemv_bf16_body<MR, NC>(c, a, w, res, m, n, k, lda, ldc);                                                           \
     }
-BF16_GEMV_KERNELS(1)
-BF16_GEMV_KERNELS(2)
-BF16_GEMV_KERNELS(4)
-BF16_GEMV_KERNELS(8)
+#define BF16_GEMV_ROWS(MR) BF16_GEMV_KERNEL(MR, 1) BF16_GEMV_KERNEL(MR, 2) BF16_GEMV_KERNEL(MR, 4) BF16_GEMV_KERNEL(MR, 8)
+BF16_GEMV_ROWS(1)
+BF16_GEMV_ROWS(2)
+BF16_GEMV_ROWS(4)
+BF16_GEMV_ROWS(8)

@@ -66,7 +66,7 @@ def call(torch, fn, kern, x, w, m, n, ldy=None, res=None, rows_alloc=None, lda=N
 
 @pytest.mark.parametrize("n,k,m", [(256, 512, 1), (1024, 1024, 3), (2048, 5120, 8), (96, 1024, 5), (48, 256, 1),
                                    (520, 768, 2), (1032, 2048, 7), (512, 512, 4), (528, 512, 6)])
-def test_gemv(env, oracle, n, k, m):
+def test_gemv(env, oracle, monkeypatch, n, k, m):
     torch, bf16, kern = env
     xb, wb = operands(n, k, m, 7 + n)
     x, w = dev_u16(torch, xb), dev_u16(torch, wb)
@@ -78,6 +78,11 @@ def test_gemv(env, oracle, n, k, m):
     for r in {0, m - 1}:
         alone = call(torch, bf16.gemv, kern, x[r:r + 1].contiguous(), w, 1, n)
         assert np.array_equal(alone[0], got[r])
+    # nor on how many columns a program takes (FE_BF16_NC overrides the library's choice)
+    for nc in (1, 2, 4, 8):
+        monkeypatch.setenv("FE_BF16_NC", str(nc))
+        assert np.array_equal(call(torch, bf16.gemv, kern, x, w, m, n), got), nc
+    monkeypatch.delenv("FE_BF16_NC")
     # residual: bf16(bf16(sum) + res), exact given the sums
     rb = bits(np.random.default_rng(3).normal(size=(m + 2, n)))
     with_res = call(torch, bf16.gemv, kern, x, w, m, n, res=dev_u16(torch, rb))

@@ -157,7 +157,7 @@ def test_linear_without_prompt_weights(env):
     assert np.all(np.abs(a - b) <= np.abs(b) / 128.0 + 1e-3 * np.sqrt((b ** 2).mean()))  # the same sums in another order
     # a linear with no weights at all
     empty = route.Linear("none", HIDDEN, INTER)
-    with pytest.raises(FeError, match="no weights"):
+    with pytest.raises(FeError, match="no bf16 weights"):
         empty.forward(c, y, HIDDEN, x, INTER, 4)
     # shapes are checked when the linear is made
     with pytest.raises(FeError):
