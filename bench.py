@@ -522,6 +522,12 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     ms = timed(lambda: bf16.gemm(bk, yb, n, xf, k, ws_b[0], m))
     res["bf16_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    wi = bf16.interleave_gu(bk, ws_b[0], ws_b[1])
+    actb = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    ms = timed(lambda: bf16.gemm_swiglu(bk, actb, xf, k, wi, m))
+    res["bf16_swiglu_front_5120x34816"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(2 * flops / ms / 1e9, 1),
+                                           "frac_mfma_peak": round(2 * flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+    del wi, actb
     for rows in (1, 8):
         reps = 30
         pairs = [(ev.new(), ev.new()) for _ in range(reps)]

@@ -118,6 +118,9 @@ SYMBOLS = {
     "fe_bf16_kernels_destroy": (I, [P]),
     "fe_bf16_gemv": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
     "fe_bf16_gemm": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
+    "fe_bf16_interleave_gu": (I, [P, P, U64, U64, U64, U32, U32]),
+    "fe_bf16_gemm_swiglu": (I, [P, P, U64, U64, U32, U64, U32, U32, U32]),
+    "fe_route_mlp_forward_w": (I, [P, P, P, P, P, U64, U64, U64, U64, U64, U32, U32, U32]),
     "fe_bf16_linear_forward": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32, U32]),
     "fe_route_linear_create": (I, [PP, C.c_char_p, U32, U32, P, P]),
     "fe_route_linear_destroy": (I, [P]),

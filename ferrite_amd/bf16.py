@@ -48,3 +48,20 @@ def gemm(kern: Kernels, y, ldy: int, x, lda: int, w, m: int, res=None, stream=No
 def forward(kern: Kernels, y, ldy: int, x, lda: int, w, m: int, res=None, dec: int = 0, stream=None):
     """The bf16 branch of Linear::forward (model.rs:310-345)."""
     check(_lib.lib().fe_bf16_linear_forward(kern.h, _stream(stream), *_args(y, ldy, x, lda, w, res, m), dec))
+
+
+def interleave_gu(kern: Kernels, gate, up, stream=None):
+    """gate, up [inter][k] bf16 -> [2 inter][k], rows interleaved in blocks of 8 (fe_interleave_gu, gemm.rs:281-296)."""
+    import torch
+    inter, k = gate.shape
+    assert up.shape == gate.shape and gate.is_contiguous() and up.is_contiguous()
+    dst = torch.empty((2 * inter, k), dtype=gate.dtype, device=gate.device)
+    check(_lib.lib().fe_bf16_interleave_gu(kern.h, _stream(stream), dst.data_ptr(), gate.data_ptr(), up.data_ptr(), inter, k))
+    return dst
+
+
+def gemm_swiglu(kern: Kernels, act, x, lda: int, w, m: int, stream=None):
+    """act[m][inter] = SwiGLU(x . W^T) over interleaved gate|up weights W [2 inter][k] (fe_gemm_swiglu, gemm.rs:264-279)."""
+    n, k = w.shape
+    assert w.is_contiguous() and w.element_size() == 2
+    check(_lib.lib().fe_bf16_gemm_swiglu(kern.h, _stream(stream), act.data_ptr(), x.data_ptr(), lda, w.data_ptr(), m, n // 2, k))

@@ -17,7 +17,7 @@ constexpr uint32_t kSmallBatch = 16;                     // X3_ROWS: batches up 
 
 struct fe_bf16_kernels {
     fe_module_t module = nullptr;
-    fe_function_t gemm = nullptr, reduce = nullptr;
+    fe_function_t gemm = nullptr, reduce = nullptr, swiglu = nullptr, swiglu_reduce = nullptr, interleave = nullptr;
     fe_function_t gemv[4][4] = {};  // [rows 1, 2, 4, 8][columns of a program 1, 2, 4, 8]
     uint32_t cus = 0;
     FeBuf part;
@@ -50,6 +50,10 @@ int fe_bf16_kernels_load(fe_bf16_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->gemm, k->module, "fe_gemm_bf16");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->reduce, k->module, "fe_gemm_bf16_reduce");
+    if (!c) c = fe_hip_module_get_function(&k->swiglu, k->module, "fe_gemm_bf16_swiglu");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->swiglu, kGemmLds);
+    if (!c) c = fe_hip_module_get_function(&k->swiglu_reduce, k->module, "fe_gemm_bf16_swiglu_reduce");
+    if (!c) c = fe_hip_module_get_function(&k->interleave, k->module, "fe_interleave_gu");
     for (int i = 0; i < 4 && !c; i++)
         for (int j = 0; j < 4 && !c; j++) {
             char nm[32];
@@ -114,6 +118,40 @@ int fe_bf16_gemm(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint
     if (!gs.cut()) return 0;
     void *rargs[] = {&y, &part, &res, &m, &n, &ldy, &group, &full, &splits};
     return fe_hip_launch(kern->reduce, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
+}
+
+int fe_bf16_interleave_gu(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t dst, fe_devptr_t gate, fe_devptr_t up,
+                          uint32_t inter, uint32_t k) {
+    const char *fn = "fe_bf16_interleave_gu";
+    if (!kern || !dst || !gate || !up) return fe_set_error(FE_ERR_ARG, fn, "null argument");
+    if (!inter || !k || inter % 8 || k % 8 || dst % 16 || gate % 16 || up % 16)
+        return fe_set_error(FE_ERR_SHAPE, fn, "inter % 8 == 0, k % 8 == 0, 16-byte aligned rows");
+    void *args[] = {&dst, &gate, &up, &k};
+    return fe_hip_launch(kern->interleave, 2 * inter, 1, 1, 256, 1, 1, 0, s, args);
+}
+
+int fe_bf16_gemm_swiglu(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t act, fe_devptr_t x, uint32_t lda,
+                        fe_devptr_t w, uint32_t m, uint32_t inter, uint32_t k) {
+    const char *fn = "fe_bf16_gemm_swiglu";
+    if (!kern) return fe_set_error(FE_ERR_ARG, fn, "null kernels");
+    if (m == 0) return 0;
+    uint32_t n = 2 * inter;
+    FE_TRY(check(fn, act, n, x, lda, w, 0, n, k));  // act rows have stride inter = n / 2, a multiple of 8
+    if (n % 16) return fe_set_error(FE_ERR_SHAPE, fn, "inter % 8 == 0");
+    if ((uint64_t)m * lda * 2 >= (1ull << 32) || (uint64_t)n * k * 2 >= (1ull << 32))
+        return fe_set_error(FE_ERR_UNSUPPORTED, fn, "operand of 4 GB or more");
+    const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
+    uint32_t group = n >= m ? 0 : tiles_m < 8 ? tiles_m : 8;
+    if (const char *e = getenv("FE_BF16_GROUP")) group = (uint32_t)atoi(e);
+    if (group > tiles_m) group = tiles_m;
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes));
+    uint32_t full = gs.full, splits = gs.splits;
+    fe_devptr_t part = kern->part.p;
+    void *args[] = {&act, &x, &w, &m, &n, &k, &lda, &group, &full, &splits, &part};
+    FE_TRY(fe_hip_launch(kern->swiglu, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (!gs.cut()) return 0;
+    void *rargs[] = {&act, &part, &m, &n, &group, &full, &splits};
+    return fe_hip_launch(kern->swiglu_reduce, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 int fe_bf16_linear_forward(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x,

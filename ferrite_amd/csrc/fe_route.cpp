@@ -340,6 +340,12 @@ int fe_route_proj_forward(const fe_route_proj *p, const fe_route_ctx *c, fe_devp
 int fe_route_mlp_forward(const fe_route_ctx *c, const fe_route_proj *gate_up, const fe_route_linear *down,
                          const fe_fp4_linear *swiglu, const fe_fp4_workspace *act_ws, fe_devptr_t x, fe_devptr_t xn,
                          fe_devptr_t big, fe_devptr_t act, uint32_t rows, uint32_t hidden, uint32_t inter) {
+    return fe_route_mlp_forward_w(c, gate_up, down, swiglu, act_ws, 0, x, xn, big, act, rows, hidden, inter);
+}
+
+int fe_route_mlp_forward_w(const fe_route_ctx *c, const fe_route_proj *gate_up, const fe_route_linear *down,
+                           const fe_fp4_linear *swiglu, const fe_fp4_workspace *act_ws, fe_devptr_t swiglu_w, fe_devptr_t x,
+                           fe_devptr_t xn, fe_devptr_t big, fe_devptr_t act, uint32_t rows, uint32_t hidden, uint32_t inter) {
     const char *fn = "fe_route_mlp_forward";
     if (!c || !gate_up || !down || !x || !xn || !big || !act) return fe_set_error(FE_ERR_ARG, fn, "null argument");
     if (down->n != hidden || down->k != inter) return fe_set_error(FE_ERR_SHAPE, fn, "down is not hidden x inter");
@@ -356,6 +362,14 @@ int fe_route_mlp_forward(const fe_route_ctx *c, const fe_route_proj *gate_up, co
         // residual in place (model.rs:3166-3178)
         FE_TRY(fe_fp4_linear_forward_swiglu(swiglu, c->fk, c->s, c->fws, act_ws, xn_p, hidden, pr_rows, down_g));
         FE_TRY(fe_fp4_linear_gemm(down->p, c->fk, c->s, act_ws, x_p, hidden, pr_rows, x_p));
+        fused = true;
+    } else if (pr_rows > FE_X3_ROWS && swiglu_w && c->bk) {
+        // interleaved bf16 gate|up weights: one GEMM with SwiGLU in its epilogue, then down over the prompt rows with the
+        // residual (model.rs:3179-3188)
+        const fe_devptr_t xn_p = xn + (size_t)d * hidden * 2, x_p = x + (size_t)d * hidden * 2;
+        const fe_devptr_t act_p = act + (size_t)d * inter * 2;
+        FE_TRY(fe_bf16_gemm_swiglu(c->bk, c->s, act_p, xn_p, hidden, swiglu_w, pr_rows, inter, hidden));
+        FE_TRY(linear_forward(down, c, 0, x_p, hidden, act_p, inter, pr_rows, x_p));
         fused = true;
     }
     const uint32_t n_rest = fused ? d : rows;

@@ -97,6 +97,80 @@ extern "C" __global__ __launch_bounds__(256) void fe_gemm_bf16_reduce(uint16_t* 
     });
 }
 
+// SwiGLU over a gate|up linear whose weight rows are interleaved in blocks of 8 ([gate 0..8, up 0..8, gate 8..16, ...],
+// fe_interleave_gu): of the 4 lanes that hold one 16-column block of a row, lanes 0, 1 have the 8 gate sums and lanes 2, 3
+// the matching up sums. Every lane takes part (a quad exchange); lanes 0, 1 store
+// act[row][8 blk + 4 (lane & 1) ..] = bf16(bf16(silu(bf16(gate))) * bf16(up)), act row stride inter = n / 2.
+// (kernels/k-core/src/gemm.rs:264-279)
+__device__ __forceinline__ void bf16_swiglu_store4(uint16_t* act, const float (&v)[4], uint32_t l32, bool live, uint32_t grow,
+                                                   uint32_t col, uint32_t n) {
+    float u[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) u[e] = dpp_quad_xor<2>(v[e]);
+    if (!live || (l32 & 2) || col >= n) return;
+    const u32x2 o = {silu_mul_bf16x2(pack_bf16x2(v[0], v[1]), pack_bf16x2(u[0], u[1])),
+                     silu_mul_bf16x2(pack_bf16x2(v[2], v[3]), pack_bf16x2(u[2], u[3]))};
+    *(u32x2*)(act + (size_t)grow * (n >> 1) + (col >> 4) * 8 + 4 * (l32 & 1)) = o;
+}
+
+// act[M][N / 2] = SwiGLU(A . W^T) for interleaved gate|up weights W [N][K], N % 16 == 0: fe_gemm_bf16 with the epilogue
+// above (and fe_gemm_bf16_swiglu_reduce for the tiles cut along K). (kernels/k-core/src/gemm.rs:264-279: fe_gemm_swiglu)
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_bf16_swiglu(uint16_t* act, const uint16_t* a, const uint16_t* w,
+                                                                         uint32_t m, uint32_t n, uint32_t k, uint32_t lda,
+                                                                         uint32_t group_m, uint32_t full_tiles,
+                                                                         uint32_t splits, float* part) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
+    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (n + GM_BN - 1) / GM_BN, group_m, k / GM_BK, full_tiles, splits);
+    const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
+    Bf16Producer prod;
+    const uint32_t chunk = tid & 7, row = tid >> 3;
+    prod.w = (const unsigned char*)w;
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint32_t r = n0 + 128 * b + row + 32 * j;
+            r = r < n ? r : n - 1;
+            prod.off[b][j] = (r * k + chunk * 8) * 2;
+        }
+    prod.st = gm_swz(row, chunk);
+    f32x16 acc[4][4];
+    gemm_mainloop<Bf16Producer, true>((const _Float16*)a, lda, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
+    if (wk.partial) {
+        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
+        return;
+    }
+    const uint32_t col = n0 + wn * 128 + 4 * (tid & 31);
+    gemm_epilogue(
+        acc, lds, [](float (&)[4][4], uint32_t) {},
+        [&](uint32_t r, uint32_t l32, float (&v)[4]) {
+            const uint32_t grow = m0 + wm * 128 + r;
+            bf16_swiglu_store4(act, v, l32, grow < m, grow, col, n);
+        });
+}
+
+extern "C" __global__ __launch_bounds__(256) void fe_gemm_bf16_swiglu_reduce(uint16_t* act, const float* part, uint32_t m,
+                                                                             uint32_t n, uint32_t group_m,
+                                                                             uint32_t full_tiles, uint32_t splits) {
+    gemm_reduce_rows(part, splits, [&](uint32_t t, uint32_t row, uint32_t cb, uint32_t l32, float (&v)[4]) {
+        uint32_t tm, tn;
+        gemm_raster(full_tiles + t, (m + GM_BM - 1) / GM_BM, (n + GM_BN - 1) / GM_BN, group_m, tm, tn);
+        const uint32_t grow = tm * GM_BM + row, col = tn * GM_BN + cb * 128 + 4 * l32;
+        bf16_swiglu_store4(act, v, l32, grow < m, grow, col, n);
+    });
+}
+
+// dst row 16 b + i = gate row 8 b + i for i < 8, up row 8 b + i - 8 otherwise: the weight layout of fe_gemm_bf16_swiglu.
+// grid 2 inter, 256 threads; k % 8 == 0. (kernels/k-core/src/gemm.rs:281-296: fe_interleave_gu)
+extern "C" __global__ __launch_bounds__(256) void fe_interleave_gu(uint16_t* dst, const uint16_t* gate, const uint16_t* up,
+                                                                   uint32_t k) {
+    const uint32_t r = blockIdx.x, b = r / 16, i = r % 16;
+    const uint16_t* src = i < 8 ? gate + (size_t)(b * 8 + i) * k : up + (size_t)(b * 8 + i - 8) * k;
+    uint16_t* d = dst + (size_t)r * k;
+    for (uint32_t j = threadIdx.x; j < k / 8; j += 256) *((u32x4*)d + j) = *((const u32x4*)src + j);
+}
+
 // ---- GEMV (1..8 rows) ------------------------------------------------------------------------------------------------
 
 __device__ __forceinline__ float dot8_bf16(u32x4 w, u32x4 x, float acc) {

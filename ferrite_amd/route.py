@@ -116,8 +116,10 @@ def copy2d(dst_ptr: int, ldd: int, src_ptr: int, lds: int, cols: int, rows: int,
 
 
 def mlp_forward(c: LinCtx, gate_up: Proj, down: Linear, x, xn, big, act, rows: int, hidden: int, inter: int, swiglu=None,
-                act_ws=None):
-    """x += down(SwiGLU(gate(xn), up(xn))) with the reference's routing of decode and prompt rows (model.rs:3160-3203)."""
-    check(_lib.lib().fe_route_mlp_forward(c.h, gate_up.h, down.h, swiglu.h if swiglu is not None else None,
-                                          act_ws.h if act_ws is not None else None, x.data_ptr(), xn.data_ptr(),
-                                          big.data_ptr(), act.data_ptr(), rows, hidden, inter))
+                act_ws=None, swiglu_w=None):
+    """x += down(SwiGLU(gate(xn), up(xn))) with the reference's routing of decode and prompt rows (model.rs:3160-3203).
+    swiglu / act_ws: the fused NVFP4 front; swiglu_w: interleaved bf16 gate|up weights [2 inter][hidden] (its second form)."""
+    check(_lib.lib().fe_route_mlp_forward_w(c.h, gate_up.h, down.h, swiglu.h if swiglu is not None else None,
+                                            act_ws.h if act_ws is not None else None,
+                                            swiglu_w.data_ptr() if swiglu_w is not None else 0, x.data_ptr(), xn.data_ptr(),
+                                            big.data_ptr(), act.data_ptr(), rows, hidden, inter))

@@ -89,6 +89,13 @@ int fe_route_mlp_forward(const fe_route_ctx *c, const fe_route_proj *gate_up, co
                          const fe_fp4_linear *swiglu, const fe_fp4_workspace *act_ws, fe_devptr_t x, fe_devptr_t xn,
                          fe_devptr_t big, fe_devptr_t act, uint32_t rows, uint32_t hidden, uint32_t inter);
 
+/* The same with the block's second fused form (model.rs:3179-3188): swiglu_w = bf16 gate|up weights [2 inter][hidden]
+ * interleaved in blocks of 8 (fe_bf16_interleave_gu), 0 = none. Taken for more than FE_X3_ROWS prompt rows when the NVFP4
+ * front does not apply and the context has the bf16 kernels: fe_bf16_gemm_swiglu into act, then down with the residual. */
+int fe_route_mlp_forward_w(const fe_route_ctx *c, const fe_route_proj *gate_up, const fe_route_linear *down,
+                           const fe_fp4_linear *swiglu, const fe_fp4_workspace *act_ws, fe_devptr_t swiglu_w, fe_devptr_t x,
+                           fe_devptr_t xn, fe_devptr_t big, fe_devptr_t act, uint32_t rows, uint32_t hidden, uint32_t inter);
+
 #ifdef __cplusplus
 }
 #endif

@@ -162,6 +162,103 @@ def test_route_linear_with_bf16_weights_only(env):
     assert np.array_equal(host_u16(y), call(torch, bf16.forward, kern, x, w, m, n, dec=5))
 
 
+def test_gemm_swiglu_over_interleaved_weights(env, oracle):
+    """fe_interleave_gu + fe_gemm_swiglu (gemm.rs:264-296): the bits of the plain GEMM over the same interleaved weights
+    followed by fe_silu_mul; against the oracle's sums and the exact formula within the bf16 steps of the two roundings."""
+    torch, bf16, kern = env
+    from ferrite_amd import route
+    for inter, k, m in ((640, 512, 300), (136, 256, 40), (2048, 1024, 700)):
+        rng = np.random.default_rng(inter)
+        xb = bits(rng.normal(size=(m, k)))
+        gb, ub = bits(rng.normal(size=(inter, k)) / np.sqrt(k) * 2), bits(rng.normal(size=(inter, k)) / np.sqrt(k) * 2)
+        x, g, u = dev_u16(torch, xb), dev_u16(torch, gb), dev_u16(torch, ub)
+        w = bf16.interleave_gu(kern, g, u)
+        torch.cuda.synchronize()
+        want_w = np.empty((2 * inter, k), np.uint16)
+        r = np.arange(2 * inter)
+        b, i = r // 16, r % 16
+        want_w[i < 8] = gb[(b * 8 + i)[i < 8]]
+        want_w[i >= 8] = ub[(b * 8 + i - 8)[i >= 8]]
+        assert np.array_equal(host_u16(w), want_w)
+        act = dev_u16(torch, np.full((m + 1, inter), CANARY, np.uint16))
+        bf16.gemm_swiglu(kern, act, x, k, w, m)
+        torch.cuda.synchronize()
+        got = host_u16(act)
+        assert (got[m:] == CANARY).all()
+        # the plain GEMM over the interleaved weights, then fe_silu_mul on its gate and up columns
+        y = call(torch, bf16.gemm, kern, x, w, m, 2 * inter)
+        yb = y.reshape(m, inter // 8, 2, 8)
+        gate, up = np.ascontiguousarray(yb[:, :, 0].reshape(m, inter)), np.ascontiguousarray(yb[:, :, 1].reshape(m, inter))
+        gd, ud = dev_u16(torch, gate), dev_u16(torch, up)
+        out = dev_u16(torch, np.zeros((m, inter), np.uint16))
+        route.silu_mul(out, gd.data_ptr(), ud.data_ptr(), inter, inter, m)
+        torch.cuda.synchronize()
+        assert np.array_equal(got[:m], host_u16(out))
+        # the formula on the oracle's sums
+        _, ag = oracle.bf16_linear_ref(xb, gb)
+        _, au = oracle.bf16_linear_ref(xb, ub)
+        gq, uq = f32(bits(ag)).astype(np.float64), f32(bits(au)).astype(np.float64)
+        ref = f32(bits(gq / (1.0 + np.exp(-gq)))).astype(np.float64) * uq
+        gotf = f32(got[:m]).astype(np.float64)
+        rms = np.sqrt((ref ** 2).mean())
+        assert (np.abs(gotf - ref) <= np.abs(ref) * 2.0 ** -6 + 2e-2 * rms).all()
+        assert np.median(np.abs(gotf - ref) / np.maximum(np.abs(ref), 1e-3 * rms)) < 2.0 ** -8
+
+
+def test_mlp_block_with_bf16_weights(env):
+    """The MLP block's second fused form (model.rs:3179-3188): more than 16 prompt rows take fe_gemm_swiglu over the
+    interleaved gate|up weights and down's GEMM with the residual; the decode rows take the per-linear path. Each group of
+    rows has the bits of the same steps called by hand."""
+    torch, bf16, kern = env
+    from ferrite_amd import route
+    hidden, inter, rows, dec = 512, 1280, 60, 4
+    rng = np.random.default_rng(17)
+    xn_b, x_b = bits(rng.normal(size=(rows, hidden))), bits(rng.normal(size=(rows, hidden)))
+    gb, ub = bits(rng.normal(size=(inter, hidden)) / np.sqrt(hidden) * 2), bits(rng.normal(size=(inter, hidden)) / np.sqrt(hidden) * 2)
+    db = bits(rng.normal(size=(hidden, inter)) / np.sqrt(inter))
+    xn, g, u, dn = dev_u16(torch, xn_b), dev_u16(torch, gb), dev_u16(torch, ub), dev_u16(torch, db)
+    wi = bf16.interleave_gu(kern, g, u)
+    ctx = route.LinCtx()
+    ctx.set_bf16(kern)
+    bf = torch.bfloat16
+    gate_up = route.Proj([(route.Linear("gate", inter, hidden, w=g.view(bf)), [inter]), (route.Linear("up", inter, hidden, w=u.view(bf)), [inter])])
+    down = route.Linear("down", hidden, inter, w=dn.view(bf))
+    big = dev_u16(torch, np.zeros((rows, 2 * inter), np.uint16))
+    act = dev_u16(torch, np.zeros((rows, inter), np.uint16))
+
+    def run(nrows, d, fused):
+        ctx.dec = d
+        x = dev_u16(torch, x_b)
+        route.mlp_forward(ctx, gate_up, down, x, xn, big, act, nrows, hidden, inter, swiglu_w=wi if fused else None)
+        torch.cuda.synchronize()
+        return host_u16(x)
+
+    def by_hand_rows(r0, r1, gemv):
+        """gate, up, fe_silu_mul, down + residual over rows [r0, r1), every linear through the GEMV or the GEMM."""
+        m = r1 - r0
+        fn = (lambda *a, **k: bf16.forward(*a, **k)) if gemv else bf16.gemm
+        xs = xn[r0:r1].contiguous()
+        yg, yu = call(torch, fn, kern, xs, g, m, inter), call(torch, fn, kern, xs, u, m, inter)
+        a = dev_u16(torch, np.zeros((m, inter), np.uint16))
+        gd, ud = dev_u16(torch, yg), dev_u16(torch, yu)
+        route.silu_mul(a, gd.data_ptr(), ud.data_ptr(), inter, inter, m)
+        return call(torch, fn, kern, a, dn, m, hidden, res=dev_u16(torch, x_b[r0:r1]))
+
+    got = run(rows, dec, True)
+    assert np.array_equal(got[:dec], by_hand_rows(0, dec, True))
+    a = dev_u16(torch, np.zeros((rows - dec, inter), np.uint16))
+    bf16.gemm_swiglu(kern, a, xn[dec:].contiguous(), hidden, wi, rows - dec)
+    want = call(torch, bf16.gemm, kern, a, dn, rows - dec, hidden, res=dev_u16(torch, x_b[dec:]))
+    assert np.array_equal(got[dec:], want)
+    # without the interleaved weights: gate and up one by one, fe_silu_mul, down (the same sums: the same bits)
+    plain = run(rows, dec, False)
+    assert np.array_equal(plain[:dec], got[:dec])
+    assert np.array_equal(plain[dec:], by_hand_rows(dec, rows, False))
+    # a batch of up to 16 rows: all decode rows, the fused form is not used
+    small = run(12, 0, True)
+    assert np.array_equal(small[:12], by_hand_rows(0, 12, True)) and np.array_equal(small[12:], x_b[12:])
+
+
 def test_argument_errors(env):
     torch, bf16, kern = env
     from ferrite_amd import _lib
