@@ -23,10 +23,11 @@ struct fe_bf16_kernels {
     FeBuf part;
 };
 
-// log2 of the columns a GEMV program takes: 4 measured best for 1..8 rows on 5120 x 17408, 17408 x 5120 and
-// 5120 x 5120 (at 8 rows 48 us against 86 us with one column, 51 us with eight); narrow linears take fewer so that the
-// grid still has a few programs a CU
-static int gemv_cols(uint32_t n) { return n >= 4096 ? 2 : n >= 1024 ? 1 : 0; }
+// log2 of the columns a GEMV program takes. Measured on 5120 x 17408, 17408 x 5120 and 5120 x 5120: 4 columns are best
+// for 1 and 2 rows (5120 x 17408: 29 us at 1 row), 8 for 3..8 rows of a wide linear (31.7 against 33.8 us at 4 rows,
+// 42.6 against 43.8 at 8; one column: 83 us at 8 rows); narrow linears take fewer so that the grid still has a few
+// programs a CU.
+static int gemv_cols(uint32_t n, int form) { return n >= 8192 && form >= 2 ? 3 : n >= 4096 ? 2 : n >= 1024 ? 1 : 0; }
 
 static int check(const char *fn, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda, fe_devptr_t w, fe_devptr_t res,
                  uint32_t n, uint32_t k) {
@@ -90,7 +91,7 @@ int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint
     const int form = m <= 1 ? 0 : m <= 2 ? 1 : m <= 4 ? 2 : 3;
     // columns of a program: the results do not depend on it. More columns read x less often (x is read once per program
     // and step, the weights once in all), fewer give more programs
-    int cols = gemv_cols(n);
+    int cols = gemv_cols(n, form);
     if (const char *e = getenv("FE_BF16_NC")) cols = atoi(e) >= 8 ? 3 : atoi(e) >= 4 ? 2 : atoi(e) >= 2 ? 1 : 0;
     void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy};
     return fe_hip_launch(kern->gemv[form][cols], n >> cols, 1, 1, 256, 1, 1, 0, s, args);

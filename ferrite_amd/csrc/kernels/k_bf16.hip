@@ -183,15 +183,18 @@ __device__ __forceinline__ float dot8_bf16(u32x4 w, u32x4 x, float acc) {
     return acc;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+// Sum over each row of 16 lanes, left in all 16 (four DPP adds: no LDS traffic, unlike a butterfly of ds_bpermute).
+__device__ __forceinline__ float row16_sum(float v) {
+    v += dpp_mov<DPP_QUAD_XOR1>(v);
+    v += dpp_mov<DPP_QUAD_XOR2>(v);
+    v += dpp_mov<DPP_HALF_MIRROR>(v);
+    v += dpp_mov<DPP_ROW_MIRROR>(v);
     return v;
 }
 
 // One wavefront: the sums of x rows 0..MR-1 (rows >= m repeat row m - 1) with NC weight rows over the 16-byte chunks
-// [c0, c1) of K, lane L taking chunks c0 + L, c0 + L + 64, ... in ascending order, one v_dot2 per element pair, then the
-// lanes meet in a butterfly.
+// [c0, c1) of K, lane L taking chunks c0 + L, c0 + L + 64, ... in ascending order, one v_dot2 per element pair; then
+// every 16 lanes add up (the sum of lanes 16 q .. 16 q + 15 is left in all of them).
 template <int MR, int NC>
 __device__ __forceinline__ void gemv_bf16_sums(const uint16_t* a, const uint16_t* const (&wr)[NC], uint32_t m, uint32_t lda,
                                                uint32_t c0, uint32_t c1, float (&acc)[MR][NC]) {
@@ -218,19 +221,19 @@ __device__ __forceinline__ void gemv_bf16_sums(const uint16_t* a, const uint16_t
 #pragma unroll
     for (int r = 0; r < MR; r++)
 #pragma unroll
-        for (int j = 0; j < NC; j++) acc[r][j] = wave_sum(acc[r][j]);
+        for (int j = 0; j < NC; j++) acc[r][j] = row16_sum(acc[r][j]);
 }
 
 // y[r][n] = bf16(x[r][:] . W[n][:]) (+ res) for r < m <= MR. grid N / NC, 256 threads: a program takes NC consecutive
 // columns; K is walked in steps of 64 chunks of 16 bytes (a 1 KB run of every weight row a step), wavefront w takes
-// steps [w S / 4, (w + 1) S / 4) of the S steps, and the four sums are added in wavefront order. So a row's bits depend
+// steps [w S / 4, (w + 1) S / 4) of the S steps, and the sixteen sums (4 wavefronts x 4 rows of 16 lanes) are added in order. So a row's bits depend
 // on K only, neither on the other rows nor on NC: the host picks NC by the shape and the row count (more columns a program
 // read x less often, fewer columns give more programs), where the reference picks between two kernels by the shape.
 // K % 8 == 0, N % NC == 0, lda % 8 == 0. (kernels/k-core/src/gemm.rs:172-262: fe_gemv_bf16 and fe_gemv_bf16_kw)
 template <int MR, int NC>
 __device__ __forceinline__ void gemv_bf16_body(uint16_t* c, const uint16_t* a, const uint16_t* w, const uint16_t* res,
                                                uint32_t m, uint32_t n, uint32_t k, uint32_t lda, uint32_t ldc) {
-    __shared__ float red[4][MR][NC];
+    __shared__ float red[16][MR][NC];
     const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = blockIdx.x * NC;
     const uint16_t* wr[NC];
 #pragma unroll
@@ -239,17 +242,17 @@ __device__ __forceinline__ void gemv_bf16_body(uint16_t* c, const uint16_t* a, c
     const uint32_t c0 = (wave * steps / 4) * 64, c1 = ((wave + 1) * steps / 4) * 64;
     float acc[MR][NC];
     gemv_bf16_sums<MR, NC>(a, wr, m, lda, c0, c1 < chunks ? c1 : chunks, acc);
-    if (lane == 0) {
+    if ((lane & 15) == 0) {
 #pragma unroll
         for (int r = 0; r < MR; r++)
 #pragma unroll
-            for (int j = 0; j < NC; j++) red[wave][r][j] = acc[r][j];
+            for (int j = 0; j < NC; j++) red[threadIdx.x >> 4][r][j] = acc[r][j];
     }
     __syncthreads();
     const uint32_t r = threadIdx.x / NC, j = threadIdx.x % NC;
     if (r < m) {
         float y = red[0][r][j];
-        for (int q = 1; q < 4; q++) y += red[q][r][j];
+        for (int q = 1; q < 16; q++) y += red[q][r][j];
         const size_t at = (size_t)r * ldc + col + j;
         if (res) y = bf16_bits_to_f32(f32_to_bf16_bits(y)) + bf16_bits_to_f32(res[at]);
         c[at] = (uint16_t)f32_to_bf16_bits(y);

@@ -24,8 +24,8 @@ typedef struct fe_bf16_kernels fe_bf16_kernels;
 int fe_bf16_kernels_load(fe_bf16_kernels **out);
 int fe_bf16_kernels_destroy(fe_bf16_kernels *k);
 
-/* fe_gemv_bf16 / fe_gemv_bf16_kw (gemm.rs:172-262): m <= 8 rows. One kernel family here: a program takes 1, 2 or 4
- * columns by the width of the linear (model.rs:316-322 picks between the two kernels by the shape), and a row's bits
+/* fe_gemv_bf16 / fe_gemv_bf16_kw (gemm.rs:172-262): m <= 8 rows. One kernel family here: a program takes 1, 2, 4
+ * or 8 columns by the width of the linear and the row count (model.rs:316-322 picks between the two kernels by the shape), and a row's bits
  * depend neither on that nor on m. res (stride ldy) may be 0; with it y = bf16(bf16(x . W) + res), res may be y. */
 int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda,
                  fe_devptr_t w, fe_devptr_t res, uint32_t m, uint32_t n, uint32_t k);
