@@ -98,6 +98,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--bracket-events", action="store_true",
+                    help="time the roofline kernel with events recorded before and after its launch instead of events attached to its dispatch")
     ap.add_argument("--no-sweep", action="store_true", help="leave out the M = 1, 4, 8, 16 sweep (for a kernel trace of the step alone)")
     ap.add_argument("--traffic-pass", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a streaming read and an elementwise update of "
@@ -168,9 +170,13 @@ def main():
                      (f_rotated, (d.h, stream, ws.xh_ptr, yd.data_ptr(), bf16, 1, ws.h))]
         launches.append((f"down_b{bits}", d.weight_bytes(), False, len(calls), calls, None))
 
-    # Event pairs on the launch stream. In the timed region only the dominant kernel's launches carry them (each record is
-    # a packet of its own on the queue and costs a few microseconds of the step); one more pass after the timed region
-    # brackets every launch for the per-launch table. The pair brackets the last call of a launch (the GEMV).
+    # Event pairs on the launch stream. In the timed region only the dominant kernel's launches carry them; one more pass
+    # after the timed region times every launch for the per-launch table. A pair is attached to the dispatch of the
+    # launch's last kernel (the GEMV), so it reads that kernel's own begin and end as a kernel trace does
+    # (fe_hip_time_next_launch); with --bracket-events it is recorded before and after the launch instead, each record
+    # a packet of its own on the queue, which adds the dispatch gap and the packets to the reading.
+    attached = not args.bracket_events
+    f_time_next = lib.fe_hip_time_next_launch
     events = [[(ev.new(), ev.new()) if la[2] else None for la in launches] for _ in range(args.steps)]
     table_events = [(ev.new(), ev.new()) for _ in launches]
 
@@ -181,11 +187,14 @@ def main():
             for fn, a in calls[:-1]:
                 rc |= fn(*a)
             pair = pairs[li] if pairs is not None else None
-            if pair is not None:
+            attach = pair is not None and attached and la[3] == len(calls)  # the last call is one kernel launch
+            if attach:
+                rc |= f_time_next(pair[0], pair[1])
+            elif pair is not None:
                 rc |= f_record(pair[0], stream)
             fn, a = calls[-1]
             rc |= fn(*a)
-            if pair is not None:
+            if pair is not None and not attach:
                 rc |= f_record(pair[1], stream)
         _lib.check(rc)
 
@@ -246,7 +255,8 @@ def main():
         "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (gate + up, 5120x17408 each, M=1)", "achieved": round(achieved, 2),
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ROOFLINE_TRAFFIC_BYTES,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms),
-                     "back_to_back_us": round(dom_b2b_us, 3)},
+                     "back_to_back_us": round(dom_b2b_us, 3),
+                     "events": "recorded around the launch" if args.bracket_events else "attached to the kernel's dispatch"},
         "cpu_baseline": cpu,
         "per_launch": per,
     }

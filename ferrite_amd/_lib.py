@@ -55,6 +55,7 @@ SYMBOLS = {
     "fe_hip_stream_create": (I, [PP]),
     "fe_hip_stream_destroy": (I, [P]),
     "fe_hip_stream_sync": (I, [P]),
+    "fe_hip_time_next_launch": (I, [P, P]),
     "fe_hip_event_create": (I, [PP]),
     "fe_hip_event_destroy": (I, [P]),
     "fe_hip_event_record": (I, [P, P]),

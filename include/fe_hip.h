@@ -62,6 +62,11 @@ int fe_hip_launch(fe_function_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32
 int fe_hip_stream_create(fe_stream_t *out);
 int fe_hip_stream_destroy(fe_stream_t s);
 int fe_hip_stream_sync(fe_stream_t s);
+/* Times one kernel by itself: the calling thread's next fe_hip_launch (whichever library call makes it) is launched with
+ * `start` and `stop` attached to its dispatch, so fe_hip_event_elapsed_ms(start, stop) after a sync is that kernel's own
+ * duration, without the marker packets fe_hip_event_record puts into the stream. Stream::time
+ * (crates/fe-cuda/src/lib.rs:766-774) brackets a closure with two recorded events instead; CUDA has no per-launch form. */
+int fe_hip_time_next_launch(fe_event_t start, fe_event_t stop);
 int fe_hip_event_create(fe_event_t *out);
 int fe_hip_event_destroy(fe_event_t e);
 int fe_hip_event_record(fe_event_t e, fe_stream_t s);
