@@ -259,6 +259,33 @@ def test_mlp_block_with_bf16_weights(env):
     assert np.array_equal(small[:12], by_hand_rows(0, 12, True)) and np.array_equal(small[12:], x_b[12:])
 
 
+def test_events_attached_to_one_launch(env):
+    """fe_hip_time_next_launch: the next launch carries the two events; the result is the launch's own, the reading a
+    kernel duration, and the launch after it is an ordinary one again."""
+    import ctypes as C
+    torch, bf16, kern = env
+    from ferrite_amd import _lib
+    lib = _lib.lib()
+    n, k = 4096, 2048
+    xb, wb = operands(n, k, 1, 9)
+    x, w = dev_u16(torch, xb), dev_u16(torch, wb)
+    plain = call(torch, bf16.gemv, kern, x, w, 1, n)
+    a, b = C.c_void_p(), C.c_void_p()
+    _lib.check(lib.fe_hip_event_create(C.byref(a)))
+    _lib.check(lib.fe_hip_event_create(C.byref(b)))
+    for _ in range(2):
+        _lib.check(lib.fe_hip_time_next_launch(a, b))
+        timed = call(torch, bf16.gemv, kern, x, w, 1, n)
+        assert np.array_equal(timed, plain)
+        _lib.check(lib.fe_hip_event_sync(b))
+        ms = C.c_float()
+        _lib.check(lib.fe_hip_event_elapsed_ms(C.byref(ms), a, b))
+        assert 1e-3 < ms.value < 5.0, ms.value  # 16 MB of weights: a few microseconds, not a host-side interval
+        assert np.array_equal(call(torch, bf16.gemv, kern, x, w, 1, n), plain)
+    _lib.check(lib.fe_hip_event_destroy(a))
+    _lib.check(lib.fe_hip_event_destroy(b))
+
+
 def test_argument_errors(env):
     torch, bf16, kern = env
     from ferrite_amd import _lib
