@@ -64,7 +64,8 @@ int fe_hip_stream_destroy(fe_stream_t s);
 int fe_hip_stream_sync(fe_stream_t s);
 /* Times one kernel by itself: the calling thread's next fe_hip_launch (whichever library call makes it) is launched with
  * `start` and `stop` attached to its dispatch, so fe_hip_event_elapsed_ms(start, stop) after a sync is that kernel's own
- * duration, without the marker packets fe_hip_event_record puts into the stream. Stream::time
+ * duration, without the marker packets fe_hip_event_record puts into the stream. Not for a launch under graph capture
+ * (a captured launch carries no events). Stream::time
  * (crates/fe-cuda/src/lib.rs:766-774) brackets a closure with two recorded events instead; CUDA has no per-launch form. */
 int fe_hip_time_next_launch(fe_event_t start, fe_event_t stop);
 int fe_hip_event_create(fe_event_t *out);
