@@ -40,11 +40,15 @@ __device__ __forceinline__ uint32_t f32_to_e2m1(float x) {
 
 // The same conversion for two values at once in hardware: byte `BYTE` of `old` becomes e2m1(a) | e2m1(b) << 4
 // (v_cvt_scalef32_pk_fp4_f32 with scale 1). Checked against f32_to_e2m1 on the GPU for every bf16 value, every f32 with
-// an exponent of 2^-5 .. 2^4 (all code boundaries and ties), the smallest and the largest magnitudes, both signs: no
-// difference. NaN inputs are not covered by that check (the quantizer's inputs are finite).
+// an exponent of 2^-5 .. 2^4 (all code boundaries and ties), the smallest and the largest magnitudes, infinities, both
+// signs: no difference. A NaN is the one input the instruction treats otherwise (largest magnitude, where the
+// definition's compare chain and the reference's table search give magnitude 0), so a NaN goes in as a zero of its sign.
+__device__ __forceinline__ float e2m1_nan_to_zero(float x) {
+    return x == x ? x : __uint_as_float(__float_as_uint(x) & 0x80000000u);
+}
 template <int BYTE>
 __device__ __forceinline__ uint32_t f32x2_to_e2m1_byte(uint32_t old, float a, float b) {
-    return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, a, b, 1.0f, BYTE);
+    return __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(old, e2m1_nan_to_zero(a), e2m1_nan_to_zero(b), 1.0f, BYTE);
 }
 
 // fp16 of twice the magnitude of the 8 e2m1 magnitudes: 0, 1, 2, 3, 4, 6, 8, 12; every low byte is zero, the high

@@ -197,6 +197,37 @@ def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
     assert np.array_equal(outs[(64, 0)][48:55], outs[(7, 48)]) and np.array_equal(outs[(64, 0)][48:], outs[(16, 48)])
 
 
+def test_quantizer_on_special_values(env, oracle):
+    """Ties between codes, the saturation boundary, signed zeros, infinities and NaN (a NaN element has magnitude 0 and
+    keeps its sign, format.rs:28-41, 66-69; it does not enter the block maximum, format.rs:76): codes and scales as the
+    oracle's, bit for bit."""
+    torch, fp4, kern = env
+    k, m = 256, 3
+    x = np.zeros((m, k), np.float32)
+    ties = np.float32([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 7.0, -0.25, -0.75, -1.25, -1.75, -2.5, -3.5, -5.0])
+    x[0, :16] = ties            # amax 7 -> scale e4m3(7/6); the elements land on and next to code boundaries
+    x[0, 16:32] = ties * 0.5
+    x[0, 32:48] = [0.0, -0.0, 1e-30, -1e-30, 3.0, -3.0, 6.0, -6.0, 1.0, 2.0, 4.0, 0.5, 1.5, -1.5, -0.5, -4.0]
+    x[1, :16] = np.float32([np.nan, 1.0, -2.0, 3.0] * 4)
+    x[1, 16:32] = np.float32([np.inf, 1.0, -np.inf, 2.0] * 4)
+    x[1, 32:48] = np.float32([-np.nan, 6.0, 0.0, -6.0] * 4)
+    x[2] = np.random.default_rng(2).normal(size=k).astype(np.float32) * 100
+    xb = bf16_bits(x)
+    xb[1, 0:16:4] = 0x7FC0      # bf16 NaN patterns survive the host-side rounding as NaN
+    xb[1, 32:48:4] = 0xFFC0
+    for g in (1.0, 0.3):
+        ws = fp4.Workspace(m, k)
+        lin = None
+        from ferrite_amd import synth
+        lin = synth.fp4_linear(128, k, 1, input_scale=1.0 / g).upload()
+        lin.quantize(kern, ws, dev_u16(torch, xb), k, m)
+        torch.cuda.synchronize()
+        codes, sf_tiled = ws.read(m, k)
+        want_codes, want_sf = oracle.quant_fp4(xb, lin.g)
+        assert np.array_equal(oracle.untile_scales(sf_tiled, m, k // 16).reshape(m, k // 16), want_sf)
+        assert np.array_equal(codes, want_codes)
+
+
 def test_fp4_argument_errors(env):
     torch, fp4, kern = env
     from ferrite_amd import synth
