@@ -52,7 +52,7 @@ int fe_hip_init(int ordinal) {
     if (ordinal < 0 || ordinal >= n) return fe_set_error(hipErrorInvalidDevice, "fe_hip_init", "no such device");
     HIPCHK(hipSetDevice(ordinal));
     g_ordinal = ordinal;
-    return 0;
+    return fe_exl3_static_setup_current_device();
 }
 
 int fe_hip_cu_count(int *out) {
@@ -152,14 +152,16 @@ static thread_local fe_event_t t_time_start = nullptr, t_time_stop = nullptr;
 
 int fe_hip_launch(fe_function_t f, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx, uint32_t by, uint32_t bz,
                   uint32_t lds_bytes, fe_stream_t s, void **params) {
+    // the events of fe_hip_time_next_launch belong to this launch, also when it is rejected below
+    fe_event_t time_start = t_time_start, time_stop = t_time_stop;
+    t_time_start = t_time_stop = nullptr;
     if (!f) return fe_set_error(hipErrorInvalidHandle, "fe_hip_launch", "null function");
     if (!gx || !gy || !gz || !bx || !by || !bz || (uint64_t)bx * by * bz > 1024)
         return fe_set_error(hipErrorInvalidConfiguration, "fe_hip_launch", "empty grid or block, or block > 1024");
-    if (t_time_start || t_time_stop) {
+    if (time_start || time_stop) {
         // one launch with events attached to its own dispatch: they take the kernel's begin and end timestamps, with no
         // marker packets in the stream around it (global sizes are in work-items here)
-        hipEvent_t a = (hipEvent_t)t_time_start, b = (hipEvent_t)t_time_stop;
-        t_time_start = t_time_stop = nullptr;
+        hipEvent_t a = (hipEvent_t)time_start, b = (hipEvent_t)time_stop;
         HIPCHK(hipExtModuleLaunchKernel((hipFunction_t)f, gx * bx, gy * by, gz * bz, bx, by, bz, lds_bytes, (hipStream_t)s, params,
                                         nullptr, a, b, 0));
         return 0;
