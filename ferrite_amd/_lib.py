@@ -79,6 +79,7 @@ SYMBOLS = {
     "fe_exl3_workspace_destroy": (I, [P]),
     "fe_exl3_workspace_xh": (I, [P, C.POINTER(U64), C.POINTER(U32), C.POINTER(U32)]),
     "fe_exl3_linear_forward": (I, [P, P, P, U64, I, U64, I, U32, P]),
+    "fe_exl3_linear_forward_static": (I, [P, P, P, U64, I, U64, I, U32]),
     "fe_exl3_linear_forward_is_one_launch": (I, [P, U32]),
     "fe_exl3_linear_keep_decoded": (I, [P, P, I]),
     "fe_exl3_linear_forward_swiglu": (I, [P, P, P, U64, U64, U32, U64, I, U32, P]),

@@ -535,6 +535,39 @@ int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern,
     return forward_from(l, kern, s, in, y, y_dtype, rows, ws, "fe_exl3_linear_forward");
 }
 
+}  // extern "C"
+
+int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                         fe_devptr_t y, int y_dtype, uint32_t rows, uint32_t max_rows, fe_devptr_t counters,
+                         size_t counters_bytes, fe_devptr_t xh, size_t xh_bytes, fe_devptr_t z, size_t z_bytes, const char *fn) {
+    if (!l || !kern || !x || !y) return fe_set_error(FE_ERR_ARG, fn, "null argument");
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32) return fe_set_error(FE_ERR_ARG, fn, "x is bf16 or f32");
+    char msg[200];
+    max_rows = std::min(max_rows, kMaxRowsPerPass);
+    if (rows == 0 || rows > max_rows) {
+        snprintf(msg, sizeof msg, "%s: %u rows (this entry point takes 1..%u)", l->name.c_str(), rows, max_rows);
+        return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
+    }
+    const size_t need_xh = (size_t)rows * l->k * 2, need_cnt = (size_t)((rows + 7) / 8) * (l->n / 128) * 4;
+    const size_t need_z = l->plan.ver == 2 ? (size_t)(l->programs + l->n / 128) * 128 * rows * 4
+                                           : (l->plan.sk > 1 ? (size_t)l->plan.sk * rows * l->n * 4 : 0);
+    if (need_xh > xh_bytes || need_cnt > counters_bytes || need_z > z_bytes) {
+        snprintf(msg, sizeof msg, "%s: %u rows of %ux%u need %zu B of rotated inputs (limit %zu), %zu B of partial sums (limit %zu), "
+                 "%zu B of counters (limit %zu)", l->name.c_str(), rows, l->k, l->n, need_xh, xh_bytes, need_z, z_bytes, need_cnt,
+                 counters_bytes);
+        return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
+    }
+    fe_exl3_workspace ws;  // views only: nothing is allocated and nothing is freed
+    ws.max_rows = rows, ws.max_k = l->k;
+    ws.xh.view(xh, xh_bytes), ws.z.view(z, z_bytes), ws.counters.view(counters, counters_bytes);
+    ws.z_len = z_bytes / 4, ws.counters_len = counters_bytes / 4;
+    RotInput in;
+    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
+    return forward_from(l, kern, s, in, y, y_dtype, rows, &ws, fn);
+}
+
+extern "C" {
+
 int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t gate,
                                   fe_devptr_t up, uint32_t ld, fe_devptr_t y, int y_dtype, uint32_t rows,
                                   const fe_exl3_workspace *ws) {

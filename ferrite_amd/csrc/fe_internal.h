@@ -69,6 +69,18 @@ struct FeBuf {
     }
 };
 
+// forward() of an EXL3 linear for at most max_rows rows over caller-provided device memory instead of a workspace object:
+// arrival counters (zero at rest), rotated inputs, split partial sums. Sizes that do not fit are FE_ERR_WORKSPACE.
+// Allocates nothing. (fe_exl3.cpp; used by fe_exl3_linear_forward_static.)
+struct fe_exl3_linear;
+struct fe_exl3_kernels;
+int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                         fe_devptr_t y, int y_dtype, uint32_t rows, uint32_t max_rows, fe_devptr_t counters,
+                         size_t counters_bytes, fe_devptr_t xh, size_t xh_bytes, fe_devptr_t z, size_t z_bytes, const char *fn);
+// Looks up the static scratch array of fe_exl3_linear_forward_static on the current device and clears its counters
+// (fe_exl3_static.hip); fe_hip_init calls it for the device it binds.
+int fe_exl3_static_setup_current_device();
+
 // How the prefill GEMM's output tiles (256 x 256) are spread over the CUs: `full` tiles are computed whole, one per
 // program; the `tiles - full` tiles of a last, mostly empty round are each cut `splits` ways along K (partials in a
 // workspace, then a reduce kernel). splits == 1 means nothing is cut (full == tiles).

@@ -262,6 +262,12 @@ class Linear:
         check(_lib.lib().fe_exl3_linear_forward(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype), y.data_ptr(),
                                                 int(y_dtype), rows, ws.h))
 
+    def forward_static(self, x, x_dtype: Dtype, y, y_dtype: Dtype, rows: int, stream=None):
+        """forward() without a Workspace and without any allocation: the scratch memory is a static device array of the
+        library (1..16 rows; larger shapes than it holds raise FeError). Calls that overlap on one GPU race."""
+        check(_lib.lib().fe_exl3_linear_forward_static(self.h, self.kern.h, _stream(stream), x.data_ptr(), int(x_dtype),
+                                                       y.data_ptr(), int(y_dtype), rows))
+
     def forward_swiglu(self, gate, up, ld: int, y, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
         """y[rows][n] = SwiGLU(gate, up)[rows][k] @ W with bf16 gate / up of row stride ld (pointers or tensors): the
         activation bf16(bf16(silu(gate)) * up) is formed as the input rotation reads it."""

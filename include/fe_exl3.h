@@ -114,6 +114,17 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
 /* Launches of that call: 1, 2, or 0 when the members run one after the other. */
 int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_t count, uint32_t rows,
                                           const fe_exl3_workspace *ws);
+/* forward() for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc). No counterpart in the reference, whose forward always takes a Workspace. The
+ * rotated inputs, split partial sums and arrival counters live in one static device array of FE_EXL3_STATIC_BYTES that
+ * every GPU the library runs on holds until the process ends; the call allocates and frees nothing. Same kernels and
+ * the same bits as fe_exl3_linear_forward. Limits: 1..FE_EXL3_STATIC_ROWS rows, rows * k * 2 <= 1 MiB of rotated inputs,
+ * plan.sk * rows * n * 4 bytes of partial sums <= FE_EXL3_STATIC_BYTES - 1 MiB - 16 KiB, n <= 524288; anything larger is
+ * FE_ERR_WORKSPACE. All calls on one GPU share the array: calls that overlap on one GPU (two streams) race; order them. */
+#define FE_EXL3_STATIC_BYTES (8u << 20)
+#define FE_EXL3_STATIC_ROWS 16
+int fe_exl3_linear_forward_static(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
+                                  int x_dtype, fe_devptr_t y, int y_dtype, uint32_t rows);
 /* Linear::rotate_input (linear.rs:289-298): xh = fp16(H(x * suh) / sqrt(128)) into the workspace. */
 int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
                                 int x_dtype, uint32_t rows, const fe_exl3_workspace *ws);
