@@ -20,6 +20,7 @@ constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row g
 constexpr uint32_t kGroupMax = 4;           // FE_EXL3_GROUP_MAX: linears of one grouped launch
 constexpr uint32_t kGroupRows = 64;         // rows of a grouped launch (one GEMV pass)
 constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
+constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one program of the balanced GEMV
 constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
 
@@ -46,6 +47,7 @@ struct fe_exl3_kernels {
     fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
     fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
     fe_function_t gemv_group[6][4] = {};                          // several linears of one input, [bits slot][row groups - 1]
+    fe_function_t gemvb[6][4] = {};                               // balanced over the CUs (plan ver 3), 1..4 linears a launch
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     fe_function_t gemm_reduce = nullptr;
@@ -121,6 +123,11 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         snprintf(nm, sizeof nm, "exl3_gemv_stream_b%d", kBits[i]);
         get(&k->gemv_stream[i], nm);
         for (int rg = 1; rg <= 4; rg++) {
+            snprintf(nm, sizeof nm, "exl3_gemvb_b%d_r%d", kBits[i], rg);
+            get(&k->gemvb[i][rg - 1], nm);
+            if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemvb[i][rg - 1], 84 * 1024);
+        }
+        for (int rg = 1; rg <= 4; rg++) {
             if (rg == 1)
                 snprintf(nm, sizeof nm, "exl3_gemv_group_b%d", kBits[i]);
             else
@@ -178,11 +185,15 @@ int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_
         if (miss < best) best = miss, sk = d;
     }
     if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) sk = 1;
-    // ver 1: the split-K GEMV for 1..64 rows, one summation order for all of them. ver 2 (FE_EXL3_STREAM=1): rows 1..16
-    // run the streamed GEMV with occ programs per CU instead.
-    uint32_t ver = env_is("FE_EXL3_STREAM", "1") ? 2 : 1, occ = 2;
+    // ver 3 (the default): the GEMV balanced over the CUs, occ programs per CU, for 1..64 rows, one summation order for all
+    // of them. ver 1 (FE_EXL3_VER=1): the split-K GEMV, sk splits. ver 2 (FE_EXL3_STREAM=1): rows 1..16 run the streamed
+    // GEMV with occ programs per CU.
+    uint32_t ver = env_is("FE_EXL3_STREAM", "1") ? 2 : 3, occ = 0;
+    if (const char *v = getenv("FE_EXL3_VER")) ver = (uint32_t)atoi(v);
+    if (ver == 2) occ = 2;
+    if (ver == 3) occ = 4;
     if (const char *o = getenv("FE_EXL3_OCC")) occ = (uint32_t)atoi(o);
-    *out = fe_exl3_plan{sk, 4, ver, ver == 2 ? occ : 0};
+    *out = fe_exl3_plan{sk, 4, ver, ver == 1 ? 0 : occ};
     return 0;
 }
 
@@ -197,6 +208,13 @@ int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out) {
 
 // Programs of the streamed GEMV: occ per CU, at most one per eight work units (FE_EXL3_PROGRAMS overrides the count).
 static uint32_t stream_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p, uint32_t k, uint32_t n) {
+    if (p.ver == 3) {
+        // balanced GEMV: occ programs per CU, each a run of at least min_units 128-channel blocks of one column block
+        const uint32_t units = (k / 128) * (n / 128), occ = p.occ ? p.occ : 4;
+        uint32_t min_units = 4;
+        if (const char *e = getenv("FE_EXL3_MIN_UNITS")) min_units = std::max(1, atoi(e));  // tuning
+        return std::max(1u, std::min(occ * std::max(kern->cus, 1u), units / min_units));
+    }
     if (p.ver != 2) return 0;
     const uint32_t units = (k / 64) * (n / 128), occ = p.occ ? p.occ : 2;
     uint32_t progs = std::min(occ * kern->cus, units / 8);
@@ -302,12 +320,13 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     std::vector<size_t> zs, nbs;  // per linear, for the grouped launch: room for the kGroupMax largest together
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
-        zs.push_back(l->plan.ver == 2 ? 0 : (size_t)l->plan.sk * l->n);
+        zs.push_back(l->plan.ver == 3 ? (size_t)(l->programs + l->n / 128) * 128 : l->plan.ver == 2 ? 0 : (size_t)l->plan.sk * l->n);
         nbs.push_back(l->n / 128);
         max_hat = std::max(max_hat, hat_bytes(l));
         max_k = std::max<size_t>(max_k, l->k);
-        if (l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
-        if (l->programs) max_zs = std::max<size_t>(max_zs, (size_t)(l->programs + l->n / 128) * 128);
+        if (l->plan.ver != 3 && l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
+        if (l->plan.ver == 3) max_z = std::max<size_t>(max_z, (size_t)(l->programs + l->n / 128) * 128);
+        if (l->plan.ver == 2) max_zs = std::max<size_t>(max_zs, (size_t)(l->programs + l->n / 128) * 128);
         max_nb = std::max<size_t>(max_nb, l->n / 128);
     }
     auto *ws = new fe_exl3_workspace;
@@ -433,6 +452,14 @@ static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
     const char *e = getenv("FE_EXL3_NO_FUSED_ROT");  // read per call: tests compare both paths in one process
     const bool off = e && atoi(e) != 0;
     const fe_exl3_plan &p = l->plan;
+    if (p.ver == 3) {
+        // every program rotates the channels of its own run: (row, 128-channel block) pairs, 8 at a time
+        if (off || rows < 1 || rows > kMaxRowsPerPass) return false;
+        uint32_t pairs = 16;
+        if (const char *t = getenv("FE_EXL3_FUSED_ROT_PAIRS")) pairs = (uint32_t)atoi(t);
+        const uint32_t units = (l->k / 128) * (l->n / 128);
+        return rows * ((units + l->programs - 1) / l->programs) <= pairs;
+    }
     if (off || rows < 1 || rows > kMaxRowsPerPass || p.ver == 2 || (l->k / 64 / p.sk) % 2) return false;
     // every column block repeats the rotation of its K range: (row, 128-block) pairs a program, 8 at a time. Measured on
     // 5120 x 17408 (8 blocks a program): one launch wins up to 4 rows (19.9 against 22.3 us at 1 row), the separate
@@ -447,6 +474,68 @@ int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devpt
     return launch_rows(l, s, xh, y, y_dtype, rows, ws, RotInput{});
 }
 
+// mirrors GemvJob of k_exl3.hip
+struct GemvJobArgs {
+    uint32_t count, first[kGroupMax + 1];
+    struct Member {
+        fe_devptr_t trellis, svh, suh, xh, y, z, counters;
+        uint32_t n, programs, stride_k, stride_nb, base, rem, inv_base, inv_base1;
+    } m[kGroupMax];
+};
+static_assert(sizeof(GemvJobArgs) == 24 + kGroupMax * 88, "GemvJob layout");
+
+// Room a balanced launch takes in the workspace: partial sums (floats) and counters of one member at `rows` rows.
+static size_t job_z(const fe_exl3_linear *l, uint32_t rows) { return (size_t)(l->programs + l->n / 128) * 128 * rows; }
+
+// The balanced GEMV (plan ver 3) for 1..4 linears of one input in one launch: member i reads its rotated input at xhs[i]
+// (in.x == 0) or rotates in.x itself and leaves the result at xhs[i]. The caller has checked rows, k and bits.
+static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t s, const fe_devptr_t *xhs, const fe_devptr_t *ys,
+                      int y_dtype, uint32_t rows, const fe_exl3_workspace *ws, const RotInput &in, const char *fn) {
+    GemvJobArgs g{};
+    g.count = (uint32_t)count;
+    uint32_t programs = 0, run_steps = 0;
+    size_t z_at = 0, cnt_at = 0;
+    char msg[200];
+    for (size_t i = 0; i < count; i++) {
+        const fe_exl3_linear *l = ls[i];
+        GemvJobArgs::Member &m = g.m[i];
+        if (z_at + job_z(l, rows) > ws->z_len || cnt_at + l->n / 128 > ws->counters_len) {
+            snprintf(msg, sizeof msg, "%s: %u rows do not fit the workspace (partial sums %zu of %zu floats, counters %zu of %zu)",
+                     l->name.c_str(), rows, z_at + job_z(l, rows), ws->z_len, cnt_at + l->n / 128, ws->counters_len);
+            return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
+        }
+        m.trellis = l->view.trellis, m.svh = l->view.svh, m.suh = l->view.suh, m.xh = xhs[i], m.y = ys[i];
+        m.z = ws->z.p + z_at * 4, m.counters = ws->counters.p + cnt_at * 4;
+        m.n = l->n, m.programs = l->programs;
+        view_strides(l->view, &m.stride_k, &m.stride_nb);
+        g.first[i] = programs;
+        programs += l->programs;
+        z_at += job_z(l, rows), cnt_at += l->n / 128;
+        const uint32_t units = (l->k / 128) * (l->n / 128);
+        m.base = units / l->programs, m.rem = units % l->programs;
+        m.inv_base = 0xffffffffu / m.base, m.inv_base1 = 0xffffffffu / (m.base + 1);
+        run_steps = std::max(run_steps, 2 * ((units + l->programs - 1) / l->programs));
+    }
+    for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
+    // staged inputs: the whole run where the LDS budget holds it for `rows` rows, else chunks of a multiple of 4 load steps
+    const uint32_t red = rows * kRedPitch * 4;
+    uint32_t chunk = std::max(4u, ((kJobLdsBudget - red) / rows - 16) / 128 / 4 * 4);
+    chunk = std::min(chunk, (run_steps + 3) / 4 * 4);
+    uint32_t lds = red + rows * (chunk * 128 + 16);
+    // Exactly occ programs a CU: the dispatcher fills a CU as far as registers and LDS allow (5 programs) before it moves
+    // on, which would leave CUs empty while others hold 5; an LDS request that fits occ times into the CU's 160 KB, and
+    // not occ + 1 times, makes the CUs take occ each.
+    if (const uint32_t occ = ls[0]->plan.occ; occ && !env_is("FE_EXL3_NO_LDS_PAD", "1")) lds = std::max(lds, 163840u / (occ + 1) + 512);
+    uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld;
+    fe_devptr_t x = in.x, x2 = in.x2;
+    // (the last argument exists only in timeline-probe builds of the code object; the shipped kernels take ten)
+    static const fe_devptr_t stamps = getenv("FE_EXL3_STAMPS") ? (fe_devptr_t)strtoull(getenv("FE_EXL3_STAMPS"), nullptr, 0) : 0;
+    fe_devptr_t st = stamps;
+    uint32_t inv_spb = 0xffffffffu / (k / 64);
+    void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb, &st};
+    return fe_hip_launch(ls[0]->kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
+}
+
 static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
                        const fe_exl3_workspace *ws, const RotInput &in) {
     if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "null argument");
@@ -459,6 +548,13 @@ static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
             return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
         }
         return launch_gemm(l, s, xh, y, y_dtype, rows, ws);
+    }
+    if (p.ver == 3) {
+        if (rows == 0 || rows > ws->max_rows) {
+            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
+            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
+        }
+        return launch_job(&l, 1, s, &xh, &y, y_dtype, rows, ws, in, "fe_exl3_linear_gemv_rotated");
     }
     if (p.ver == 2 && rows >= 1 && rows <= kStreamRows) {
         if (rows > ws->max_rows || ws->z_len < (size_t)(l->programs + l->n / 128) * 128 * rows || ws->counters_len < l->n / 128) {
@@ -549,7 +645,8 @@ int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, f
         return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
     }
     const size_t need_xh = (size_t)rows * l->k * 2, need_cnt = (size_t)((rows + 7) / 8) * (l->n / 128) * 4;
-    const size_t need_z = l->plan.ver == 2 ? (size_t)(l->programs + l->n / 128) * 128 * rows * 4
+    const size_t need_z = l->plan.ver == 3 ? job_z(l, rows) * 4
+                          : l->plan.ver == 2 ? (size_t)(l->programs + l->n / 128) * 128 * rows * 4
                                            : (l->plan.sk > 1 ? (size_t)l->plan.sk * rows * l->n * 4 : 0);
     if (need_xh > xh_bytes || need_cnt > counters_bytes || need_z > z_bytes) {
         snprintf(msg, sizeof msg, "%s: %u rows of %ux%u need %zu B of rotated inputs (limit %zu), %zu B of partial sums (limit %zu), "
@@ -608,9 +705,11 @@ static bool group_fits(const fe_exl3_linear *const *ls, size_t count, uint32_t r
     bool f = true;
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = ls[i];
-        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.ver == 2) return false;
+        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.ver == 2 ||
+            l->plan.ver != ls[0]->plan.ver)
+            return false;
         f = f && fused_rotation_fits(l, rows);
-        z += (size_t)l->plan.sk * rows * l->n;
+        z += l->plan.ver == 3 ? job_z(l, rows) : (size_t)l->plan.sk * rows * l->n;
         nb += l->n / 128;
     }
     if (!f && count * (size_t)rows * ls[0]->k * 2 > ws->xh.bytes) return false;
@@ -637,6 +736,24 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
     if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
         return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "x is bf16 or f32");
     if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "bad y dtype");
+    if (ls[0]->plan.ver == 3) {
+        RotGroupArgs r{};
+        fe_devptr_t xhs[kGroupMax] = {};
+        for (size_t i = 0; i < count; i++) {
+            if (!ys[i]) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null output");
+            xhs[i] = ws->xh.p + i * (size_t)rows * ls[i]->k * 2;
+            r.suh[i] = ls[i]->view.suh, r.xh[i] = xhs[i];
+        }
+        RotInput in;
+        uint32_t x_mode = (uint32_t)x_dtype & 1, k = ls[0]->k;
+        if (fused) {
+            in.x = x, in.mode = x_mode, in.ld = k;
+        } else {  // one launch rotates the input for every member
+            void *rargs[] = {&r, &x, &x_mode, &k};
+            FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
+        }
+        return launch_job(ls, count, s, xhs, ys, y_dtype, rows, ws, in, "fe_exl3_linear_forward_group");
+    }
     GemvGroupArgs g{};
     RotGroupArgs r{};
     g.count = (uint32_t)count;

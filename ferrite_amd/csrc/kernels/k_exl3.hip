@@ -232,6 +232,9 @@ struct LaneWords {
     uint32_t w[BITS + 1];  // w[0] = the word before the lane's run
 };
 
+#ifdef FE_NO_NT
+#define __builtin_nontemporal_load(p) (*(p))
+#endif
 template <int BITS>
 __device__ __forceinline__ LaneWords<BITS> load_lane_words(const uint32_t* run, const uint32_t* prev) {
     LaneWords<BITS> r;
@@ -263,49 +266,50 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words(const uint32_t* run, 
     return r;
 }
 
-// The 32-bit window of the lane's local stream starting at bit S (bit 0 = most significant bit of w[0]).
-template <int BITS, int S>
-__device__ __forceinline__ uint32_t window32(const LaneWords<BITS>& lw) {
-    constexpr int wi = S / 32, o = S % 32;
-    if constexpr (o == 0) {
-        return lw.w[wi];
-    } else {
-        uint32_t r = __builtin_amdgcn_alignbit(lw.w[wi], lw.w[wi + 1], 32 - o);
-        // opaque to the optimizer: two states share this window (one funnel shift for both); without this the
-        // compiler re-derives each state from the words with its own shift
+// The lane's local stream: bit 0 = most significant bit of w[0]; local position U (0..31) owns the 16 bits ending at local
+// bit (U + 1) * BITS + 32. A state either lies inside one word (one extract), or straddles the boundary between w[i - 1]
+// and w[i]: all states that straddle one boundary are cut out of one 32-bit window over it (low half of w[i - 1], high
+// half of w[i]): BITS funnel shifts a load step instead of one per state or per pair of states.
+template <int BITS>
+struct LaneWindows {
+    uint32_t b[BITS + 1];  // b[i], i >= 1: the window over the boundary in front of w[i]
+};
+template <int BITS>
+__device__ __forceinline__ LaneWindows<BITS> lane_windows(const LaneWords<BITS>& lw) {
+    LaneWindows<BITS> win;
+    win.b[0] = 0;
+#pragma unroll
+    for (int i = 1; i <= BITS; i++) {
+        uint32_t r = __builtin_amdgcn_alignbit(lw.w[i - 1], lw.w[i], 16);
+        // opaque to the optimizer, which would otherwise fold window and extract into a funnel shift and a mask per state
         asm("" : "+v"(r));
-        return r;
+        win.b[i] = r;
     }
+    return win;
 }
 
-// x = state * MUL1 of local position U (0..31): its state ends at local stream bit (U + 1) * BITS + 32.
+// x = state * MUL1 of local position U.
 template <int BITS, int U>
-__device__ __forceinline__ uint32_t lane_x(const LaneWords<BITS>& lw) {
-    constexpr int end = (U + 1) * BITS + 32;
-    if constexpr (16 % BITS == 0) {
-        // positions 16 / BITS apart share one 32-bit window: the earlier one in its high half
-        constexpr int D = 16 / BITS;
-        if constexpr ((U / D) % 2 == 0)
-            return mul1_x<1>(window32<BITS, end - 16>(lw));
-        else
-            return mul1_x<0>(window32<BITS, end - 32>(lw));
-    } else {
-        if constexpr (end % 32 == 16)
-            return mul1_x<1>(lw.w[end / 32]);
-        else if constexpr (end % 32 == 0)
-            return mul1_x<0>(lw.w[end / 32 - 1]);
-        else if constexpr (end % 32 > 16)
-            return mul1_x<0>(lw.w[end / 32] >> (32 - end % 32));
-        else
-            return mul1_x<0>(window32<BITS, end - 32>(lw));
-    }
+__device__ __forceinline__ uint32_t lane_x(const LaneWords<BITS>& lw, const LaneWindows<BITS>& win) {
+    constexpr int end = (U + 1) * BITS + 32, wi = end / 32, r = end % 32;
+    uint32_t state;
+    if constexpr (r == 0)
+        state = lw.w[wi - 1] & 0xffffu;
+    else if constexpr (r == 16)
+        state = lw.w[wi] >> 16;
+    else if constexpr (r > 16)
+        state = __builtin_amdgcn_ubfe(lw.w[wi], 32 - r, 16);
+    else
+        state = __builtin_amdgcn_ubfe(win.b[wi], 16 - r, 16);
+    return state * 0x83DCD12Du;
 }
 
 // The lane's 32 values as MFMA operands op[h][kh]: rows n = q + 8 h of the tile, k = 8 kh .. 8 kh + 7 in order.
 // Local position u = 8 c + i (fragment lane 4q + c, value i) is k = 2c + (i & 1) + 8 ((i >> 1) & 1), n half i >> 2.
 template <int BITS>
 __device__ __forceinline__ void decode_lane(const LaneWords<BITS>& lw, f16x8 (&op)[2][2]) {
-#define FE_PAIR(H, KH, C) mul1_finish2(lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H)>(lw), lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H) + 1>(lw))
+    const LaneWindows<BITS> win = lane_windows<BITS>(lw);
+#define FE_PAIR(H, KH, C) mul1_finish2(lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H)>(lw, win), lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H) + 1>(lw, win))
 #define FE_OP(H, KH)                                                                             \
     {                                                                                            \
         u32x4 t = {FE_PAIR(H, KH, 0), FE_PAIR(H, KH, 1), FE_PAIR(H, KH, 2), FE_PAIR(H, KH, 3)};  \
@@ -559,7 +563,7 @@ __device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const
         const float* src = red + row * GEMV_RED_PITCH + 4 * l32;
         store_agent_f32x4(z + ((size_t)split * m + row) * n + col0 + 4 * l32, *(const f32x4*)src);
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's stores are acknowledged at agent scope
+    agent_stores_wait();  // this lane's stores are acknowledged at agent scope
     __syncthreads();
     if (tid == 0) {
         uint32_t old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -657,6 +661,424 @@ GEMV_GROUP_FAMILY(4)
 GEMV_GROUP_FAMILY(5)
 GEMV_GROUP_FAMILY(6)
 GEMV_GROUP_FAMILY(8)
+
+// ---- decode GEMV, balanced over the CUs (1..64 rows) ------------------------------------------------------------------
+//
+// Work unit = one 128-channel block of K of one 128-column block of N (two load steps); units are ordered column block
+// by column block and the member's `programs` programs each take one contiguous run of them, base or base + 1 units long,
+// whatever the shape: every program decodes the same number of weights, so with a multiple of the CU count of programs
+// every CU does. A run may start and end inside a column block, so a block's sum is assembled from segments: each program
+// leaves the partial sums of its segment of block nb in z[program + nb] and bumps the block's arrival counter; the
+// program that arrives last adds the segments in program order (the order does not depend on who is last: deterministic),
+// applies the output rotation and re-arms the counter. The partition depends on (k, n, programs) only, never on the
+// row count: row r of a batch has the bits of the single-row call. Inside a program the work is laid out as in the
+// split-K kernel above: 4 wavefronts owning 2 of the block's 8 tiles each, the rotated inputs of the run staged in LDS
+// (rotated here when src.x is set), four load steps in flight per lane.
+struct GemvMember {
+    const uint32_t* trellis;
+    const uint16_t *svh, *suh;
+    uint16_t* xh;        // rotated inputs [m][k]: read, or (rotating here) left there by the programs of column block 0
+    void* y;
+    float* z;            // segment partial sums [programs + n / 128][m][128]
+    uint32_t* counters;  // arrivals per column block, zero at rest
+    uint32_t n, programs, stride_k, stride_nb;
+    uint32_t base, rem;            // units / programs, units % programs
+    uint32_t inv_base, inv_base1;  // floor((2^32 - 1) / base), floor((2^32 - 1) / (base + 1))
+};
+struct GemvJob {
+    uint32_t count, first[FE_EXL3_GROUP_MAX + 1];  // member i owns programs first[i] .. first[i + 1] - 1 of the grid
+    GemvMember m[FE_EXL3_GROUP_MAX];
+};
+
+// x / d for x < 2^31 with inv = floor((2^32 - 1) / d): a multiply-high and one correction (uniform operands: scalar code).
+__device__ __forceinline__ uint32_t udiv_inv(uint32_t x, uint32_t d, uint32_t inv) {
+    uint32_t q = __umulhi(x, inv);
+    return q + ((q + 1) * d <= x ? 1u : 0u);
+}
+
+// FE_STAMP builds (timeline probes, never the shipped code object) take one more kernel argument: 16 slots per program,
+// wall-clock stamps (100 MHz) written by thread 0 and the hardware id of the CU.
+#ifdef FE_STAMP
+#define FE_STAMP_ARG , uint64_t* stamps
+#define FE_STAMP_PASS , stamps
+#define FE_STAMP_AT(i) \
+    if (threadIdx.x == 0) stamps[(size_t)blockIdx.x * 16 + (i)] = __builtin_amdgcn_s_memrealtime()
+#else
+#define FE_STAMP_ARG
+#define FE_STAMP_PASS
+#define FE_STAMP_AT(i)
+#endif
+
+// The ring of load steps turned left by `phase` slots, so that the oldest step in flight sits in slot 0 again.
+template <int BITS, int DEPTH>
+__device__ __forceinline__ void ring_turn(LaneWords<BITS> (&ring)[DEPTH], uint32_t phase) {
+    for (; phase; phase--) {
+        LaneWords<BITS> t = ring[0];
+#pragma unroll
+        for (int i = 0; i + 1 < DEPTH; i++) ring[i] = ring[i + 1];
+        ring[DEPTH - 1] = t;
+    }
+}
+
+// A lane's words of one load step through a buffer resource over the whole trellis: the lane's byte offsets (run, word
+// before the run) are loop constants in vector registers and the step's position is a scalar offset, so walking the run
+// costs no vector instructions; reads past the end of the trellis return zero instead of faulting. Streaming (nt) loads.
+template <int BITS>
+__device__ __forceinline__ LaneWords<BITS> load_lane_words_buf(__amdgpu_buffer_rsrc_t rs, uint32_t run_b, uint32_t prev_b,
+                                                               uint32_t soff) {
+    constexpr int NT = 2;
+    LaneWords<BITS> r;
+    r.w[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, prev_b, soff, NT);
+    if constexpr (BITS == 1) {
+        r.w[1] = __builtin_amdgcn_raw_buffer_load_b32(rs, run_b, soff, NT);
+    } else if constexpr (BITS == 2) {
+        u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(rs, run_b, soff, NT);
+        r.w[1] = t[0], r.w[2] = t[1];
+    } else if constexpr (BITS == 3) {
+        u32x3 t = __builtin_amdgcn_raw_buffer_load_b96(rs, run_b, soff, NT);
+        r.w[1] = t[0], r.w[2] = t[1], r.w[3] = t[2];
+    } else {
+        u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(rs, run_b, soff, NT);
+        r.w[1] = t[0], r.w[2] = t[1], r.w[3] = t[2], r.w[4] = t[3];
+        if constexpr (BITS == 5) {
+            r.w[5] = __builtin_amdgcn_raw_buffer_load_b32(rs, run_b + 16, soff, NT);
+        } else if constexpr (BITS == 6) {
+            u32x2 u = __builtin_amdgcn_raw_buffer_load_b64(rs, run_b + 16, soff, NT);
+            r.w[5] = u[0], r.w[6] = u[1];
+        } else if constexpr (BITS == 7) {
+            u32x3 u = __builtin_amdgcn_raw_buffer_load_b96(rs, run_b + 16, soff, NT);
+            r.w[5] = u[0], r.w[6] = u[1], r.w[7] = u[2];
+        } else if constexpr (BITS == 8) {
+            u32x4 u = __builtin_amdgcn_raw_buffer_load_b128(rs, run_b + 16, soff, NT);
+            r.w[5] = u[0], r.w[6] = u[1], r.w[7] = u[2], r.w[8] = u[3];
+        }
+    }
+    return r;
+}
+
+template <int BITS, int RG>
+__device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uint32_t k, uint32_t m, uint32_t y_mode,
+                                           uint32_t chunk, uint32_t inv_spb, const RotSrc src FE_STAMP_ARG) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    __shared__ uint32_t last_flag;
+    FE_STAMP_AT(0);
+#ifdef FE_STAMP
+    if (threadIdx.x == 0) {
+        uint32_t hw = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_REG_HW_ID
+        uint32_t xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // HW_REG_XCC_ID
+        stamps[(size_t)blockIdx.x * 16 + 8] = ((uint64_t)xcc << 32) | hw;
+        stamps[(size_t)blockIdx.x * 16 + 9] = __builtin_amdgcn_s_memtime();
+    }
+#endif
+    constexpr uint32_t tw = 8 * BITS;
+#ifndef FE_GEMVB_DEPTH
+#define FE_GEMVB_DEPTH 4
+#endif
+    constexpr int DEPTH = FE_GEMVB_DEPTH;  // load steps in flight per lane
+    constexpr int GROUP = 8;               // steps of straight-line code per loop iteration (a multiple of DEPTH)
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
+    const uint32_t n = mb.n, spb = k / 64, upb = spb / 2;  // load steps, units a column block
+    const uint32_t base = mb.base, rem = mb.rem;
+    const uint32_t u0 = p * base + (p < rem ? p : rem);
+    const uint32_t S = 2 * (base + (p < rem ? 1 : 0));  // load steps of this run
+    if (S == 0) return;
+    uint32_t nb = udiv_inv(2 * u0, spb, inv_spb), st = 2 * u0 - nb * spb;  // where the run stands: column block, load step
+    const uint32_t nb_run0 = nb, st_run0 = st;
+
+    float* red = (float*)lds;                                        // [m][GEMV_RED_PITCH] sums of a finished segment
+    unsigned char* xs = (unsigned char*)(red + m * GEMV_RED_PITCH);  // [m][xpitch] rotated inputs of a chunk of the run
+    const uint32_t xpitch = chunk * 128 + 16;
+
+    const uint32_t lane_word = g * mb.stride_k + (2 * wave + tau) * tw;
+    const uint32_t run_b = 4 * (lane_word + q * BITS), prev_b = 4 * (lane_word + (q * BITS + tw - 1) % tw);
+    const uint32_t step_bytes = 16 * mb.stride_k;                     // 4 k steps
+    const uint32_t wrap_bytes = 4 * mb.stride_nb - spb * step_bytes;  // from the end of a column block to the next (mod 2^32)
+    const __amdgpu_buffer_rsrc_t trs =
+        __builtin_amdgcn_make_buffer_rsrc((void*)mb.trellis, 0, (k / 16) * (n / 16) * tw * 4, 0x00020000);
+    uint32_t snext = nb * mb.stride_nb * 4 + st * step_bytes;  // byte offset of the next load step to request
+
+    uint32_t xrow[RG];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) {
+        uint32_t row = 16 * rg + r;
+        xrow[rg] = (row < m ? row : m - 1) * xpitch + g * 32;
+    }
+    f32x4 acc[RG][2];
+#pragma unroll
+    for (int rg = 0; rg < RG; rg++) acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+    const uint32_t hw = tid >> 5, l32 = tid & 31;
+    // Rotating here: (row, 128-channel block) pairs of a chunk go to the half wavefronts: half wavefront hw takes blocks hw,
+    // hw + 8, ... of every row. The first pair's loads go out ahead of the trellis loads (loads return in order), so
+    // that the rotation runs while the first trellis words are still on their way.
+    const bool rotating = src.x != nullptr;
+    struct RotAt {
+        size_t at, xat;
+        uint32_t c, off;
+        bool keep;
+    };
+    auto rot_at = [&](uint32_t c0, uint32_t row, uint32_t b) {
+        RotAt a;
+        uint32_t gst = st_run0 + c0 + 2 * b, blk = 0;  // load step counted from the start of the run's first column block
+        if (gst >= spb) gst -= spb, blk = 1;
+        if (gst >= spb) blk += gst / spb, gst %= spb;
+        a.c = gst * 64 + 4 * l32;
+        a.at = (size_t)row * k + a.c;
+        a.xat = (size_t)row * src.ld + a.c;
+        a.off = row * xpitch + b * 256 + 8 * l32;
+        a.keep = nb_run0 + blk == 0;  // column block 0 sees every channel: its programs leave xh behind
+        return a;
+    };
+    RotRaw rot_raw = {};
+    if (rotating) {
+        const uint32_t nblk = (S < chunk ? S : chunk) / 2;
+        if (hw < nblk) {
+            RotAt a = rot_at(0, 0, hw);
+            rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+        }
+    }
+    // the output scales of this lane's four columns of the block the run stands in (for the program that finishes it)
+    u32x2 sv = *(const u32x2*)(mb.svh + nb * 128 + 4 * l32);
+
+    // refill cursor: the next load step to request
+    uint32_t rj = 0, rst = st;
+    auto issue = [&](LaneWords<BITS>& slot) {
+        slot = load_lane_words_buf<BITS>(trs, run_b, prev_b, snext);
+        if (rj + 1 < S) {  // past the end of the run the last step is requested again (and never used)
+            rj++;
+            snext += step_bytes;
+            if (++rst == spb) rst = 0, snext += wrap_bytes;
+        }
+    };
+    LaneWords<BITS> ring[DEPTH];  // indexed by constants only, so it stays in registers
+#pragma unroll
+    for (int j = 0; j < DEPTH; j++) issue(ring[j]);
+
+    auto one = [&](LaneWords<BITS>& slot, uint32_t t) {  // t: load step within the staged chunk
+        f16x8 op[2][2];
+        decode_lane<BITS>(slot, op);
+        issue(slot);
+        // keep the refill where it is issued: left alone, the scheduler sinks the loads to the end of the group, right in
+        // front of the wait for them
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            const unsigned char* xp = xs + xrow[rg] + t * 128;
+            f16x8 x0 = *(const f16x8*)xp, x1 = *(const f16x8*)(xp + 16);
+            acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[rg][0], 0, 0, 0);
+            acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[rg][1], 0, 0, 0);
+            acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[rg][0], 0, 0, 0);
+            acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    // H over the 128 sums of a row (4 a lane of a half wavefront), * svh / sqrt(128) with the prefetched scales, stored.
+    auto finish = [&](float (&v)[4], uint32_t col0, uint32_t row) {
+        fwht128_half_wave(v, l32);
+        v[0] = v[0] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] & 0xffff);
+        v[1] = v[1] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] >> 16);
+        v[2] = v[2] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] & 0xffff);
+        v[3] = v[3] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] >> 16);
+        store4(mb.y, y_mode, (size_t)row * n + col0 + 4 * l32, v);
+    };
+
+    // The segment of column block fnb that ends here: its sums meet in LDS, and then either are the block's sums (the
+    // block lies in this run alone) or go to z for the program that arrives last at the block.
+    auto flush = [&](uint32_t fnb) {
+        FE_STAMP_AT(2);
+        __syncthreads();  // the previous segment's readers are done with `red`
+        // rows 4 g .. 4 g + 3 of A are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32 (tile g >> 1 of
+        // its pair, n = 4 (g & 1) + i + 8 h): a lane's four sums of either half are four neighbouring columns
+        float* rp = red + 32 * wave + 16 * (g >> 1) + 4 * (g & 1);
+#pragma unroll
+        for (int rg = 0; rg < RG; rg++) {
+            uint32_t row = 16 * rg + r;  // accumulator column = input row
+            if (row < m) {
+                *(f32x4*)(rp + row * GEMV_RED_PITCH) = acc[rg][0];
+                *(f32x4*)(rp + row * GEMV_RED_PITCH + 8) = acc[rg][1];
+            }
+            acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        }
+        __syncthreads();
+        const uint32_t col0 = fnb * 128;
+        // programs of the block's first and last unit (units are dealt base + 1 to the first rem programs, base to the rest)
+        const uint32_t cut = rem * (base + 1), ua = fnb * upb, ub = ua + upb - 1;
+        const uint32_t first_prog = ua < cut ? udiv_inv(ua, base + 1, mb.inv_base1) : rem + udiv_inv(ua - cut, base, mb.inv_base);
+        const uint32_t last_prog = ub < cut ? udiv_inv(ub, base + 1, mb.inv_base1) : rem + udiv_inv(ub - cut, base, mb.inv_base);
+        if (first_prog == last_prog) {
+            for (uint32_t row = hw; row < m; row += 8) {
+                f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
+                float v[4] = {t[0], t[1], t[2], t[3]};
+                finish(v, col0, row);
+            }
+            return;
+        }
+        // Hand-off of the segment's sums to another program, possibly on another XCD with its own L2:
+        //  1. every lane stores its piece with agent-scope (write-through) stores and waits until they are acknowledged;
+        //  2. the workgroup barrier orders all lanes' acknowledged stores before lane 0's arrival at the counter
+        //     (an agent-scope atomic, performed at the shared level);
+        //  3. the program whose arrival completes the count reads the segments with agent-scope loads (past its own L2)
+        //     after the barrier that publishes last_flag.
+        // Every byte that crosses is written through and read through, so no cache write-back or invalidate is needed.
+        float* zseg = mb.z + (size_t)(p + fnb) * m * 128;
+        for (uint32_t row = hw; row < m; row += 8)
+            store_agent_f32x4(zseg + row * 128 + 4 * l32, *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32));
+        FE_STAMP_AT(3);
+        agent_stores_wait();
+        __syncthreads();
+        FE_STAMP_AT(4);
+        if (tid == 0) {
+            uint32_t old = __hip_atomic_fetch_add(&mb.counters[fnb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            last_flag = (old == last_prog - first_prog);
+        }
+        __syncthreads();
+        FE_STAMP_AT(5);
+        if (last_flag) {
+            // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB segments each, 8 or 12 agent-scope
+            // loads in flight (each takes a trip to memory: the trips overlap); every row's segments are added in program
+            // order (as many in flight as the registers hold without costing the kernel a resident wavefront). Up to 8 rows
+            // every half wavefront has at most one row and takes all of the batch from it.
+            const uint32_t nseg = last_prog - first_prog + 1;
+            const __amdgpu_buffer_rsrc_t zrs = __builtin_amdgcn_make_buffer_rsrc(
+                (void*)(mb.z + (size_t)(first_prog + fnb) * m * 128), 0, nseg * m * 512, 0x00020000);
+            auto rows_of = [&](auto rb_tag) {
+                constexpr int RB = decltype(rb_tag)::value, SB = (BITS <= 4 && RG == 1 ? 12 : 8) / RB;
+                for (uint32_t row0 = hw; row0 < m; row0 += 8 * RB) {
+                    float v[RB][4];
+#pragma unroll
+                    for (int j = 0; j < RB; j++) v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.f;
+                    for (uint32_t sp0 = 0; sp0 < nseg; sp0 += SB) {
+                        f32x4 t[RB * SB];
+#pragma unroll
+                        for (int j = 0; j < RB; j++) {
+                            const uint32_t row = row0 + 8 * j < m ? row0 + 8 * j : row0;
+#pragma unroll
+                            for (int b = 0; b < SB; b++)  // (past the last segment: out of the buffer's range, reads zero)
+                                t[j * SB + b] = load_agent_f32x4(zrs, row * 512 + 16 * l32, (sp0 + b) * m * 512);
+                        }
+#pragma unroll
+                        for (int j = 0; j < RB; j++)
+#pragma unroll
+                            for (int b = 0; b < SB; b++)
+                                if (sp0 + b < nseg) {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) v[j][e] += t[j * SB + b][e];
+                                }
+                    }
+#pragma unroll
+                    for (int j = 0; j < RB; j++) {
+                        const uint32_t row = row0 + 8 * j;
+                        if (row < m) finish(v[j], col0, row);
+                    }
+                }
+            };
+            if (m <= 8)
+                rows_of(std::integral_constant<int, 1>{});
+            else
+                rows_of(std::integral_constant<int, 2>{});
+            if (tid == 0) __hip_atomic_store(&mb.counters[fnb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            FE_STAMP_AT(6);
+        }
+    };
+
+    for (uint32_t c0 = 0; c0 < S; c0 += chunk) {
+        const uint32_t cs = S - c0 < chunk ? S - c0 : chunk;
+        if (c0) __syncthreads();  // the previous chunk's readers are done with xs
+        if (rotating) {
+            const uint32_t nblk = cs / 2;
+            uint32_t row = 0, b = hw;
+            RotAt a = {};
+            const bool any = b < nblk;
+            if (any) {
+                a = rot_at(c0, row, b);
+                if (c0) rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+            }
+            while (any && row < m) {
+                u32x2 o = rot_finish(rot_raw, src.mode, l32);
+                *(u32x2*)(xs + a.off) = o;
+                if (a.keep && mb.xh) *(u32x2*)(mb.xh + a.at) = o;
+                b += 8;
+                if (b >= nblk) b = hw, row++;
+                if (row < m) {
+                    a = rot_at(c0, row, b);
+                    rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+                }
+            }
+        } else {  // rotated inputs of the chunk's load steps -> xs [row][cs * 64 fp16], NB 16-byte pieces in flight a thread
+            constexpr int NB = RG == 1 ? FE_STAGE_NB1 : 8;
+            const uint32_t chunks16 = cs * 8, total = m * chunks16, inv16 = 0xffffffffu / chunks16;
+            for (uint32_t i0 = tid; i0 < total; i0 += 256 * NB) {
+                u32x4 v[NB];
+                uint32_t off[NB];
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    const uint32_t i = i0 + 256 * j < total ? i0 + 256 * j : i0;  // past the end: a piece again, not stored
+                    const uint32_t row = udiv_inv(i, chunks16, inv16), c = i - row * chunks16;
+                    uint32_t gst = st_run0 + c0 + (c >> 3);
+                    if (gst >= spb) gst -= spb;
+                    if (gst >= spb) gst %= spb;
+                    v[j] = *(const u32x4*)(mb.xh + (size_t)row * k + gst * 64 + (c & 7) * 8);
+                    off[j] = row * xpitch + c * 16;
+                }
+#pragma unroll
+                for (int j = 0; j < NB; j++)
+                    if (i0 + 256 * j < total) *(u32x4*)(xs + off[j]) = v[j];
+            }
+        }
+        __syncthreads();
+        if (c0 == 0) { FE_STAMP_AT(1); }
+        // the chunk's load steps, segment by segment (a segment ends with its column block or with the chunk)
+        uint32_t i = 0;
+        while (i < cs) {
+            const uint32_t seg = cs - i < spb - st ? cs - i : spb - st;
+            // Whole groups of GROUP steps run as straight-line code: no branches inside, and the refill of a ring slot is
+            // unconditional, so each load lands straight in the slot its words were just decoded from and only that
+            // slot's next use waits for it. The wait at the top of a group has to cover every load in flight (the
+            // compiler cannot count across the back edge).
+            const uint32_t full = seg / GROUP * GROUP;
+            for (uint32_t s0 = 0; s0 < full; s0 += GROUP) {
+#pragma unroll
+                for (int j = 0; j < GROUP; j++) one(ring[j % DEPTH], i + s0 + j);
+            }
+            for (uint32_t s0 = full; s0 < seg; s0 += DEPTH) {  // the remainder, slot by slot
+#pragma unroll
+                for (int j = 0; j < DEPTH; j++)
+                    if (s0 + j < seg) one(ring[j], i + s0 + j);
+            }
+            ring_turn<BITS, DEPTH>(ring, seg % DEPTH);
+            i += seg, st += seg;
+            if (st == spb) {
+                flush(nb);
+                nb++, st = 0;
+                if (c0 + i < S) sv = *(const u32x2*)(mb.svh + nb * 128 + 4 * l32);  // the next block's output scales
+            }
+        }
+    }
+    if (st) flush(nb);
+    FE_STAMP_AT(7);
+#ifdef FE_STAMP
+    if (threadIdx.x == 0) stamps[(size_t)blockIdx.x * 16 + 10] = __builtin_amdgcn_s_memtime();
+#endif
+}
+
+#define GEMVB_KERNEL(BITS, RG)                                                                                        \
+    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemvb_b##BITS##_r##RG(                                   \
+        GemvJob job, const void* x, const void* x2, uint32_t x_mode, uint32_t ldx, uint32_t k, uint32_t m,             \
+        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb FE_STAMP_ARG) {                                             \
+        uint32_t i = 0;                                                                                               \
+        while (i + 1 < job.count && blockIdx.x >= job.first[i + 1]) i++;                                              \
+        gemvb_body<BITS, RG>(job.m[i], blockIdx.x - job.first[i], k, m, y_mode, chunk, inv_spb,                       \
+                             RotSrc{x, x2, x_mode, ldx} FE_STAMP_PASS);                                               \
+    }
+#define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
+GEMVB_FAMILY(2)
+GEMVB_FAMILY(3)
+GEMVB_FAMILY(4)
+GEMVB_FAMILY(5)
+GEMVB_FAMILY(6)
+GEMVB_FAMILY(8)
 
 // ---- decode GEMV, streamed over the whole tensor (1..16 rows) -------------------------------------------------------------
 //
@@ -768,7 +1190,7 @@ __device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh
             store_agent_f32x4(zp + 8, acc[1]);
         }
         acc[0] = acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wavefront's partial sums are acknowledged at agent scope
+        agent_stores_wait();  // this wavefront's partial sums are acknowledged at agent scope
         // the program's four wavefronts meet on an LDS counter; the last of them reports the segment to the block's
         // global arrival counter, and the last segment to arrive finishes the block
         uint32_t old = 0;

@@ -684,7 +684,7 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
             for (int h = 0; h < 2; h++) store_agent_f32x4(z + ((size_t)split * m + row) * n + col + 16 * h, sum[xr][h]);
         }
     }
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this lane's stores are acknowledged at agent scope
+    agent_stores_wait();  // this lane's stores are acknowledged at agent scope
     __syncthreads();
     if (tid == 0) {
         uint32_t old = __hip_atomic_fetch_add(&counters[nt], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

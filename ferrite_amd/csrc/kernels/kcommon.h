@@ -11,6 +11,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // dword-aligned forms: a lane's run of trellis words starts at any word
 typedef uint32_t u32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
@@ -138,21 +139,26 @@ __device__ __forceinline__ uint32_t silu_mul_bf16x2(uint32_t g, uint32_t u) {
     return pack_bf16x2(v[0], v[1]);
 }
 
-// 16 bytes at agent scope: partial sums that one program leaves for another, possibly on another XCD with its own L2.
-// The store goes through to memory, the load reads past this XCD's L2 (the sc1 forms that clang emits for 4-byte
-// agent-scope atomics; it has no 16-byte ones). The compiler does not count these loads: agent_loads_wait must come
-// between the last load and the first use of any loaded value.
+// Data that one program leaves for another, possibly on another XCD with its own L2, crosses at agent scope: stores go
+// through to memory (the sc1 form that clang emits for agent-scope atomic stores; it has no 16-byte ones), loads read past
+// this XCD's L2. agent_stores_wait() returns when the lane's stores are acknowledged. The loads are 8-byte relaxed
+// agent-scope atomic loads, which the compiler counts in its own s_waitcnt.
 __device__ __forceinline__ void store_agent_f32x4(float* p, f32x4 v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
 }
+__device__ __forceinline__ void agent_stores_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ f32x4 load_agent_f32x4(const float* p) {
-    f32x4 v;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(v) : "v"(p) : "memory");
-    return v;
+    const uint64_t a = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t b = __hip_atomic_load((const uint64_t*)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return (f32x4){__uint_as_float((uint32_t)a), __uint_as_float((uint32_t)(a >> 32)), __uint_as_float((uint32_t)b),
+                   __uint_as_float((uint32_t)(b >> 32))};
 }
+// The same 16-byte agent-scope load through a buffer resource (cache policy bit 4 = sc1): an ordinary load to the
+// compiler, which schedules many of them together and counts them in its waits. Byte offsets: voff per lane, soff uniform;
+// out of the resource's range the load returns zero.
+__device__ __forceinline__ f32x4 load_agent_f32x4(__amdgpu_buffer_rsrc_t rs, uint32_t voff, uint32_t soff) {
+    return __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 16));
+}
+// For code written around explicit waits: nothing to do, the compiler waits for the loads above itself.
 template <int N>
-__device__ __forceinline__ void agent_loads_wait(f32x4 (&t)[N]) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#pragma unroll
-    for (int i = 0; i < N; i++) asm volatile("" : "+v"(t[i]));
-}
+__device__ __forceinline__ void agent_loads_wait(f32x4 (&)[N]) {}

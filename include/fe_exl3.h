@@ -119,9 +119,9 @@ int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_
  * rotated inputs, split partial sums and arrival counters live in one static device array of FE_EXL3_STATIC_BYTES that
  * every GPU the library runs on holds until the process ends; the call allocates and frees nothing. Same kernels and
  * the same bits as fe_exl3_linear_forward. Limits: 1..FE_EXL3_STATIC_ROWS rows, rows * k * 2 <= 1 MiB of rotated inputs,
- * plan.sk * rows * n * 4 bytes of partial sums <= FE_EXL3_STATIC_BYTES - 1 MiB - 16 KiB, n <= 524288; anything larger is
+ * (programs + n / 128) * rows * 512 bytes of partial sums (programs: about 4 per CU) <= FE_EXL3_STATIC_BYTES - 1 MiB - 16 KiB, n <= 524288; anything larger is
  * FE_ERR_WORKSPACE. All calls on one GPU share the array: calls that overlap on one GPU (two streams) race; order them. */
-#define FE_EXL3_STATIC_BYTES (8u << 20)
+#define FE_EXL3_STATIC_BYTES (12u << 20)
 #define FE_EXL3_STATIC_ROWS 16
 int fe_exl3_linear_forward_static(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
                                   int x_dtype, fe_devptr_t y, int y_dtype, uint32_t rows);

@@ -122,7 +122,7 @@ def test_plans():
             p = Linear.plan_for(k, n, 4, blocks)
             steps = k // 64
             least = min(8, max(2, steps // 2))
-            assert steps % p.sk == 0 and steps // p.sk >= min(least, steps) and p.ver == 1
+            assert steps % p.sk == 0 and steps // p.sk >= min(least, steps) and p.ver in (1, 3)
             miss = lambda d: abs(math.log(n // 128 * d / blocks))
             fits = [d for d in range(1, steps + 1) if steps % d == 0 and steps // d >= least] or [1]
             assert miss(p.sk) <= min(miss(d) for d in fits) + 1e-12
