@@ -68,6 +68,7 @@ SYMBOLS = {
     # fe_exl3.h
     "fe_exl3_kernels_load": (I, [PP]),
     "fe_exl3_kernels_destroy": (I, [P]),
+    "fe_exl3_kernels_set_option": (I, [P, C.c_char_p, U32]),
     "fe_exl3_plan_for": (I, [U32, U32, U32, U32, C.POINTER(PlanC)]),
     "fe_exl3_plan_parse": (I, [C.c_char_p, C.POINTER(PlanC)]),
     "fe_exl3_linear_from_view": (I, [PP, P, C.c_char_p, C.POINTER(View), C.POINTER(PlanC)]),
@@ -94,6 +95,7 @@ SYMBOLS = {
     # fe_fp4.h
     "fe_fp4_kernels_load": (I, [PP]),
     "fe_fp4_kernels_destroy": (I, [P]),
+    "fe_fp4_kernels_set_option": (I, [P, C.c_char_p, C.c_int32]),
     "fe_fp4_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, P, F]),
     "fe_fp4_linear_from_view": (I, [PP, C.c_char_p, U32, U32, U64, U64, U64, F]),
     "fe_fp8_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, F]),
@@ -118,6 +120,7 @@ SYMBOLS = {
     # fe_bf16.h
     "fe_bf16_kernels_load": (I, [PP]),
     "fe_bf16_kernels_destroy": (I, [P]),
+    "fe_bf16_kernels_set_option": (I, [P, C.c_char_p, C.c_int32]),
     "fe_bf16_gemv": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
     "fe_bf16_gemm": (I, [P, P, U64, U32, U64, U32, U64, U64, U32, U32, U32]),
     "fe_bf16_interleave_gu": (I, [P, P, U64, U64, U64, U32, U32]),

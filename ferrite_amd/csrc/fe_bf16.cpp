@@ -6,6 +6,8 @@
 #include <cstdlib>
 
 #include "fe_exl3.h"  // error codes
+#include <string>
+
 #include "fe_internal.h"
 
 namespace {
@@ -21,6 +23,10 @@ struct fe_bf16_kernels {
     fe_function_t gemv[4][4] = {};  // [rows 1, 2, 4, 8][columns of a program 1, 2, 4, 8]
     uint32_t cus = 0;
     FeBuf part;
+    // Switches, read from the environment once at load (fe_bf16_kernels_set_option changes them afterwards)
+    int32_t nc = -1;           // columns a GEMV program takes (1, 2, 4, 8); -1 = by the shape (FE_BF16_NC)
+    int32_t raster_group = -1; // raster group of the GEMM; -1 = by the shape (FE_BF16_GROUP)
+    uint32_t gemm_splits = 8;  // most pieces a cut output tile takes (FE_GEMM_SPLITS; 1: never cut)
 };
 
 // log2 of the columns a GEMV program takes. Measured on 5120 x 17408, 17408 x 5120 and 5120 x 5120: 4 columns are best
@@ -73,6 +79,9 @@ int fe_bf16_kernels_load(fe_bf16_kernels **out) {
     int cus = 0;
     if (!c) c = fe_hip_cu_count(&cus);
     k->cus = (uint32_t)cus;
+    if (const char *e = getenv("FE_BF16_NC")) k->nc = atoi(e);
+    if (const char *e = getenv("FE_BF16_GROUP")) k->raster_group = atoi(e);
+    if (const char *e = getenv("FE_GEMM_SPLITS")) k->gemm_splits = (uint32_t)atoi(e);
     if (!c) c = k->part.alloc((size_t)kFeGemmSlotsPerCu * k->cus * kFeGemmPartBytes);
     if (c) {
         fe_bf16_kernels_destroy(k);
@@ -90,6 +99,16 @@ int fe_bf16_kernels_destroy(fe_bf16_kernels *k) {
     return 0;
 }
 
+int fe_bf16_kernels_set_option(fe_bf16_kernels *k, const char *name, int32_t value) {
+    if (!k || !name) return fe_set_error(FE_ERR_ARG, "fe_bf16_kernels_set_option", "null argument");
+    const std::string nm = name;
+    if (nm == "nc") k->nc = value;
+    else if (nm == "raster_group") k->raster_group = value;
+    else if (nm == "gemm_splits") k->gemm_splits = (uint32_t)value;
+    else return fe_set_error(FE_ERR_ARG, "fe_bf16_kernels_set_option", name);
+    return 0;
+}
+
 int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint32_t ldy, fe_devptr_t x, uint32_t lda,
                  fe_devptr_t w, fe_devptr_t res, uint32_t m, uint32_t n, uint32_t k) {
     const char *fn = "fe_bf16_gemv";
@@ -101,7 +120,7 @@ int fe_bf16_gemv(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint
     // columns of a program: the results do not depend on it. More columns read x less often (x is read once per program
     // and step, the weights once in all), fewer give more programs
     int cols = gemv_cols(n, form);
-    if (const char *e = getenv("FE_BF16_NC")) cols = atoi(e) >= 8 ? 3 : atoi(e) >= 4 ? 2 : atoi(e) >= 2 ? 1 : 0;
+    if (kern->nc > 0) cols = kern->nc >= 8 ? 3 : kern->nc >= 4 ? 2 : kern->nc >= 2 ? 1 : 0;
     void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy};
     return fe_hip_launch(kern->gemv[form][cols], n >> cols, 1, 1, 256, 1, 1, 0, s, args);
 }
@@ -116,9 +135,9 @@ int fe_bf16_gemm(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t y, uint
         return fe_set_error(FE_ERR_UNSUPPORTED, fn, "operand of 4 GB or more");
     const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
     uint32_t group = bf16_raster_group(m, n, k, tiles_m);
-    if (const char *e = getenv("FE_BF16_GROUP")) group = (uint32_t)atoi(e);
+    if (kern->raster_group >= 0) group = (uint32_t)kern->raster_group;
     if (group > tiles_m) group = tiles_m;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes), kern->gemm_splits);
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = kern->part.p;
     void *args[] = {&y, &x, &w, &res, &m, &n, &k, &lda, &ldy, &group, &full, &splits, &part};
@@ -150,9 +169,9 @@ int fe_bf16_gemm_swiglu(const fe_bf16_kernels *kern, fe_stream_t s, fe_devptr_t 
         return fe_set_error(FE_ERR_UNSUPPORTED, fn, "operand of 4 GB or more");
     const uint32_t tiles_m = (m + kTileM - 1) / kTileM, tiles_n = (n + kTileN - 1) / kTileN;
     uint32_t group = bf16_raster_group(m, n, k, tiles_m);
-    if (const char *e = getenv("FE_BF16_GROUP")) group = (uint32_t)atoi(e);
+    if (kern->raster_group >= 0) group = (uint32_t)kern->raster_group;
     if (group > tiles_m) group = tiles_m;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(kern->part.bytes / kFeGemmPartBytes), kern->gemm_splits);
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = kern->part.p;
     void *args[] = {&act, &x, &w, &m, &n, &k, &lda, &group, &full, &splits, &part};

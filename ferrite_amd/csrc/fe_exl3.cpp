@@ -10,19 +10,18 @@
 #include <string>
 #include <vector>
 
+#include "fe_exl3_plans.h"
 #include "fe_internal.h"
 
 namespace {
 
-constexpr uint32_t kMaxRowsPerPass = 64;    // 4 row groups of 16
-constexpr uint32_t kHatRows = 513;          // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
-constexpr uint32_t kStreamRows = 16;        // the streamed GEMV takes one row group
-constexpr uint32_t kGroupMax = 4;           // FE_EXL3_GROUP_MAX: linears of one grouped launch
-constexpr uint32_t kGroupRows = 64;         // rows of a grouped launch (one GEMV pass)
-constexpr uint32_t kLdsBudget = 60 * 1024;  // staged inputs of one GEMV program
-constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one program of the balanced GEMV
-constexpr uint32_t kRedPitch = 132;         // GEMV_RED_PITCH
+constexpr uint32_t kMaxRowsPerPass = 64;       // 4 row groups of 16
+constexpr uint32_t kHatRows = 513;             // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
+constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
+constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
+constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
+constexpr uint32_t kCuLds = 160 * 1024;        // LDS of a CU
 
 bool env_is(const char *name, const char *v) {
     const char *e = getenv(name);
@@ -39,28 +38,37 @@ int bits_slot(uint32_t bits) {
 
 }  // namespace
 
+// Switches of the launch paths. Read from the environment once, when the kernels are loaded; fe_exl3_kernels_set_option
+// changes them afterwards (tests compare both forms of a path in one process). No forward call reads the environment.
+struct fe_exl3_options {
+    uint32_t fused_rot = 1;        // the GEMV rotates its own input where that pays (FE_EXL3_NO_FUSED_ROT=1: never)
+    uint32_t fused_rot_pairs = 16; // ... up to this many (row, 128-channel block) pairs a program (FE_EXL3_FUSED_ROT_PAIRS)
+    uint32_t group = 1;            // linears of one input share a launch (FE_EXL3_NO_GROUP=1: one launch each)
+    uint32_t hat_rows = kHatRows;  // rows from which the prefill decodes once (FE_EXL3_HAT_ROWS; 0: never)
+    uint32_t lds_pad = 1;          // LDS request that pins the programs per CU to the plan's occ (FE_EXL3_NO_LDS_PAD=1: off)
+    uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
+    uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
+};
+
 struct fe_exl3_kernels {
     fe_module_t module = nullptr;
     fe_function_t recon_hat_f32 = nullptr, recon_hat_f16 = nullptr, had_rows = nullptr, had_cols_bf16 = nullptr;
     fe_function_t rot_in = nullptr, rot_in_group = nullptr, probe_v4 = nullptr;
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
-    fe_function_t gemv[6][4] = {};                                // [bits slot][row groups - 1]
-    fe_function_t gemv_stream[6] = {};                            // 1..16 rows, streamed over the whole tensor
-    fe_function_t gemv_group[6][4] = {};                          // several linears of one input, [bits slot][row groups - 1]
-    fe_function_t gemvb[6][4] = {};                               // balanced over the CUs (plan ver 3), 1..4 linears a launch
+    fe_function_t gemvb[6][4] = {};                               // the decode GEMV, [bits slot][row groups - 1]
     uint32_t cus = 0;
     fe_function_t gemm[6] = {};
     fe_function_t gemm_reduce = nullptr;
     fe_function_t hat_tiles[6] = {};  // trellis -> fp16 weights as the GEMM's LDS images
     fe_function_t gemm_hat = nullptr; // the GEMM over them
-    uint32_t group_m = 8;
+    fe_exl3_options opt;
 };
 
 struct fe_exl3_linear {
     std::string name;
     uint32_t k = 0, n = 0, bits = 0;
     fe_exl3_plan plan{};
-    uint32_t programs = 0;  // grid of the streamed GEMV (plan.ver == 2)
+    uint32_t programs = 0;  // grid of the decode GEMV under this plan
     fe_exl3_view view{};
     FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
     FeBuf hat;                // decoded fp16 tiles kept with the linear (fe_exl3_linear_keep_decoded), else empty
@@ -70,7 +78,7 @@ struct fe_exl3_linear {
 struct fe_exl3_workspace {
     uint32_t max_rows = 0, max_k = 0;
     FeBuf xh, z, counters, part;  // part: partial tiles of the prefill GEMM (rows > 64 only)
-    FeBuf hat;                    // decoded fp16 weights of one linear (workspaces of kHatRows rows or more)
+    FeBuf hat;                    // decoded fp16 weights of one linear (workspaces of hat_rows rows or more)
     size_t z_len = 0, counters_len = 0;
 };
 
@@ -90,6 +98,11 @@ static void view_strides(const fe_exl3_view &v, uint32_t *stride_k, uint32_t *st
         *stride_k = v.n / 16 * tw;
         *stride_nb = 8 * tw;
     }
+}
+
+static uint32_t env_u32(const char *name, uint32_t fallback) {
+    const char *e = getenv(name);
+    return e && *e ? (uint32_t)strtoul(e, nullptr, 0) : fallback;
 }
 
 extern "C" {
@@ -116,24 +129,9 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     for (int i = 0; i < 6; i++) {
         char nm[64];
         for (int rg = 1; rg <= 4; rg++) {
-            snprintf(nm, sizeof nm, "exl3_gemv_b%d_r%d", kBits[i], rg);
-            get(&k->gemv[i][rg - 1], nm);
-            if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv[i][rg - 1], 64 * 1024);
-        }
-        snprintf(nm, sizeof nm, "exl3_gemv_stream_b%d", kBits[i]);
-        get(&k->gemv_stream[i], nm);
-        for (int rg = 1; rg <= 4; rg++) {
             snprintf(nm, sizeof nm, "exl3_gemvb_b%d_r%d", kBits[i], rg);
             get(&k->gemvb[i][rg - 1], nm);
             if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemvb[i][rg - 1], 84 * 1024);
-        }
-        for (int rg = 1; rg <= 4; rg++) {
-            if (rg == 1)
-                snprintf(nm, sizeof nm, "exl3_gemv_group_b%d", kBits[i]);
-            else
-                snprintf(nm, sizeof nm, "exl3_gemv_group_b%d_r%d", kBits[i], rg);
-            get(&k->gemv_group[i][rg - 1], nm);
-            if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemv_group[i][rg - 1], 64 * 1024);
         }
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
@@ -144,7 +142,14 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     }
     get(&k->gemm_hat, "exl3_gemm_hat");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm_hat, kGemmLds);
-    if (const char *g = getenv("FE_EXL3_GROUP")) k->group_m = (uint32_t)atoi(g);
+    fe_exl3_options &o = k->opt;
+    o.fused_rot = env_u32("FE_EXL3_NO_FUSED_ROT", 0) ? 0 : 1;
+    o.fused_rot_pairs = env_u32("FE_EXL3_FUSED_ROT_PAIRS", o.fused_rot_pairs);
+    o.group = env_u32("FE_EXL3_NO_GROUP", 0) ? 0 : 1;
+    if (getenv("FE_EXL3_HAT_ROWS")) fe_exl3_kernels_set_option(k, "hat_rows", (uint32_t)std::max(0, atoi(getenv("FE_EXL3_HAT_ROWS"))));
+    o.lds_pad = env_u32("FE_EXL3_NO_LDS_PAD", 0) ? 0 : 1;
+    o.gemm_group_m = env_u32("FE_EXL3_GROUP", o.gemm_group_m);
+    o.gemm_splits = env_u32("FE_GEMM_SPLITS", o.gemm_splits);
     if (!c) {
         int cus = 0;
         c = fe_hip_cu_count(&cus);
@@ -165,35 +170,45 @@ int fe_exl3_kernels_destroy(fe_exl3_kernels *k) {
     return 0;
 }
 
-// K splits for `blocks` programs: the divisor of the load-step count whose program count comes closest to the target
-// while a program keeps at least min_steps load steps (the role of tf_plan, crates/fe-exl3/src/linear.rs:100-129; one
-// load step = 4 k steps = 64 input channels). Programs of fewer than 8 steps cost more in start-up, partial sums and
-// hand-off than their spread over the CUs gains: 5120 x 5120 at 1 row takes 11.9 us cut 10 ways and 13.3 us cut 16
-// ways, 5120 x 1024 9.5 us cut 10 ways and 13.8 us cut 40 ways.
+int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t value) {
+    if (!k || !name) return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", "null argument");
+    fe_exl3_options &o = k->opt;
+    const std::string nm = name;
+    if (nm == "fused_rot") o.fused_rot = value;
+    else if (nm == "fused_rot_pairs") o.fused_rot_pairs = value;
+    else if (nm == "group") o.group = value;
+    else if (nm == "hat_rows") o.hat_rows = value == 0 ? 0xffffffffu : std::max(value, kMaxRowsPerPass + 1);
+    else if (nm == "lds_pad") o.lds_pad = value;
+    else if (nm == "gemm_group_m") o.gemm_group_m = value;
+    else if (nm == "gemm_splits") o.gemm_splits = value;
+    else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
+    return 0;
+}
+
+// Launch plan for one shape. The decode GEMV deals 128-channel x 128-column units to `programs` programs in equal runs;
+// what is chosen is how many programs: occ per CU (ver 3), each at least wk units long. The tuned table holds the measured
+// choice for the shapes it knows on this CU count (FE_EXL3_UNTUNED=1 skips it: plans::tuned and its override,
+// crates/fe-exl3/src/plans.rs:123-131, linear.rs:217-233); other shapes take the rule: the program target `blocks`
+// (default 4 per CU, linear.rs:131-134) rounded to whole programs per CU, runs of at least 4 units, because programs of
+// fewer than 8 load steps cost more in start-up and hand-off than their spread over the CUs gains. sk records the K splits
+// per column block that this amounts to. FE_EXL3_NOSPLIT=1 / FE_EXL3_SPLIT=0: one program per column block (ver 1, sk 1).
 int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_exl3_plan *out) {
-    (void)bits;
     if (!out || !k || !n || k % 128 || n % 128) return fe_set_error(FE_ERR_SHAPE, "fe_exl3_plan_for", "k, n must be multiples of 128");
-    const uint32_t steps = k / 64, nb = n / 128, min_steps = std::min(8u, std::max(2u, steps / 2));
-    // the divisor of the step count whose program count nb * d comes closest (as a ratio) to `blocks`
-    uint32_t sk = 1;
-    double best = 1e30;
-    for (uint32_t d = 1; d <= steps; d++) {
-        if (steps % d) continue;
-        if (steps / d < min_steps) break;
-        double ratio = (double)nb * d / (blocks ? blocks : 1);
-        double miss = ratio < 1.0 ? 1.0 / ratio : ratio;
-        if (miss < best) best = miss, sk = d;
+    if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) {
+        *out = fe_exl3_plan{1, 4, 1, 0};
+        return 0;
     }
-    if (env_is("FE_EXL3_NOSPLIT", "1") || env_is("FE_EXL3_SPLIT", "0")) sk = 1;
-    // ver 3 (the default): the GEMV balanced over the CUs, occ programs per CU, for 1..64 rows, one summation order for all
-    // of them. ver 1 (FE_EXL3_VER=1): the split-K GEMV, sk splits. ver 2 (FE_EXL3_STREAM=1): rows 1..16 run the streamed
-    // GEMV with occ programs per CU.
-    uint32_t ver = env_is("FE_EXL3_STREAM", "1") ? 2 : 3, occ = 0;
-    if (const char *v = getenv("FE_EXL3_VER")) ver = (uint32_t)atoi(v);
-    if (ver == 2) occ = 2;
-    if (ver == 3) occ = 4;
-    if (const char *o = getenv("FE_EXL3_OCC")) occ = (uint32_t)atoi(o);
-    *out = fe_exl3_plan{sk, 4, ver, ver == 1 ? 0 : occ};
+    int cus = 0;
+    if (fe_hip_cu_count(&cus) || cus <= 0) cus = 256;  // planning without a device: the MI355X count
+    uint32_t occ = blocks ? std::min(5u, std::max(1u, (blocks + (uint32_t)cus / 2) / (uint32_t)cus)) : 4, wk = 4;
+    if (!env_is("FE_EXL3_UNTUNED", "1")) {
+        for (const FeTunedPlan &t : kFeTunedPlans)
+            if (t.k == k && t.n == n && t.bits == bits && t.cus == (uint32_t)cus) occ = t.occ, wk = t.min_units;
+    }
+    occ = env_u32("FE_EXL3_OCC", occ), wk = std::max(1u, env_u32("FE_EXL3_MIN_UNITS", wk));  // tuning runs
+    const uint32_t units = (k / 128) * (n / 128), nb = n / 128;
+    const uint32_t programs = std::max(1u, std::min(occ * (uint32_t)cus, units / wk));
+    *out = fe_exl3_plan{(programs + nb - 1) / nb, wk, 3, occ};
     return 0;
 }
 
@@ -206,20 +221,21 @@ int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out) {
     return 0;
 }
 
-// Programs of the streamed GEMV: occ per CU, at most one per eight work units (FE_EXL3_PROGRAMS overrides the count).
-static uint32_t stream_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p, uint32_t k, uint32_t n) {
-    if (p.ver == 3) {
-        // balanced GEMV: occ programs per CU, each a run of at least min_units 128-channel blocks of one column block
-        const uint32_t units = (k / 128) * (n / 128), occ = p.occ ? p.occ : 4;
-        uint32_t min_units = 4;
-        if (const char *e = getenv("FE_EXL3_MIN_UNITS")) min_units = std::max(1, atoi(e));  // tuning
-        return std::max(1u, std::min(occ * std::max(kern->cus, 1u), units / min_units));
-    }
-    if (p.ver != 2) return 0;
-    const uint32_t units = (k / 64) * (n / 128), occ = p.occ ? p.occ : 2;
-    uint32_t progs = std::min(occ * kern->cus, units / 8);
-    if (const char *e = getenv("FE_EXL3_PROGRAMS")) progs = std::min((uint32_t)atoi(e), units);  // tuning and tests
-    return std::max(1u, progs);
+}  // extern "C"
+
+// Programs of the decode GEMV under a plan. ver 1 (the reference's meaning of a plan): sk programs per column block.
+// ver 2 and 3: occ programs per CU, each a run of at least wk units. ver 4: sk programs in all (tests and tuners: any
+// partition). Never more programs than units.
+static uint32_t plan_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p, uint32_t k, uint32_t n) {
+    const uint32_t units = (k / 128) * (n / 128);
+    uint32_t progs;
+    if (p.ver <= 1)
+        progs = n / 128 * std::max(p.sk, 1u);
+    else if (p.ver == 4)
+        progs = std::max(p.sk, 1u);
+    else
+        progs = (p.occ ? p.occ : 4) * std::max(kern->cus, 1u), progs = std::min(progs, units / std::max(p.wk, 1u));
+    return std::max(1u, std::min(progs, units));
 }
 
 static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, const fe_exl3_plan &p) {
@@ -229,12 +245,14 @@ static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, co
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear", msg);
     }
     // linear.rs:244: k, n multiples of 128 and the K range divides into the plan's pieces (here: load steps of 64)
-    if (!k || !n || k % 128 || n % 128 || p.sk == 0 || (k / 64) % p.sk) {
+    if (!k || !n || k % 128 || n % 128 || p.sk == 0 || (p.ver <= 1 && (k / 64) % p.sk)) {
         snprintf(msg, sizeof msg, "%s: %ux%u does not fit plan sk %u", name, k, n, p.sk);
         return fe_set_error(FE_ERR_SHAPE, "fe_exl3_linear", msg);
     }
     return 0;
 }
+
+extern "C" {
 
 int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, const char *name, const fe_exl3_view *view,
                              const fe_exl3_plan *plan) {
@@ -246,7 +264,7 @@ int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, 
     l->plan = *plan;
     l->view = *view;
     l->kern = kern;
-    l->programs = stream_programs(kern, *plan, view->k, view->n);
+    l->programs = plan_programs(kern, *plan, view->k, view->n);
     *out = l;
     return 0;
 }
@@ -264,7 +282,7 @@ int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, con
     auto *l = new fe_exl3_linear;
     l->name = name ? name : "";
     l->k = k, l->n = n, l->bits = bits, l->plan = p, l->kern = kern;
-    l->programs = stream_programs(kern, p, k, n);
+    l->programs = plan_programs(kern, p, k, n);
     const size_t tw = 8 * (size_t)bits, kt = k / 16, nt = n / 16, words = kt * nt * tw;
     int c = 0;
     if (strips) {
@@ -302,32 +320,30 @@ int fe_exl3_linear_view(const fe_exl3_linear *l, fe_exl3_view *view, fe_exl3_pla
 
 size_t fe_exl3_linear_weight_bytes(const fe_exl3_linear *l) { return l ? (size_t)l->k * l->n * l->bits / 8 : 0; }
 
+}  // extern "C"
+
 // Many rows: decoding the trellis once into fp16 tiles and running the GEMM over them beats decoding inside the GEMM,
-// where each 256-row tile of the output decodes its weights again. From kHatRows rows on (FE_EXL3_HAT_ROWS overrides; 0
-// turns the form off) and only with a workspace created for that many rows, which then holds the largest linear's
-// decoded weights (2 bytes a weight).
-static uint32_t hat_rows() {
-    const char *e = getenv("FE_EXL3_HAT_ROWS");  // read per call: tests compare both forms in one process
-    if (!e) return kHatRows;
-    int v = atoi(e);
-    return v <= 0 ? 0xffffffffu : std::max<uint32_t>((uint32_t)v, kMaxRowsPerPass + 1);
-}
+// where each 256-row tile of the output decodes its weights again. From opt.hat_rows rows on and only with a workspace
+// created for that many rows, which then holds the largest linear's decoded weights (2 bytes a weight).
 static size_t hat_bytes(const fe_exl3_linear *l) { return (size_t)((l->n / 128 + 1) / 2) * 256 * l->k * 2; }
+
+// Room one linear's GEMV takes in a workspace at `rows` rows: a slot of 128 sums per (program, column block it touches).
+static size_t job_z(const fe_exl3_linear *l, uint32_t rows) { return (size_t)(l->programs + l->n / 128) * 128 * rows; }
+
+extern "C" {
 
 int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *linears, size_t count, uint32_t max_rows) {
     if (!out || (count && !linears) || !max_rows) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_create", "bad argument");
-    size_t max_k = 128, max_z = 0, max_zs = 0, max_nb = 1, max_hat = 0;
-    std::vector<size_t> zs, nbs;  // per linear, for the grouped launch: room for the kGroupMax largest together
+    size_t max_k = 128, max_hat = 0;
+    uint32_t hat_rows = kHatRows;
+    std::vector<size_t> zs, nbs;  // per linear; a launch of several linears needs room for the kGroupMax largest together
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
-        zs.push_back(l->plan.ver == 3 ? (size_t)(l->programs + l->n / 128) * 128 : l->plan.ver == 2 ? 0 : (size_t)l->plan.sk * l->n);
+        zs.push_back(job_z(l, 1));
         nbs.push_back(l->n / 128);
         max_hat = std::max(max_hat, hat_bytes(l));
         max_k = std::max<size_t>(max_k, l->k);
-        if (l->plan.ver != 3 && l->plan.sk > 1) max_z = std::max<size_t>(max_z, (size_t)l->plan.sk * l->n);
-        if (l->plan.ver == 3) max_z = std::max<size_t>(max_z, (size_t)(l->programs + l->n / 128) * 128);
-        if (l->plan.ver == 2) max_zs = std::max<size_t>(max_zs, (size_t)(l->programs + l->n / 128) * 128);
-        max_nb = std::max<size_t>(max_nb, l->n / 128);
+        hat_rows = l->kern->opt.hat_rows;
     }
     auto *ws = new fe_exl3_workspace;
     ws->max_rows = max_rows, ws->max_k = (uint32_t)max_k;
@@ -337,19 +353,18 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
         for (size_t i = 0; i < v.size() && i < kGroupMax; i++) t += v[i];
         return t;
     };
-    const size_t group_z = top(zs), group_nb = top(nbs);
-    ws->z_len = std::max<size_t>(std::max(max_z * std::min(max_rows, kMaxRowsPerPass), max_zs * std::min(max_rows, kStreamRows)), 4);
-    ws->z_len = std::max(ws->z_len, group_z * std::min(max_rows, kGroupRows));
-    ws->counters_len = std::max((size_t)((max_rows + 7) / 8) * max_nb, group_nb);
-    // (rotated inputs: one linear's at max_rows, or a group's at up to kGroupRows rows each)
-    int c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * std::min(max_rows, kGroupRows)) * max_k * 2);
+    const uint32_t gemv_rows = std::min(max_rows, kMaxRowsPerPass);
+    ws->z_len = std::max<size_t>(top(zs) * gemv_rows, 4);
+    ws->counters_len = std::max<size_t>(top(nbs), 1);
+    // (rotated inputs: one linear's at max_rows, or those of the linears of one launch at up to 64 rows each)
+    int c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * gemv_rows) * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
     int cus = 0;
     if (!c && max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
     if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes);
     // zeroed once: the unused half of the last tile of an odd count of column blocks is read (and its sums discarded)
-    if (!c && max_rows >= hat_rows() && max_hat) c = ws->hat.zeroed(max_hat);
+    if (!c && max_rows >= hat_rows && max_hat) c = ws->hat.zeroed(max_hat);
     if (c) {
         delete ws;
         return c;
@@ -371,6 +386,8 @@ int fe_exl3_workspace_xh(const fe_exl3_workspace *ws, fe_devptr_t *xh, uint32_t 
     return 0;
 }
 
+}  // extern "C"
+
 // The input of a rotation: bf16 (mode 0) or f32 (mode 1) rows of stride ld, or (mode 2) SwiGLU of two bf16 arrays,
 // x = gate and x2 = up, taken on the way in (RotSrc of k_exl3.hip).
 struct RotInput {
@@ -391,16 +408,6 @@ static int launch_rot(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_s
     return fe_hip_launch(kern->rot_in, (k + 511) / 512, rows, 1, 128, 1, 1, 0, s, args);
 }
 
-int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
-                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
-    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "null argument");
-    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
-        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "x is bf16 or f32");
-    RotInput in;
-    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
-    return launch_rot(l, kern, s, in, rows, ws, "fe_exl3_linear_rotate_input");
-}
-
 // trellis -> fp16 tiles (exl3_hat_tiles_b*) into `hat`, hat_bytes(l) bytes
 static int launch_decode(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t hat) {
     const fe_exl3_kernels *kern = l->kern;
@@ -416,17 +423,18 @@ static int launch_decode(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t hat
 static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
                        const fe_exl3_workspace *ws) {
     const fe_exl3_kernels *kern = l->kern;
-    uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb, group = kern->group_m;
+    uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb, group = kern->opt.gemm_group_m;
     view_strides(l->view, &stride_k, &stride_nb);
     if ((uint64_t)rows * k * 2 >= (1ull << 32))
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear_gemv_rotated", "rotated input of 4 GB or more");
     const uint32_t tiles_m = (rows + 255) / 256, tiles_n = (n / 128 + 1) / 2;
     if (group == 0 || group > tiles_m) group = tiles_m;
-    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes),
+                                  kern->opt.gemm_splits);
     uint32_t full = g.full, splits = g.splits;
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
     const bool kept = l->hat.bytes != 0;  // decoded once and kept: any row count above the GEMV's runs over it
-    if (kept || (rows >= hat_rows() && ws->hat.bytes >= hat_bytes(l))) {
+    if (kept || (rows >= kern->opt.hat_rows && ws->hat.bytes >= hat_bytes(l))) {
         fe_devptr_t hat = kept ? l->hat.p : ws->hat.p;
         if (!kept) FE_TRY(launch_decode(l, s, hat));
         group = 0;  // the raster that deals column tiles to the XCDs: each decoded weight panel goes through one L2
@@ -441,37 +449,14 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
     return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
-// Decode-sized rows. With in.x != 0 the split-K kernel rotates that input itself and leaves the rotated rows in xh
-// (callers check fused_rotation_fits first); otherwise it reads xh.
-static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
-                       const fe_exl3_workspace *ws, const RotInput &in);
-static uint32_t gemv_chunk(uint32_t rows, uint32_t steps);
-
-// The split-K kernel can rotate its own input when every program's K range is whole 128-element blocks.
+// The GEMV can rotate its own input: every program rotates the channels of its own run, (row, 128-channel block) pairs,
+// 8 at a time, so every column block repeats the rotation of its K range. Measured on 5120 x 17408: one launch wins up
+// to a few rows, the separate rotation launch from about 8 rows on.
 static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
-    const char *e = getenv("FE_EXL3_NO_FUSED_ROT");  // read per call: tests compare both paths in one process
-    const bool off = e && atoi(e) != 0;
-    const fe_exl3_plan &p = l->plan;
-    if (p.ver == 3) {
-        // every program rotates the channels of its own run: (row, 128-channel block) pairs, 8 at a time
-        if (off || rows < 1 || rows > kMaxRowsPerPass) return false;
-        uint32_t pairs = 16;
-        if (const char *t = getenv("FE_EXL3_FUSED_ROT_PAIRS")) pairs = (uint32_t)atoi(t);
-        const uint32_t units = (l->k / 128) * (l->n / 128);
-        return rows * ((units + l->programs - 1) / l->programs) <= pairs;
-    }
-    if (off || rows < 1 || rows > kMaxRowsPerPass || p.ver == 2 || (l->k / 64 / p.sk) % 2) return false;
-    // every column block repeats the rotation of its K range: (row, 128-block) pairs a program, 8 at a time. Measured on
-    // 5120 x 17408 (8 blocks a program): one launch wins up to 4 rows (19.9 against 22.3 us at 1 row), the separate
-    // rotation from 8 rows on (25.2 against 23.7 us).
-    uint32_t pairs = 32;
-    if (const char *t = getenv("FE_EXL3_FUSED_ROT_PAIRS")) pairs = (uint32_t)atoi(t);
-    return rows * (l->k / 128 / p.sk) <= pairs;
-}
-
-int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
-                                uint32_t rows, const fe_exl3_workspace *ws) {
-    return launch_rows(l, s, xh, y, y_dtype, rows, ws, RotInput{});
+    const fe_exl3_options &o = l->kern->opt;
+    if (!o.fused_rot || rows < 1 || rows > kMaxRowsPerPass) return false;
+    const uint32_t units = (l->k / 128) * (l->n / 128);
+    return rows * ((units + l->programs - 1) / l->programs) <= o.fused_rot_pairs;
 }
 
 // mirrors GemvJob of k_exl3.hip
@@ -483,11 +468,11 @@ struct GemvJobArgs {
     } m[kGroupMax];
 };
 static_assert(sizeof(GemvJobArgs) == 24 + kGroupMax * 88, "GemvJob layout");
+struct RotGroupArgs {  // RotGroup
+    fe_devptr_t suh[kGroupMax], xh[kGroupMax];
+};
 
-// Room a balanced launch takes in the workspace: partial sums (floats) and counters of one member at `rows` rows.
-static size_t job_z(const fe_exl3_linear *l, uint32_t rows) { return (size_t)(l->programs + l->n / 128) * 128 * rows; }
-
-// The balanced GEMV (plan ver 3) for 1..4 linears of one input in one launch: member i reads its rotated input at xhs[i]
+// The decode GEMV for 1..4 linears of one input in one launch, 1..64 rows: member i reads its rotated input at xhs[i]
 // (in.x == 0) or rotates in.x itself and leaves the result at xhs[i]. The caller has checked rows, k and bits.
 static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t s, const fe_devptr_t *xhs, const fe_devptr_t *ys,
                       int y_dtype, uint32_t rows, const fe_exl3_workspace *ws, const RotInput &in, const char *fn) {
@@ -525,86 +510,29 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     // Exactly occ programs a CU: the dispatcher fills a CU as far as registers and LDS allow (5 programs) before it moves
     // on, which would leave CUs empty while others hold 5; an LDS request that fits occ times into the CU's 160 KB, and
     // not occ + 1 times, makes the CUs take occ each.
-    if (const uint32_t occ = ls[0]->plan.occ; occ && !env_is("FE_EXL3_NO_LDS_PAD", "1")) lds = std::max(lds, 163840u / (occ + 1) + 512);
-    uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld;
+    const fe_exl3_kernels *kern = ls[0]->kern;
+    if (const uint32_t occ = ls[0]->plan.occ; occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
+    uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld, inv_spb = 0xffffffffu / (k / 64);
     fe_devptr_t x = in.x, x2 = in.x2;
-    // (the last argument exists only in timeline-probe builds of the code object; the shipped kernels take ten)
-    static const fe_devptr_t stamps = getenv("FE_EXL3_STAMPS") ? (fe_devptr_t)strtoull(getenv("FE_EXL3_STAMPS"), nullptr, 0) : 0;
-    fe_devptr_t st = stamps;
-    uint32_t inv_spb = 0xffffffffu / (k / 64);
-    void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb, &st};
-    return fe_hip_launch(ls[0]->kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
+    void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb};
+    return fe_hip_launch(kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 
+// Decode-sized rows run the GEMV (with in.x != 0 it rotates that input itself and leaves the rotated rows in xh; callers
+// check fused_rotation_fits first), more rows the GEMM.
 static int launch_rows(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype, uint32_t rows,
                        const fe_exl3_workspace *ws, const RotInput &in) {
-    if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "null argument");
-    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_gemv_rotated", "bad y dtype");
-    const fe_exl3_plan &p = l->plan;
-    char msg[200];
-    if (rows > kMaxRowsPerPass) {
-        if (rows > ws->max_rows) {
-            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
-            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
-        }
-        return launch_gemm(l, s, xh, y, y_dtype, rows, ws);
+    const char *fn = "fe_exl3_linear_gemv_rotated";
+    if (!l || !ws || !xh || !y) return fe_set_error(FE_ERR_ARG, fn, "null argument");
+    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, fn, "bad y dtype");
+    if (rows == 0 || rows > ws->max_rows) {  // linear.rs:302-307
+        char msg[200];
+        snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
+        return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
     }
-    if (p.ver == 3) {
-        if (rows == 0 || rows > ws->max_rows) {
-            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u)", l->name.c_str(), rows, ws->max_rows);
-            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
-        }
-        return launch_job(&l, 1, s, &xh, &y, y_dtype, rows, ws, in, "fe_exl3_linear_gemv_rotated");
-    }
-    if (p.ver == 2 && rows >= 1 && rows <= kStreamRows) {
-        if (rows > ws->max_rows || ws->z_len < (size_t)(l->programs + l->n / 128) * 128 * rows || ws->counters_len < l->n / 128) {
-            snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u, z %zu)", l->name.c_str(), rows, ws->max_rows,
-                     ws->z_len);
-            return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
-        }
-        uint32_t n = l->n, k = l->k, mode = (uint32_t)y_dtype, stride_k, stride_nb;
-        view_strides(l->view, &stride_k, &stride_nb);
-        fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
-        void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &mode, &stride_k, &stride_nb};
-        return fe_hip_launch(l->kern->gemv_stream[bits_slot(l->bits)], l->programs, 1, 1, 256, 1, 1, 0, s, args);
-    }
-    // linear.rs:302-307
-    if (rows == 0 || rows > ws->max_rows || (p.sk > 1 && ws->z_len < (size_t)p.sk * rows * l->n)) {
-        snprintf(msg, sizeof msg, "%s: rows %u do not fit the workspace (max %u, z %zu)", l->name.c_str(), rows, ws->max_rows,
-                 ws->z_len);
-        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
-    }
-    if (ws->counters_len < (size_t)((rows + 7) / 8) * (l->n / 128)) {
-        snprintf(msg, sizeof msg, "%s: workspace counters too small for %u rows", l->name.c_str(), rows);
-        return fe_set_error(FE_ERR_WORKSPACE, "fe_exl3_linear_gemv_rotated", msg);
-    }
-    const uint32_t rg = (rows + 15) / 16;
-    const uint32_t steps = l->k / 64 / p.sk;
-    uint32_t chunk = gemv_chunk(rows, steps);
-    const uint32_t lds = std::max(rows * (chunk * 128 + 16), rows * kRedPitch * 4);
-    uint32_t n = l->n, k = l->k, sk = p.sk, mode = (uint32_t)y_dtype, stride_k, stride_nb;
-    view_strides(l->view, &stride_k, &stride_nb);
-    fe_devptr_t tr = l->view.trellis, svh = l->view.svh, z = ws->z.p, cnt = ws->counters.p;
-    fe_devptr_t suh = l->view.suh, x = in.x, x2 = in.x2;
-    uint32_t x_mode = in.mode, ldx = in.ld;
-    void *args[] = {&xh, &tr, &svh, &y, &z, &cnt, &n, &k, &rows, &sk, &mode, &stride_k, &stride_nb, &chunk, &x, &x_mode, &suh, &xh, &x2, &ldx};
-    return fe_hip_launch(l->kern->gemv[bits_slot(l->bits)][rg - 1], n / 128 * sk, 1, 1, 256, 1, 1, lds, s, args);
+    if (rows > kMaxRowsPerPass) return launch_gemm(l, s, xh, y, y_dtype, rows, ws);
+    return launch_job(&l, 1, s, &xh, &y, y_dtype, rows, ws, in, fn);
 }
-
-int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on) {
-    if (!l) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_keep_decoded", "null linear");
-    if (!on) {
-        l->hat.release();
-        return 0;
-    }
-    if (l->hat.bytes) return 0;
-    FE_TRY(l->hat.zeroed(hat_bytes(l)));  // zeroed: the unused half of the last tile of an odd count of column blocks is read
-    int c = launch_decode(l, s, l->hat.p);
-    if (c) l->hat.release();
-    return c;
-}
-
-int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }
 
 // forward() on a described input: one launch where the GEMV rotates its own input, else the rotation and the linear.
 static int forward_from(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, const RotInput &in, fe_devptr_t y,
@@ -618,20 +546,8 @@ static int forward_from(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe
         return launch_rows(l, s, ws->xh.p, y, y_dtype, rows, ws, in);
     }
     FE_TRY(launch_rot(l, kern, s, in, rows, ws, fn));
-    return fe_exl3_linear_gemv_rotated(l, s, ws->xh.p, y, y_dtype, rows, ws);
+    return launch_rows(l, s, ws->xh.p, y, y_dtype, rows, ws, RotInput{});
 }
-
-int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
-                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
-    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "null argument");
-    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
-        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "x is bf16 or f32");
-    RotInput in;
-    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
-    return forward_from(l, kern, s, in, y, y_dtype, rows, ws, "fe_exl3_linear_forward");
-}
-
-}  // extern "C"
 
 int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
                          fe_devptr_t y, int y_dtype, uint32_t rows, uint32_t max_rows, fe_devptr_t counters,
@@ -644,10 +560,7 @@ int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, f
         snprintf(msg, sizeof msg, "%s: %u rows (this entry point takes 1..%u)", l->name.c_str(), rows, max_rows);
         return fe_set_error(FE_ERR_WORKSPACE, fn, msg);
     }
-    const size_t need_xh = (size_t)rows * l->k * 2, need_cnt = (size_t)((rows + 7) / 8) * (l->n / 128) * 4;
-    const size_t need_z = l->plan.ver == 3 ? job_z(l, rows) * 4
-                          : l->plan.ver == 2 ? (size_t)(l->programs + l->n / 128) * 128 * rows * 4
-                                           : (l->plan.sk > 1 ? (size_t)l->plan.sk * rows * l->n * 4 : 0);
+    const size_t need_xh = (size_t)rows * l->k * 2, need_cnt = (size_t)(l->n / 128) * 4, need_z = job_z(l, rows) * 4;
     if (need_xh > xh_bytes || need_cnt > counters_bytes || need_z > z_bytes) {
         snprintf(msg, sizeof msg, "%s: %u rows of %ux%u need %zu B of rotated inputs (limit %zu), %zu B of partial sums (limit %zu), "
                  "%zu B of counters (limit %zu)", l->name.c_str(), rows, l->k, l->n, need_xh, xh_bytes, need_z, z_bytes, need_cnt,
@@ -665,6 +578,46 @@ int fe_exl3_forward_over(const fe_exl3_linear *l, const fe_exl3_kernels *kern, f
 
 extern "C" {
 
+int fe_exl3_linear_rotate_input(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
+                                int x_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "null argument");
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_rotate_input", "x is bf16 or f32");
+    RotInput in;
+    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
+    return launch_rot(l, kern, s, in, rows, ws, "fe_exl3_linear_rotate_input");
+}
+
+int fe_exl3_linear_gemv_rotated(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, fe_devptr_t y, int y_dtype,
+                                uint32_t rows, const fe_exl3_workspace *ws) {
+    return launch_rows(l, s, xh, y, y_dtype, rows, ws, RotInput{});
+}
+
+int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on) {
+    if (!l) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_keep_decoded", "null linear");
+    if (!on) {
+        l->hat.release();
+        return 0;
+    }
+    if (l->hat.bytes) return 0;
+    FE_TRY(l->hat.zeroed(hat_bytes(l)));  // zeroed: the unused half of the last tile of an odd count of column blocks is read
+    int c = launch_decode(l, s, l->hat.p);
+    if (c) l->hat.release();
+    return c;
+}
+
+int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }
+
+int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,
+                           fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    if (!l || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "null argument");
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
+        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward", "x is bf16 or f32");
+    RotInput in;
+    in.x = x, in.mode = (uint32_t)x_dtype & 1, in.ld = l->k;
+    return forward_from(l, kern, s, in, y, y_dtype, rows, ws, "fe_exl3_linear_forward");
+}
+
 int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t gate,
                                   fe_devptr_t up, uint32_t ld, fe_devptr_t y, int y_dtype, uint32_t rows,
                                   const fe_exl3_workspace *ws) {
@@ -676,46 +629,28 @@ int fe_exl3_linear_forward_swiglu(const fe_exl3_linear *l, const fe_exl3_kernels
     return forward_from(l, kern, s, in, y, y_dtype, rows, ws, fn);
 }
 
-// mirrors GemvGroup of k_exl3.hip
-struct GemvGroupArgs {
-    uint32_t count, first[kGroupMax + 1];
-    struct Member {
-        fe_devptr_t trellis, svh, suh, xh, y, z, counters;
-        uint32_t n, sk, stride_k, stride_nb, chunk, pad;
-    } m[kGroupMax];
-};
-struct RotGroupArgs {  // RotGroup
-    fe_devptr_t suh[kGroupMax], xh[kGroupMax];
-};
+}  // extern "C"
 
-static uint32_t gemv_chunk(uint32_t rows, uint32_t steps) {
-    // staged input chunk: as many load steps as the LDS budget holds for `rows` rows, a multiple of 4
-    uint32_t chunk = (kLdsBudget / rows - 16) / 128 / 4 * 4;
-    chunk = std::max(chunk, 4u);
-    return std::min(chunk, (steps + 3) / 4 * 4);
-}
-
-// The grouped launch: the same input, width and kernel, and room in the workspace for every member's partials (and,
-// where the members do not rotate their own input, rotated inputs) side by side. *fused: the GEMV rotates its own input.
+// One launch for several linears: the same input, width and kernel, and room in the workspace for every member's partial
+// sums (and rotated inputs) side by side. *fused: the GEMV rotates its own input.
 static bool group_fits(const fe_exl3_linear *const *ls, size_t count, uint32_t rows, const fe_exl3_workspace *ws, bool *fused) {
-    const char *e = getenv("FE_EXL3_NO_GROUP");  // read per call: tests compare both paths in one process
-    if (e && atoi(e) != 0) return false;
-    if (!ls || !ws || count < 2 || count > kGroupMax || rows < 1 || rows > kGroupRows || rows > ws->max_rows) return false;
+    if (!ls || !ws || count < 2 || count > kGroupMax || rows < 1 || rows > kMaxRowsPerPass || rows > ws->max_rows) return false;
+    if (!ls[0] || !ls[0]->kern->opt.group) return false;
     size_t z = 0, nb = 0;
     bool f = true;
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = ls[i];
-        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.ver == 2 ||
-            l->plan.ver != ls[0]->plan.ver)
-            return false;
+        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.occ != ls[0]->plan.occ) return false;
         f = f && fused_rotation_fits(l, rows);
-        z += l->plan.ver == 3 ? job_z(l, rows) : (size_t)l->plan.sk * rows * l->n;
+        z += job_z(l, rows);
         nb += l->n / 128;
     }
-    if (!f && count * (size_t)rows * ls[0]->k * 2 > ws->xh.bytes) return false;
+    if (count * (size_t)rows * ls[0]->k * 2 > ws->xh.bytes) return false;
     if (fused) *fused = f;
     return z <= ws->z_len && nb <= ws->counters_len && ls[0]->k <= ws->max_k;
 }
+
+extern "C" {
 
 int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_t count, uint32_t rows,
                                           const fe_exl3_workspace *ws) {
@@ -727,63 +662,31 @@ int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_
 int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, const fe_exl3_kernels *kern, fe_stream_t s,
                                  fe_devptr_t x, int x_dtype, const fe_devptr_t *ys, int y_dtype, uint32_t rows,
                                  const fe_exl3_workspace *ws) {
-    if (!ls || !ys || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null argument");
+    const char *fn = "fe_exl3_linear_forward_group";
+    if (!ls || !ys || !kern || !ws || !x) return fe_set_error(FE_ERR_ARG, fn, "null argument");
     bool fused = false;
     if (!group_fits(ls, count, rows, ws, &fused)) {  // member by member: the same bits, more launches
         for (size_t i = 0; i < count; i++) FE_TRY(fe_exl3_linear_forward(ls[i], kern, s, x, x_dtype, ys[i], y_dtype, rows, ws));
         return 0;
     }
-    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32)
-        return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "x is bf16 or f32");
-    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "bad y dtype");
-    if (ls[0]->plan.ver == 3) {
-        RotGroupArgs r{};
-        fe_devptr_t xhs[kGroupMax] = {};
-        for (size_t i = 0; i < count; i++) {
-            if (!ys[i]) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null output");
-            xhs[i] = ws->xh.p + i * (size_t)rows * ls[i]->k * 2;
-            r.suh[i] = ls[i]->view.suh, r.xh[i] = xhs[i];
-        }
-        RotInput in;
-        uint32_t x_mode = (uint32_t)x_dtype & 1, k = ls[0]->k;
-        if (fused) {
-            in.x = x, in.mode = x_mode, in.ld = k;
-        } else {  // one launch rotates the input for every member
-            void *rargs[] = {&r, &x, &x_mode, &k};
-            FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
-        }
-        return launch_job(ls, count, s, xhs, ys, y_dtype, rows, ws, in, "fe_exl3_linear_forward_group");
-    }
-    GemvGroupArgs g{};
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32) return fe_set_error(FE_ERR_ARG, fn, "x is bf16 or f32");
+    if (y_dtype < 0 || y_dtype > 3) return fe_set_error(FE_ERR_ARG, fn, "bad y dtype");
     RotGroupArgs r{};
-    g.count = (uint32_t)count;
-    uint32_t lds = 0, programs = 0;
-    size_t z_at = 0, cnt_at = 0;
+    fe_devptr_t xhs[kGroupMax] = {};
     for (size_t i = 0; i < count; i++) {
-        const fe_exl3_linear *l = ls[i];
-        if (!ys[i]) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_forward_group", "null output");
-        GemvGroupArgs::Member &m = g.m[i];
-        m.trellis = l->view.trellis, m.svh = l->view.svh, m.suh = l->view.suh, m.y = ys[i];
-        m.xh = ws->xh.p + i * (size_t)rows * l->k * 2;
-        r.suh[i] = m.suh, r.xh[i] = m.xh;
-        m.z = ws->z.p + z_at * 4, m.counters = ws->counters.p + cnt_at * 4;
-        m.n = l->n, m.sk = l->plan.sk;
-        view_strides(l->view, &m.stride_k, &m.stride_nb);
-        m.chunk = gemv_chunk(rows, l->k / 64 / m.sk);
-        lds = std::max(lds, std::max(rows * (m.chunk * 128 + 16), rows * kRedPitch * 4));
-        g.first[i] = programs;
-        programs += l->n / 128 * m.sk;
-        z_at += (size_t)m.sk * rows * l->n, cnt_at += l->n / 128;
+        if (!ys[i]) return fe_set_error(FE_ERR_ARG, fn, "null output");
+        xhs[i] = ws->xh.p + i * (size_t)rows * ls[i]->k * 2;
+        r.suh[i] = ls[i]->view.suh, r.xh[i] = xhs[i];
     }
-    for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
-    uint32_t x_mode = (uint32_t)x_dtype & 1, k = ls[0]->k, mode = (uint32_t)y_dtype;
-    if (!fused) {  // one launch rotates the input for every member, and the GEMV reads the members' rotated inputs
+    RotInput in;
+    uint32_t x_mode = (uint32_t)x_dtype & 1, k = ls[0]->k;
+    if (fused) {
+        in.x = x, in.mode = x_mode, in.ld = k;
+    } else {  // one launch rotates the input for every member
         void *rargs[] = {&r, &x, &x_mode, &k};
         FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
-        x = 0;
     }
-    void *args[] = {&g, &x, &x_mode, &k, &rows, &mode};
-    return fe_hip_launch(kern->gemv_group[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
+    return launch_job(ls, count, s, xhs, ys, y_dtype, rows, ws, in, fn);
 }
 
 int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out) {

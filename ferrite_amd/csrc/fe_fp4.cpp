@@ -24,7 +24,14 @@ struct fe_fp4_kernels {
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
     uint32_t cus = 0;
-    uint32_t group_m = 8;  // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
+    // Switches of the launch paths: read from the environment once, at load; fe_fp4_kernels_set_option changes them
+    // afterwards. No forward call reads the environment.
+    uint32_t group_m = 8;      // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
+    uint32_t gemv = 1;         // up to 64 rows run the GEMV (FE_FP4_NO_GEMV=1: the GEMM's single tile row)
+    uint32_t gemv_sk = 0;      // K splits of the GEMV; 0 = two programs a CU (FE_FP4_GEMV_SK)
+    int32_t xcd = -1;          // column tiles dealt to the XCDs: -1 = where the weights are the larger operand (FE_FP4_XCD)
+    uint32_t fp8_f16 = 0;      // FP8 linears as fp16 expansion on the 16-bit matrix instruction (FE_FP8_F16=1)
+    uint32_t gemm_splits = 8;  // most pieces a cut output tile takes (FE_GEMM_SPLITS; 1: never cut)
 };
 
 struct fe_fp4_linear {
@@ -72,6 +79,11 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_cu_count(&cus);
     k->cus = (uint32_t)cus;
     if (const char *g = getenv("FE_FP4_GROUP")) k->group_m = (uint32_t)atoi(g);
+    if (const char *e = getenv("FE_FP4_NO_GEMV")) k->gemv = atoi(e) ? 0 : 1;
+    if (const char *e = getenv("FE_FP4_GEMV_SK")) k->gemv_sk = (uint32_t)atoi(e);
+    if (const char *e = getenv("FE_FP4_XCD")) k->xcd = atoi(e) ? 1 : 0;
+    if (const char *e = getenv("FE_FP8_F16")) k->fp8_f16 = atoi(e) ? 1 : 0;
+    if (const char *e = getenv("FE_GEMM_SPLITS")) k->gemm_splits = (uint32_t)atoi(e);
     if (c) {
         fe_fp4_kernels_destroy(k);
         return c;
@@ -84,6 +96,19 @@ int fe_fp4_kernels_destroy(fe_fp4_kernels *k) {
     if (!k) return 0;
     if (k->module) fe_hip_module_unload(k->module);
     delete k;
+    return 0;
+}
+
+int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value) {
+    if (!k || !name) return fe_set_error(FE_ERR_ARG, "fe_fp4_kernels_set_option", "null argument");
+    const std::string nm = name;
+    if (nm == "group_m") k->group_m = (uint32_t)value;
+    else if (nm == "gemv") k->gemv = value ? 1 : 0;
+    else if (nm == "gemv_sk") k->gemv_sk = (uint32_t)value;
+    else if (nm == "xcd") k->xcd = value;
+    else if (nm == "fp8_f16") k->fp8_f16 = value ? 1 : 0;
+    else if (nm == "gemm_splits") k->gemm_splits = (uint32_t)value;
+    else return fe_set_error(FE_ERR_ARG, "fe_fp4_kernels_set_option", name);
     return 0;
 }
 
@@ -273,12 +298,12 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     if (!y || ldy % 8 || y % 16 || (res && res % 16) || ldy < l->n)
         return fe_set_error(FE_ERR_ARG, "fe_fp4_linear_gemm", "gemm: y/res must be 16-byte aligned rows");
     uint32_t n = l->n, k = l->k;
-    if (!l->fp8 && m <= kGemvMaxRows && n / kTile <= kGemvCounters && !getenv("FE_FP4_NO_GEMV")) {
+    if (!l->fp8 && m <= kGemvMaxRows && n / kTile <= kGemvCounters && kern->gemv) {
         // decode-sized: the weight-read-bound GEMV, up to 48 rows a pass. Two programs fit a CU: as many programs as run
         // at once, not more (a second round of short programs costs more than idle CUs in the first).
         const uint32_t nts = n / kTile, kts = k / 64;
         uint32_t sk = 2 * kern->cus / nts;
-        if (const char *e = getenv("FE_FP4_GEMV_SK")) sk = (uint32_t)atoi(e);
+        if (kern->gemv_sk) sk = kern->gemv_sk;
         if (sk > 16) sk = 16;
         if (sk > kts / 4) sk = kts / 4;
         while (sk > 1 && (size_t)sk * kGemvRows * n * 4 > ws->part.bytes) sk--;
@@ -300,14 +325,14 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     // FP8 codes: the weights are the larger operand from n >= m on, and at the 8-bit instruction's rate their traffic
     // shows: column tiles are dealt to the XCDs (gemm_raster with group 0), each weight panel through one L2
     if (l->fp8 && n >= m) group = 0;
-    if (const char *e = getenv("FE_FP4_XCD")) group = atoi(e) ? 0 : group ? group : tiles_m;
+    if (kern->xcd >= 0) group = kern->xcd ? 0 : group ? group : tiles_m;
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
     // FP8 runs on the 8-bit matrix instruction over the codes of both operands, k tiles of 128 (FE_FP8_F16=1: the fp16
     // expansion on the 16-bit instruction, k tiles of 64; same products, another order of the f32 sums)
-    const char *f16env = getenv("FE_FP8_F16");
-    const bool codes8 = l->fp8 && !(f16env && atoi(f16env) != 0);
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    const bool codes8 = l->fp8 && !kern->fp8_f16;
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes),
+                                   kern->gemm_splits);
     uint32_t full = gs.full, splits = gs.splits;
     fe_devptr_t part = ws->part.p;
     float scale = l->fp8 ? 1.0f : 0.0625f;  // what the fp16 expansions of the two operands carry (FP4_OPERAND_SCALE)
@@ -356,7 +381,7 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p, part = ws->part.p;
     fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes));
+    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes), kern->gemm_splits);
     uint32_t full = gs.full, splits = gs.splits;
     void *args[] = {&aq,    &w,     &sw,   &alpha, &m,    &n,      &k,    &group,   &w_snt, &w_skt, &w_sr,
                     &s_snt, &s_skt, &s_sr, &full,  &splits, &part, &q_codes, &q_sf, &q_aq,  &down_g};

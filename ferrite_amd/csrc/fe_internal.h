@@ -93,15 +93,13 @@ constexpr size_t kFeGemmPartBytes = 256 * 256 * 4;  // one partial slot
 constexpr uint32_t kFeGemmSlotsPerCu = 2;           // slots a workspace holds per CU
 // The cut that finishes the last round soonest: s pieces a tile take ceil(rem s / cus) rounds of 1 / s of a tile's time;
 // every piece also writes its 256 KB partial and the reduce kernel reads it back (about 2 % of a tile's time a piece).
-// At most `slots` pieces.
-inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus, uint32_t slots) {
+// At most `slots` pieces in all and `cap` a tile (1: never cut).
+inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus, uint32_t slots, uint32_t cap = 8) {
     FeGemmSplit g;
     g.tiles = g.full = tiles;
     if (!cus || !slots) return g;
     const uint32_t rem = tiles % cus;
     if (rem == 0) return g;
-    uint32_t cap = 8;
-    if (const char *e = getenv("FE_GEMM_SPLITS")) cap = (uint32_t)atoi(e);  // 1: never cut
     cap = std::min(cap, ktiles / 4);                                        // at least 4 k tiles a program
     cap = std::min(cap, slots / rem);
     uint32_t best = 1;

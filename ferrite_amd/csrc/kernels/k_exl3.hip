@@ -206,7 +206,7 @@ extern "C" __global__ __launch_bounds__(128) void exl3_rot_in(const void* x, uin
     rot_in_body(RotSrc{x, x2, x_mode, ldx}, suh, xh, k);
 }
 
-#define FE_EXL3_GROUP_MAX 4  // linears of one grouped launch
+#define FE_EXL3_GROUP_MAX 4  // linears of one launch
 
 // The same input rotated for several linears (each by its own suh into its own xh): grid (ceil(k / 512), rows, members).
 struct RotGroup {
@@ -217,9 +217,9 @@ extern "C" __global__ __launch_bounds__(128) void exl3_rot_in_group(RotGroup g, 
     rot_in_body(RotSrc{x, nullptr, x_mode, k}, g.suh[blockIdx.z], g.xh[blockIdx.z], k);
 }
 
-// ---- decode GEMV -----------------------------------------------------------------------------------------------------
+// ---- decode GEMV: the lane mapping and the decode ----------------------------------------------------------------------
 //
-// One program = one 128-column block x one K split; 256 threads = 4 wavefronts, wavefront w owning tiles 2w, 2w + 1 of
+// A program works on one 128-column block at a time; 256 threads = 4 wavefronts, wavefront w owning tiles 2w, 2w + 1 of
 // the block's 8. A wavefront's load step covers 4 consecutive k steps of its two tiles: lane L = 16 g + r reads k step g,
 // tile r >> 3, the BITS words of fragment lanes 4q .. 4q + 3 (q = r & 7) plus the word before them, which is all its 32
 // states need. Those states are rows n = q and n = q + 8 of the tile over all 16 k, so after decoding the lane holds, for
@@ -232,9 +232,6 @@ struct LaneWords {
     uint32_t w[BITS + 1];  // w[0] = the word before the lane's run
 };
 
-#ifdef FE_NO_NT
-#define __builtin_nontemporal_load(p) (*(p))
-#endif
 template <int BITS>
 __device__ __forceinline__ LaneWords<BITS> load_lane_words(const uint32_t* run, const uint32_t* prev) {
     LaneWords<BITS> r;
@@ -363,317 +360,20 @@ __device__ __forceinline__ f32x4 row_scales(const uint16_t* svh, uint32_t col) {
 #endif
 #define GEMV_RED_PITCH 132  // floats a row of the 128-column partial sums (16-byte aligned, banks spread)
 
-// y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for m <= 16 RG rows. grid (n / 128 * sk), 256 threads. The rotated
-// inputs of the program's K range pass through LDS in chunks of `chunk` load steps (a multiple of 4): dynamic LDS
-// max(m * (chunk * 128 + 16), m * GEMV_RED_PITCH * 4) bytes. With sk > 1 the splits leave f32 partials in
-// z[split][m][n]; the last to arrive (counters[column block]) adds them in split order, finishes the block and re-arms
-// the counter. With src.x != nullptr the kernel rotates its own inputs from src (as exl3_rot_in does, bit for bit) instead of
-// reading xh, and leaves them in xh_out: one launch for the whole linear. That needs every staged K range to be whole
-// 128-element blocks: k / 64 / sk and chunk even. (kernels/k-exl3/src/gemv.rs:412-587)
-template <int BITS, int RG>
-__device__ __forceinline__ void gemv_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
-                                          const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
-                                          uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode,
-                                          uint32_t stride_k, uint32_t stride_nb, uint32_t chunk, const RotSrc src,
-                                          const uint16_t* __restrict__ suh, uint16_t* xh_out, uint32_t program) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    __shared__ uint32_t last_flag;
-    constexpr uint32_t tw = 8 * BITS;
-    constexpr int DEPTH = 4;   // load steps in flight per lane
-    constexpr int GROUP = 16;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
-    const uint32_t nbs = n / 128, nb = program % nbs, split = program / nbs;
-    const uint32_t per_split = (k / 16) / sk;  // k steps of this program, a multiple of 4
-    const uint32_t kt0 = split * per_split;
-    const uint32_t col0 = nb * 128;
-    const uint32_t steps = per_split / 4;
-    const uint32_t xpitch = chunk * 128 + 16;  // bytes a row of staged inputs
-
-    const uint32_t tile_word = (2 * wave + tau) * tw;
-    const uint32_t* base = trellis + (size_t)nb * stride_nb + (size_t)(kt0 + g) * stride_k + tile_word;
-    const uint32_t run_off = q * BITS, prev_off = (q * BITS + tw - 1) % tw;
-    const size_t step_words = (size_t)4 * stride_k;
-
-    uint32_t xrow[RG];
-#pragma unroll
-    for (int rg = 0; rg < RG; rg++) {
-        uint32_t row = 16 * rg + r;
-        xrow[rg] = (row < m ? row : m - 1) * xpitch + g * 32;
-    }
-
-    f32x4 acc[RG][2];
-#pragma unroll
-    for (int rg = 0; rg < RG; rg++) acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    // Rotating here: the first block's loads go out ahead of the trellis loads (loads return in order), so that the
-    // rotation runs while the first trellis words are still on their way.
-    const uint32_t rot_hw = tid >> 5, rot_l32 = tid & 31;
-    const void* x = src.x;
-    auto rot_at = [&](uint32_t c0, uint32_t nblk, uint32_t p, size_t& at, size_t& xat, uint32_t& c, uint32_t& off) {
-        uint32_t row = p / nblk, b = p - row * nblk;
-        c = (kt0 + 4 * c0) * 16 + b * 128 + 4 * rot_l32;
-        at = (size_t)row * k + c;
-        xat = (size_t)row * src.ld + c;
-        off = row * xpitch + b * 256 + 8 * rot_l32;
-    };
-    RotRaw rot_raw = {};
-    if (x) {
-        const uint32_t nblk = (steps < chunk ? steps : chunk) / 2;
-        if (rot_hw < m * nblk) {
-            size_t at, xat;
-            uint32_t c, off;
-            rot_at(0, nblk, rot_hw, at, xat, c, off);
-            rot_raw = rot_load(src, suh, xat, c);
-        }
-    }
-
-    // the ring is indexed by constants only, so it stays in registers
-    LaneWords<BITS> ring[DEPTH];
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) {
-        const uint32_t* p = base + (size_t)(j < (int)steps ? j : 0) * step_words;
-        ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
-    }
-    for (uint32_t c0 = 0; c0 < steps; c0 += chunk) {
-        const uint32_t cs = steps - c0 < chunk ? steps - c0 : chunk;
-        if (c0) __syncthreads();
-        if (x) {
-            // the input rotation of this K range, done here: half wavefronts take (row, 128-block) pairs; the programs
-            // of column block 0 also leave the rotated input in xh_out. The range starts and ends on block boundaries
-            // (the launcher's condition for passing x).
-            const uint32_t nblk = cs / 2, total = m * nblk;
-            uint32_t p = rot_hw, c = 0, off = 0;
-            size_t at = 0, xat = 0;
-            if (p < total) {
-                rot_at(c0, nblk, p, at, xat, c, off);
-                if (c0) rot_raw = rot_load(src, suh, xat, c);
-            }
-            while (p < total) {
-                u32x2 o = rot_finish(rot_raw, src.mode, rot_l32);
-                *(u32x2*)(lds + off) = o;
-                if (nb == 0 && xh_out) *(u32x2*)(xh_out + at) = o;
-                p += 8;
-                if (p < total) {
-                    rot_at(c0, nblk, p, at, xat, c, off);
-                    rot_raw = rot_load(src, suh, xat, c);
-                }
-            }
-        } else {  // rotated inputs of k steps kt0 + 4 c0 .. + 4 cs -> LDS [row][cs * 64 fp16]
-            // (NB loads in flight a thread: one after the other they cost a trip to L2 each, 8 per chunk at 64 rows;
-            // fewer for one row group, whose kernels would lose a resident wavefront to the registers)
-            constexpr int NB = RG == 1 ? FE_STAGE_NB1 : 8;
-            const uint32_t chunks16 = cs * 8, total = m * chunks16;  // 16-byte pieces a row, pieces in all
-            const uint16_t* xsrc = xh + (size_t)(kt0 + 4 * c0) * 16;
-            for (uint32_t i0 = tid; i0 < total; i0 += 256 * NB) {
-                u32x4 v[NB];
-                uint32_t off[NB];
-#pragma unroll
-                for (int j = 0; j < NB; j++) {
-                    const uint32_t i = i0 + 256 * j < total ? i0 + 256 * j : i0;  // past the end: a piece again, not stored
-                    const uint32_t row = i / chunks16, c = i - row * chunks16;
-                    v[j] = *(const u32x4*)(xsrc + (size_t)row * k + c * 8);
-                    off[j] = row * xpitch + c * 16;
-                }
-#pragma unroll
-                for (int j = 0; j < NB; j++)
-                    if (i0 + 256 * j < total) *(u32x4*)(lds + off[j]) = v[j];
-            }
-        }
-        __syncthreads();
-        auto mma = [&](const f16x8 (&op)[2][2], uint32_t sl) {
-#pragma unroll
-            for (int rg = 0; rg < RG; rg++) {
-                const unsigned char* xp = lds + xrow[rg] + sl * 128;
-                f16x8 x0 = *(const f16x8*)xp, x1 = *(const f16x8*)(xp + 16);
-                acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[rg][0], 0, 0, 0);
-                acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[rg][1], 0, 0, 0);
-                acc[rg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[rg][0], 0, 0, 0);
-                acc[rg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[rg][1], 0, 0, 0);
-            }
-        };
-        // Whole groups of GROUP steps run as straight-line code: no branches inside, and the refill of a ring slot is
-        // unconditional (the step index is clamped to the last one), so each load lands straight in the slot its words
-        // were just decoded from and only that slot's next use waits for it. The wait at the top of a group has to
-        // cover every load in flight (the compiler cannot count across the back edge), hence long groups.
-        const uint32_t full = cs / GROUP * GROUP;
-        for (uint32_t s0 = 0; s0 < full; s0 += GROUP) {
-#pragma unroll
-            for (int j = 0; j < GROUP; j++) {
-                f16x8 op[2][2];
-                decode_lane<BITS>(ring[j % DEPTH], op);
-                uint32_t nxt = c0 + s0 + j + DEPTH;
-                nxt = nxt < steps ? nxt : steps - 1;
-                const uint32_t* p = base + (size_t)nxt * step_words;
-                ring[j % DEPTH] = load_lane_words<BITS>(p + run_off, p + prev_off);
-                // keep each refill where it is issued: left alone, the scheduler sinks the loads to the end of the
-                // group, right in front of the wait for them
-                __builtin_amdgcn_sched_barrier(0);
-                mma(op, s0 + j);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-        for (uint32_t s0 = full; s0 < cs; s0 += DEPTH) {  // the remainder, slot by slot
-#pragma unroll
-            for (int j = 0; j < DEPTH; j++)
-                if (s0 + j < cs) {
-                    f16x8 op[2][2];
-                    decode_lane<BITS>(ring[j], op);
-                    uint32_t nxt = c0 + s0 + j + DEPTH;
-                    nxt = nxt < steps ? nxt : steps - 1;
-                    const uint32_t* p = base + (size_t)nxt * step_words;
-                    ring[j] = load_lane_words<BITS>(p + run_off, p + prev_off);
-                    mma(op, s0 + j);
-                }
-        }
-    }
-
-    // the block's sums -> LDS [row][128] (the input rows are no longer needed)
-    __syncthreads();
-    float* red = (float*)lds;
-#pragma unroll
-    for (int rg = 0; rg < RG; rg++) {
-        uint32_t row = 16 * rg + r;  // accumulator column = input row
-        if (row < m) {
-#pragma unroll
-            for (int h = 0; h < 2; h++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    uint32_t arow = 4 * g + i;  // row of A: tile arow >> 3 of the pair, n = (arow & 7) + 8 h
-                    uint32_t col = 32 * wave + 16 * (arow >> 3) + (arow & 7) + 8 * h;
-                    red[row * GEMV_RED_PITCH + col] = acc[rg][h][i];
-                }
-        }
-    }
-    __syncthreads();
-
-    const uint32_t hw = tid >> 5, l32 = tid & 31;
-    if (sk == 1) {
-        for (uint32_t row = hw; row < m; row += 8) {
-            f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
-            float v[4] = {t[0], t[1], t[2], t[3]};
-            finish_row(v, l32, svh, col0 + 4 * l32, y, y_mode, (size_t)row * n + col0 + 4 * l32);
-        }
-        return;
-    }
-    // Split partials cross to another program, possibly on another XCD with its own L2: they are written and read with
-    // agent-scope accesses (write-through / L2-bypassing), ordered by the barrier around the arrival counter, so no
-    // device-wide cache write-back or invalidate is needed.
-    for (uint32_t row = hw; row < m; row += 8) {
-        const float* src = red + row * GEMV_RED_PITCH + 4 * l32;
-        store_agent_f32x4(z + ((size_t)split * m + row) * n + col0 + 4 * l32, *(const f32x4*)src);
-    }
-    agent_stores_wait();  // this lane's stores are acknowledged at agent scope
-    __syncthreads();
-    if (tid == 0) {
-        uint32_t old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        last_flag = (old == sk - 1);
-    }
-    __syncthreads();
-    if (last_flag) {
-        // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB splits each, so that 16 loads are
-        // in flight (an agent-scope load takes a trip to memory); every row's partials are added in split order.
-        constexpr int RB = RG == 1 ? 2 : 4, SB = 16 / RB;
-        for (uint32_t row0 = hw; row0 < m; row0 += 8 * RB) {
-            float v[RB][4];
-#pragma unroll
-            for (int j = 0; j < RB; j++) v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.f;
-            for (uint32_t sp0 = 0; sp0 < sk; sp0 += SB) {
-                f32x4 t[RB * SB];
-#pragma unroll
-                for (int j = 0; j < RB; j++) {
-                    const uint32_t row = row0 + 8 * j < m ? row0 + 8 * j : row0;
-#pragma unroll
-                    for (int b = 0; b < SB; b++)
-                        t[j * SB + b] = load_agent_f32x4(z + ((size_t)(sp0 + b < sk ? sp0 + b : sk - 1) * m + row) * n + col0 + 4 * l32);
-                }
-                agent_loads_wait(t);
-#pragma unroll
-                for (int j = 0; j < RB; j++)
-#pragma unroll
-                    for (int b = 0; b < SB; b++)
-                        if (sp0 + b < sk) {
-#pragma unroll
-                            for (int e = 0; e < 4; e++) v[j][e] += t[j * SB + b][e];
-                        }
-            }
-#pragma unroll
-            for (int j = 0; j < RB; j++) {
-                const uint32_t row = row0 + 8 * j;
-                if (row < m) finish_row(v[j], l32, svh, col0 + 4 * l32, y, y_mode, (size_t)row * n + col0 + 4 * l32);
-            }
-        }
-        if (tid == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-}
-
-#define GEMV_KERNEL(BITS, RG)                                                                                         \
-    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_b##BITS##_r##RG(                                      \
-        const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,       \
-        uint32_t n, uint32_t k, uint32_t m, uint32_t sk, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb,       \
-        uint32_t chunk, const void* x, uint32_t x_mode, const uint16_t* suh, uint16_t* xh_out, const void* x2,         \
-        uint32_t ldx) {                                                                                               \
-        gemv_body<BITS, RG>(xh, trellis, svh, y, z, counters, n, k, m, sk, y_mode, stride_k, stride_nb, chunk,        \
-                            RotSrc{x, x2, x_mode, ldx}, suh, xh_out, blockIdx.x);                                     \
-    }
-#define GEMV_FAMILY(BITS) GEMV_KERNEL(BITS, 1) GEMV_KERNEL(BITS, 2) GEMV_KERNEL(BITS, 3) GEMV_KERNEL(BITS, 4)
-
-// Several linears of one input in one launch (the projections a model applies to the same activations: q, k, v; gate,
-// up): the programs of member i are first[i] .. first[i + 1] - 1, each exactly the program of the member's own launch
-// (same split, same sums, same bits), rotating the input by the member's own suh (x != nullptr) or reading the member's
-// rotated input xh (exl3_rot_in_group). The launches' start-up and tails overlap and the members' programs fill each
-// other's gaps on the CUs. 1..64 rows (16 RG).
-struct GemvGroup {
-    uint32_t count, first[FE_EXL3_GROUP_MAX + 1];
-    struct Member {
-        const uint32_t* trellis;
-        const uint16_t *svh, *suh, *xh;
-        void* y;
-        float* z;
-        uint32_t* counters;
-        uint32_t n, sk, stride_k, stride_nb, chunk, pad;
-    } m[FE_EXL3_GROUP_MAX];
-};
-#define GEMV_GROUP_KERNEL(BITS, RG, NAME)                                                                              \
-    extern "C" __global__ __launch_bounds__(256, 2) void NAME(GemvGroup g, const void* x, uint32_t x_mode, uint32_t k, \
-                                                              uint32_t m, uint32_t y_mode) {                           \
-        uint32_t i = 0;                                                                                                \
-        while (i + 1 < g.count && blockIdx.x >= g.first[i + 1]) i++;                                                   \
-        const GemvGroup::Member& mb = g.m[i];                                                                          \
-        gemv_body<BITS, RG>(mb.xh, mb.trellis, mb.svh, mb.y, mb.z, mb.counters, mb.n, k, m, mb.sk, y_mode,             \
-                            mb.stride_k, mb.stride_nb, mb.chunk, RotSrc{x, nullptr, x_mode, k}, mb.suh, nullptr,       \
-                            blockIdx.x - g.first[i]);                                                                  \
-    }
-#define GEMV_GROUP_FAMILY(BITS)                                 \
-    GEMV_GROUP_KERNEL(BITS, 1, exl3_gemv_group_b##BITS)         \
-    GEMV_GROUP_KERNEL(BITS, 2, exl3_gemv_group_b##BITS##_r2)    \
-    GEMV_GROUP_KERNEL(BITS, 3, exl3_gemv_group_b##BITS##_r3)    \
-    GEMV_GROUP_KERNEL(BITS, 4, exl3_gemv_group_b##BITS##_r4)
-GEMV_FAMILY(2)
-GEMV_FAMILY(3)
-GEMV_FAMILY(4)
-GEMV_FAMILY(5)
-GEMV_FAMILY(6)
-GEMV_FAMILY(8)
-GEMV_GROUP_FAMILY(2)
-GEMV_GROUP_FAMILY(3)
-GEMV_GROUP_FAMILY(4)
-GEMV_GROUP_FAMILY(5)
-GEMV_GROUP_FAMILY(6)
-GEMV_GROUP_FAMILY(8)
-
 // ---- decode GEMV, balanced over the CUs (1..64 rows) ------------------------------------------------------------------
 //
 // Work unit = one 128-channel block of K of one 128-column block of N (two load steps); units are ordered column block
-// by column block and the member's `programs` programs each take one contiguous run of them, base or base + 1 units long,
-// whatever the shape: every program decodes the same number of weights, so with a multiple of the CU count of programs
-// every CU does. A run may start and end inside a column block, so a block's sum is assembled from segments: each program
+// by column block and the member's `programs` programs each take one contiguous run of them, base + 1 units for the first
+// rem programs and base for the rest, whatever the shape: with a multiple of the CU count of programs, which the CUs take
+// round by round, the CUs' shares differ by at most one unit. (Spreading the longer runs evenly over the program numbers
+// is worse: their period can divide the CU count, and then a CU gets only long runs or only short ones.) A run may start and end inside a column block, so a block's sum is assembled from segments: each program
 // leaves the partial sums of its segment of block nb in z[program + nb] and bumps the block's arrival counter; the
 // program that arrives last adds the segments in program order (the order does not depend on who is last: deterministic),
 // applies the output rotation and re-arms the counter. The partition depends on (k, n, programs) only, never on the
-// row count: row r of a batch has the bits of the single-row call. Inside a program the work is laid out as in the
-// split-K kernel above: 4 wavefronts owning 2 of the block's 8 tiles each, the rotated inputs of the run staged in LDS
-// (rotated here when src.x is set), four load steps in flight per lane.
+// row count: row r of a batch has the bits of the single-row call. Inside a program: 4 wavefronts owning 2 of the
+// block's 8 tiles each, the rotated inputs of the run staged in LDS (rotated here when src.x is set), four load steps in
+// flight per lane. Several linears of one input share a launch: each member's programs are exactly those of its own
+// launch (same runs, same sums, same bits). (kernels/k-exl3/src/gemv.rs:412-587 is the reference's split-K form.)
 struct GemvMember {
     const uint32_t* trellis;
     const uint16_t *svh, *suh;
@@ -682,7 +382,7 @@ struct GemvMember {
     float* z;            // segment partial sums [programs + n / 128][m][128]
     uint32_t* counters;  // arrivals per column block, zero at rest
     uint32_t n, programs, stride_k, stride_nb;
-    uint32_t base, rem;            // units / programs, units % programs
+    uint32_t base, rem;            // units / programs, units % programs, units = (n / 128) * (k / 128)
     uint32_t inv_base, inv_base1;  // floor((2^32 - 1) / base), floor((2^32 - 1) / (base + 1))
 };
 struct GemvJob {
@@ -709,14 +409,20 @@ __device__ __forceinline__ uint32_t udiv_inv(uint32_t x, uint32_t d, uint32_t in
 #define FE_STAMP_AT(i)
 #endif
 
-// The ring of load steps turned left by `phase` slots, so that the oldest step in flight sits in slot 0 again.
+// The ring of load steps turned left by `phase` slots (phase < DEPTH), so that the oldest step in flight sits in slot 0
+// again: one pass of moves whatever the phase.
 template <int BITS, int DEPTH>
 __device__ __forceinline__ void ring_turn(LaneWords<BITS> (&ring)[DEPTH], uint32_t phase) {
-    for (; phase; phase--) {
+    static_assert(DEPTH == 4, "the turns below are written out for four slots");
+    if (phase == 1) {
         LaneWords<BITS> t = ring[0];
-#pragma unroll
-        for (int i = 0; i + 1 < DEPTH; i++) ring[i] = ring[i + 1];
-        ring[DEPTH - 1] = t;
+        ring[0] = ring[1], ring[1] = ring[2], ring[2] = ring[3], ring[3] = t;
+    } else if (phase == 2) {
+        LaneWords<BITS> t0 = ring[0], t1 = ring[1];
+        ring[0] = ring[2], ring[1] = ring[3], ring[2] = t0, ring[3] = t1;
+    } else if (phase == 3) {
+        LaneWords<BITS> t = ring[3];
+        ring[3] = ring[2], ring[2] = ring[1], ring[1] = ring[0], ring[0] = t;
     }
 }
 
@@ -771,11 +477,8 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
     }
 #endif
     constexpr uint32_t tw = 8 * BITS;
-#ifndef FE_GEMVB_DEPTH
-#define FE_GEMVB_DEPTH 4
-#endif
-    constexpr int DEPTH = FE_GEMVB_DEPTH;  // load steps in flight per lane
-    constexpr int GROUP = 8;               // steps of straight-line code per loop iteration (a multiple of DEPTH)
+    constexpr int DEPTH = 4;  // load steps in flight per lane (8 measured slower: 22.9 against 20.7 us)
+    constexpr int GROUP = 8;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
     const uint32_t n = mb.n, spb = k / 64, upb = spb / 2;  // load steps, units a column block
@@ -903,7 +606,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
         }
         __syncthreads();
         const uint32_t col0 = fnb * 128;
-        // programs of the block's first and last unit (units are dealt base + 1 to the first rem programs, base to the rest)
+        // programs of the block's first and last unit
         const uint32_t cut = rem * (base + 1), ua = fnb * upb, ub = ua + upb - 1;
         const uint32_t first_prog = ua < cut ? udiv_inv(ua, base + 1, mb.inv_base1) : rem + udiv_inv(ua - cut, base, mb.inv_base);
         const uint32_t last_prog = ub < cut ? udiv_inv(ub, base + 1, mb.inv_base1) : rem + udiv_inv(ub - cut, base, mb.inv_base);
@@ -1063,8 +766,9 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
 #endif
 }
 
+// (second launch bound: wavefronts per SIMD the registers must allow. Four programs a CU for up to 16 rows.)
 #define GEMVB_KERNEL(BITS, RG)                                                                                        \
-    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemvb_b##BITS##_r##RG(                                   \
+    extern "C" __global__ __launch_bounds__(256, RG == 1 ? 4 : 2) void exl3_gemvb_b##BITS##_r##RG(                                   \
         GemvJob job, const void* x, const void* x2, uint32_t x_mode, uint32_t ldx, uint32_t k, uint32_t m,             \
         uint32_t y_mode, uint32_t chunk, uint32_t inv_spb FE_STAMP_ARG) {                                             \
         uint32_t i = 0;                                                                                               \
@@ -1079,195 +783,6 @@ GEMVB_FAMILY(4)
 GEMVB_FAMILY(5)
 GEMVB_FAMILY(6)
 GEMVB_FAMILY(8)
-
-// ---- decode GEMV, streamed over the whole tensor (1..16 rows) -------------------------------------------------------------
-//
-// Work unit = one load step (64 input channels) of one 128-column block; units are ordered column block by column block
-// (in the strips layout that is the byte order of the trellis), and the gridDim.x programs each take one contiguous,
-// equally long run of them, whatever the shape: every CU streams the same number of bytes. A run may start and end in
-// the middle of a column block, so a block's sum is assembled from segments: each wavefront of each segment leaves its
-// partial sums in z[program + block] and bumps the block's arrival counter; the wavefront that arrives last adds the
-// segments in order, applies the output rotation and re-arms the counter. The four wavefronts of a program own two tiles
-// of the block each and never exchange data: no LDS, no barriers; the rotated inputs come straight from L2 with the
-// weights, one ring slot per load step.
-
-template <int BITS>
-struct StreamSlot {
-    LaneWords<BITS> w;
-    f16x8 x0, x1;  // rotated inputs of the lane's input row, k 0..7 and 8..15 of the lane's k step
-    // member-wise copy: a whole-struct copy would also move the padding bytes and pin them to the stack
-    __device__ __forceinline__ void take(const StreamSlot& o) {
-#pragma unroll
-        for (int i = 0; i <= BITS; i++) w.w[i] = o.w.w[i];
-        x0 = o.x0, x1 = o.x1;
-    }
-};
-
-// Program that owns unit u when U units are dealt as base + 1 to the first rem programs and base to the rest.
-__device__ __forceinline__ uint32_t stream_owner(uint32_t u, uint32_t base, uint32_t rem) {
-    uint32_t cut = rem * (base + 1);
-    return u < cut ? u / (base + 1) : rem + (u - cut) / base;
-}
-
-template <int BITS>
-__device__ __forceinline__ void gemv_stream_body(const uint16_t* __restrict__ xh, const uint32_t* __restrict__ trellis,
-                                                 const uint16_t* __restrict__ svh, void* y, float* z, uint32_t* counters,
-                                                 uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t stride_k,
-                                                 uint32_t stride_nb) {
-    constexpr uint32_t tw = 8 * BITS;
-    constexpr int DEPTH = 4;  // load steps in flight per lane
-    constexpr int GROUP = 8;  // steps of straight-line code per loop iteration
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
-    const uint32_t steps = k / 64, nbs = n / 128, units = nbs * steps;
-    const uint32_t progs = gridDim.x, p = blockIdx.x;
-    const uint32_t base = units / progs, rem = units % progs;
-    const uint32_t u0 = p * base + (p < rem ? p : rem), u1 = u0 + base + (p < rem ? 1 : 0);
-    if (u0 >= u1) return;
-    // arrivals of this program's wavefronts per column block touched (index: block - first block, wrapped)
-    __shared__ uint32_t arrived[64];
-    if (tid < 64) arrived[tid] = 0;
-    __syncthreads();
-    const uint32_t nb_first = u0 / steps;
-
-    const uint32_t lane_word = (2 * wave + tau) * tw, run_off = lane_word + q * BITS, prev_off = lane_word + (q * BITS + tw - 1) % tw;
-    const uint16_t* xrow = xh + (size_t)(r < m ? r : m - 1) * k + g * 16;
-
-    // refill cursor: the next unit to request, as (column block, step)
-    uint32_t ru = u0, rnb = u0 / steps, rst = u0 % steps;
-    auto issue = [&](StreamSlot<BITS>& slot) {
-        const uint32_t* wp = trellis + (size_t)rnb * stride_nb + (size_t)(4 * rst + g) * stride_k;
-        slot.w = load_lane_words<BITS>(wp + run_off, wp + prev_off);
-        const uint16_t* xp = xrow + rst * 64;
-        slot.x0 = *(const f16x8*)xp;
-        slot.x1 = *(const f16x8*)(xp + 8);
-        if (ru + 1 < u1) {  // past the end of the run the last unit is requested again (and never used)
-            ru++;
-            if (++rst == steps) rst = 0, rnb++;
-        }
-    };
-
-    StreamSlot<BITS> ring[DEPTH];
-#pragma unroll
-    for (int j = 0; j < DEPTH; j++) issue(ring[j]);
-
-    f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-    auto one = [&](StreamSlot<BITS>& slot) {
-        f16x8 op[2][2];
-        decode_lane<BITS>(slot.w, op);
-        f16x8 x0 = slot.x0, x1 = slot.x1;
-        issue(slot);
-        __builtin_amdgcn_sched_barrier(0);  // the refill stays here, ahead of the matrix work
-        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], x0, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], x0, acc[1], 0, 0, 0);
-        acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], x1, acc[0], 0, 0, 0);
-        acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], x1, acc[1], 0, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-    };
-
-    uint32_t u = u0, nb = u0 / steps, st = u0 % steps;
-    while (u < u1) {
-        const uint32_t seg = (steps - st < u1 - u) ? steps - st : u1 - u;  // units left in this column block
-        const uint32_t full = seg / GROUP * GROUP;
-        for (uint32_t i = 0; i < full; i += GROUP) {
-#pragma unroll
-            for (int j = 0; j < GROUP; j++) one(ring[j % DEPTH]);
-        }
-        const uint32_t tail = seg - full;
-        for (uint32_t i = 0; i < tail; i += DEPTH) {
-#pragma unroll
-            for (int j = 0; j < DEPTH; j++)
-                if (i + j < tail) one(ring[j]);
-        }
-
-        // segment end: partial sums of this wavefront's 32 columns -> z[program + block][row][128]
-        const uint32_t col0 = nb * 128;
-        const uint32_t first_prog = stream_owner(nb * steps, base, rem), last_prog = stream_owner(nb * steps + steps - 1, base, rem);
-        if (r < m) {
-            // A rows 4 g .. 4 g + 3 of half h are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32
-            float* zp = z + ((size_t)(p + nb) * m + r) * 128 + 32 * wave + 16 * (g >> 1) + 4 * (g & 1);
-            store_agent_f32x4(zp, acc[0]);
-            store_agent_f32x4(zp + 8, acc[1]);
-        }
-        acc[0] = acc[1] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        agent_stores_wait();  // this wavefront's partial sums are acknowledged at agent scope
-        // the program's four wavefronts meet on an LDS counter; the last of them reports the segment to the block's
-        // global arrival counter, and the last segment to arrive finishes the block
-        uint32_t old = 0;
-        if (lane == 0) old = __hip_atomic_fetch_add(&arrived[(nb - nb_first) & 63], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        old = __builtin_amdgcn_readfirstlane(old);
-        bool finisher = false;
-        if (old == 3) {
-            uint32_t g_old = 0;
-            if (lane == 0) g_old = __hip_atomic_fetch_add(&counters[nb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            finisher = (uint32_t)__builtin_amdgcn_readfirstlane(g_old) == last_prog - first_prog;
-        }
-        if (finisher) {
-            // add the segments in program order, rotate, scale, store; two rows at a time, 8 segments' loads in flight
-            const uint32_t l32 = lane & 31;
-            for (uint32_t row0 = 0; row0 < m; row0 += 2) {
-                const uint32_t row = row0 + (lane >> 5);
-                const bool live = row < m;
-                float v[4] = {0.f, 0.f, 0.f, 0.f};
-                for (uint32_t sp0 = first_prog; sp0 <= last_prog; sp0 += 8) {
-                    f32x4 t[8];
-#pragma unroll
-                    for (int b = 0; b < 8; b++) {
-                        const uint32_t sp = sp0 + b <= last_prog ? sp0 + b : last_prog;
-                        t[b] = load_agent_f32x4(z + ((size_t)(sp + nb) * m + (live ? row : 0)) * 128 + 4 * l32);
-                    }
-                    agent_loads_wait(t);
-#pragma unroll
-                    for (int b = 0; b < 8; b++)
-                        if (sp0 + b <= last_prog) {
-#pragma unroll
-                            for (int e = 0; e < 4; e++) v[e] += t[b][e];
-                        }
-                }
-                fwht128_half_wave(v, l32);
-                if (live) {
-                    u32x2 sv = *(const u32x2*)(svh + col0 + 4 * l32);
-                    v[0] = v[0] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] & 0xffff);
-                    v[1] = v[1] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] >> 16);
-                    v[2] = v[2] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] & 0xffff);
-                    v[3] = v[3] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] >> 16);
-                    store4(y, y_mode, (size_t)row * n + col0 + 4 * l32, v);
-                }
-            }
-            if (lane == 0) __hip_atomic_store(&counters[nb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-
-        // the next unit sits in slot tail % DEPTH: turn the ring so that it is slot 0 again (nothing is in flight here)
-        const uint32_t phase = tail % DEPTH;
-        if (phase == 1) {
-            StreamSlot<BITS> t;
-            t.take(ring[0]), ring[0].take(ring[1]), ring[1].take(ring[2]), ring[2].take(ring[3]), ring[3].take(t);
-        } else if (phase == 2) {
-            StreamSlot<BITS> t0, t1;
-            t0.take(ring[0]), t1.take(ring[1]);
-            ring[0].take(ring[2]), ring[1].take(ring[3]), ring[2].take(t0), ring[3].take(t1);
-        } else if (phase == 3) {
-            StreamSlot<BITS> t;
-            t.take(ring[3]), ring[3].take(ring[2]), ring[2].take(ring[1]), ring[1].take(ring[0]), ring[0].take(t);
-        }
-        u += seg;
-        st += seg;
-        if (st == steps) st = 0, nb++;
-    }
-}
-
-#define GEMV_STREAM_KERNEL(BITS)                                                                                       \
-    extern "C" __global__ __launch_bounds__(256, 2) void exl3_gemv_stream_b##BITS(                                     \
-        const uint16_t* xh, const uint32_t* trellis, const uint16_t* svh, void* y, float* z, uint32_t* counters,        \
-        uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb) {                   \
-        gemv_stream_body<BITS>(xh, trellis, svh, y, z, counters, n, k, m, y_mode, stride_k, stride_nb);                \
-    }
-GEMV_STREAM_KERNEL(2)
-GEMV_STREAM_KERNEL(3)
-GEMV_STREAM_KERNEL(4)
-GEMV_STREAM_KERNEL(5)
-GEMV_STREAM_KERNEL(6)
-GEMV_STREAM_KERNEL(8)
 
 // ---- prefill GEMM ----------------------------------------------------------------------------------------------------
 

@@ -156,8 +156,8 @@ class Plan:
 
 
 def default_blocks(cu_count: int) -> int:
-    """Programs a GEMV launch aims for (the role of linear.rs:131-134; 2.75 a CU measured best on MI355X)."""
-    return 11 * cu_count // 4
+    """Programs a GEMV launch aims for: 4 a CU (linear.rs:131-134)."""
+    return 4 * cu_count
 
 
 def _stream(s):
@@ -186,6 +186,10 @@ class Kernels:
         if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
             _lib._lib.fe_exl3_kernels_destroy(self.h)
             self.h = None
+
+    def set_option(self, name: str, value: int):
+        """A switch of the launch paths ("fused_rot", "group", "hat_rows", ...: include/fe_exl3.h)."""
+        check(_lib.lib().fe_exl3_kernels_set_option(self.h, name.encode(), int(value)))
 
     def reconstruct_hat_f16(self, view: Exl3View, out, stream=None):
         """Rotated-basis W_hat as fp16 [k][n] (gpu/mod.rs:159-165)."""
@@ -337,36 +341,54 @@ class Workspace:
             self.h = None
 
 
-def tune(kern: Kernels, t: Exl3Tensor, iters: int = 50, w16: float = 0.25, copies_bytes: int = 600 << 20):
-    """Times every fitting plan on one tensor shape at 1 and 16 rows and returns (best plan, table), the table a list of
+def tune(kern: Kernels, t: Exl3Tensor, iters: int = 50, w16: float = 0.25, copies_bytes: int = 600 << 20,
+         occs=(2, 3, 4, 5), min_units=(2, 4, 8)):
+    """Times every candidate plan on one tensor shape at 1 and 16 rows and returns (best plan, table), the table a list of
     (plan, us at 1 row, us at 16 rows) sorted by us1 + w16 * us16 (the measure of
     crates/fe-exl3/src/bin/exl3-tune.rs:75-118). Launches cycle over enough copies of the weights that none is served
-    from a cache; candidates are the split counts that divide the K steps (ver 1) and the streamed form at 2 and 3
-    programs per CU (ver 2)."""
+    from a cache. Candidates: occ programs per CU, each a run of at least wk units of 128 channels x 128 columns; plans
+    that come to the same program count are timed once."""
     import torch
-    steps = t.k // 64
-    cands = [Plan(sk, 4, 1, 0) for sk in range(1, steps // 2 + 1) if steps % sk == 0 and sk <= 64]
-    cands += [Plan(1, 4, 2, occ) for occ in (2, 3)]
     copies = max(2, min(64, copies_bytes // max(1, t.trellis_bytes()) + 1))
     devs = [DeviceExl3.upload_strips(t) for _ in range(copies)]
     x = torch.full((16, t.k), 1.0, dtype=torch.bfloat16, device="cuda")
     y = torch.zeros((16, t.n), dtype=torch.bfloat16, device="cuda")
-    table = []
-    for p in cands:
-        lins = [Linear.from_view(kern, d.name, d.view, p) for d in devs]
-        ws = Workspace(lins[:1], 16)
-        us = []
-        for rows in (1, 16):
-            lins[0].rotate_input(x, Dtype.Bf16, rows, ws)
-            for lin in lins[:2]:
-                lin.gemv_rotated(ws.xh_ptr, y, Dtype.Bf16, rows, ws)
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for i in range(iters):
-                lins[i % copies].gemv_rotated(ws.xh_ptr, y, Dtype.Bf16, rows, ws)
-            b.record()
-            torch.cuda.synchronize()
-            us.append(a.elapsed_time(b) * 1e3 / iters)
-        table.append((p, us[0], us[1]))
+    units, cus = (t.k // 128) * (t.n // 128), cu_count()
+    table, seen = [], set()
+    for occ in occs:
+        for wk in min_units:
+            programs = max(1, min(occ * cus, units // wk))
+            if (occ, programs) in seen:
+                continue
+            seen.add((occ, programs))
+            p = Plan(-(-programs // (t.n // 128)), wk, 3, occ)
+            lins = [Linear.from_view(kern, d.name, d.view, p) for d in devs]
+            ws = Workspace(lins[:1], 16)
+            us = []
+            for rows in (1, 16):
+                for lin in lins[:2]:
+                    lin.forward(x, Dtype.Bf16, y, Dtype.Bf16, rows, ws)
+                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record()
+                for i in range(iters):
+                    lins[i % copies].forward(x, Dtype.Bf16, y, Dtype.Bf16, rows, ws)
+                b.record()
+                torch.cuda.synchronize()
+                us.append(a.elapsed_time(b) * 1e3 / iters)
+            table.append((p, us[0], us[1]))
     table.sort(key=lambda e: e[1] + w16 * e[2])
     return table[0][0], table
+
+
+if __name__ == "__main__":
+    # python -m ferrite_amd.exl3 tune [k n bits]...: prints rows for ferrite_amd/csrc/fe_exl3_plans.h
+    import sys
+    from . import synth
+    if len(sys.argv) >= 2 and sys.argv[1] == "tune":
+        shapes = [tuple(int(v) for v in a.split("x")) for a in sys.argv[2:]] or [
+            (k, n, b) for b in (3, 4, 5) for k, n in ((5120, 17408), (17408, 5120))] + [(5120, 5120, 4), (5120, 1024, 4)]
+        kern = Kernels.load()
+        for k, n, bits in shapes:
+            best, table = tune(kern, synth.exl3_tensor(k, n, bits, 1))
+            print(f"    {{{k}, {n}, {bits}, {cu_count()}, {best.occ}, {best.wk}}},  // " +
+                  "; ".join(f"occ {p.occ} wk {p.wk}: {u1:.1f} / {u16:.1f} us" for p, u1, u16 in table[:4]), flush=True)

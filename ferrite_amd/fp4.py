@@ -131,6 +131,10 @@ class Kernels:
     def load(cls):
         return cls()
 
+    def set_option(self, name: str, value: int):
+        """A switch of the launch paths, by name (the header lists them)."""
+        check(_lib.lib().fe_fp4_kernels_set_option(self.h, name.encode(), int(value)))
+
     def __del__(self):
         if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
             _lib._lib.fe_fp4_kernels_destroy(self.h)

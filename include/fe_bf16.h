@@ -23,6 +23,9 @@ extern "C" {
 typedef struct fe_bf16_kernels fe_bf16_kernels;
 int fe_bf16_kernels_load(fe_bf16_kernels **out);
 int fe_bf16_kernels_destroy(fe_bf16_kernels *k);
+/* Switches by name: "nc" columns a GEMV program takes (FE_BF16_NC; -1 = by the shape), "raster_group" (FE_BF16_GROUP;
+ * -1 = by the shape), "gemm_splits" (FE_GEMM_SPLITS). Read from the environment once, at load; no call reads it later. */
+int fe_bf16_kernels_set_option(fe_bf16_kernels *k, const char *name, int32_t value);
 
 /* fe_gemv_bf16 / fe_gemv_bf16_kw (gemm.rs:172-262): m <= 8 rows. One kernel family here: a program takes 1, 2, 4
  * or 8 columns by the width of the linear and the row count (model.rs:316-322 picks between the two kernels by the shape), and a row's bits

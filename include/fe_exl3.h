@@ -36,8 +36,11 @@ typedef struct {
     uint32_t strips;
 } fe_exl3_view;
 
-/* Launch plan (Plan, crates/fe-exl3/src/linear.rs:33-43): sk K splits per 128-column block; wk, ver, occ are kept for
- * the reference's plan strings ("sk,wk[,ver[,occ]]") and recorded, the gfx950 kernels use one form (256 threads). */
+/* Launch plan (Plan, crates/fe-exl3/src/linear.rs:33-43), the reference's plan strings "sk,wk[,ver[,occ]]". The gfx950
+ * decode GEMV deals 128-channel x 128-column units of the tensor to its programs in equal contiguous runs; a plan says how
+ * many programs. ver 1 (the reference's meaning): sk programs per 128-column block, i.e. sk K splits (needs k / 64
+ * divisible by sk). ver 2, 3 (what fe_exl3_plan_for returns): occ programs per CU, each a run of at least wk units; sk then
+ * records the K splits per column block this amounts to. ver 4: sk programs in all (any partition: tests and tuners). */
 typedef struct {
     uint32_t sk, wk, ver, occ;
 } fe_exl3_plan;
@@ -50,9 +53,17 @@ typedef struct fe_exl3_workspace fe_exl3_workspace; /* Workspace, crates/fe-exl3
  * crates/fe-exl3/src/gpu/mod.rs:88-93). */
 int fe_exl3_kernels_load(fe_exl3_kernels **out);
 int fe_exl3_kernels_destroy(fe_exl3_kernels *k);
+/* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
+ * "fused_rot" 0/1 (FE_EXL3_NO_FUSED_ROT), "fused_rot_pairs" (FE_EXL3_FUSED_ROT_PAIRS), "group" 0/1 (FE_EXL3_NO_GROUP),
+ * "hat_rows" (FE_EXL3_HAT_ROWS; 0 = never), "lds_pad" 0/1 (FE_EXL3_NO_LDS_PAD), "gemm_group_m" (FE_EXL3_GROUP),
+ * "gemm_splits" (FE_GEMM_SPLITS). forward() reads no environment variable; tests and tuners flip a switch here. Not for
+ * use while launches with this handle are being issued from another thread. No counterpart in the reference, which reads
+ * its switches (FE_EXL3_NOSPLIT, FE_EXL3_UNTUNED, ...) from the environment at plan time. */
+int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t value);
 
-/* Linear::plan_for (crates/fe-exl3/src/linear.rs:217-233): `blocks` is the program target (4 per CU is the default,
- * default_blocks linear.rs:132-134). Honours FE_EXL3_NOSPLIT=1 / FE_EXL3_SPLIT=0. */
+/* Linear::plan_for (crates/fe-exl3/src/linear.rs:217-233): the tuned plan of the shape where the table has one for this
+ * CU count (plans::tuned; FE_EXL3_UNTUNED=1 skips the table), else the rule: `blocks` is the program target (4 per CU is the
+ * default, default_blocks linear.rs:132-134), rounded to whole programs per CU. Honours FE_EXL3_NOSPLIT=1 / FE_EXL3_SPLIT=0. */
 int fe_exl3_plan_for(uint32_t k, uint32_t n, uint32_t bits, uint32_t blocks, fe_exl3_plan *out);
 /* Plan::parse "sk,wk[,ver[,occ]]" (linear.rs:47-55). */
 int fe_exl3_plan_parse(const char *s, fe_exl3_plan *out);

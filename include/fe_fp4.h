@@ -24,6 +24,11 @@ typedef struct fe_fp4_workspace fe_fp4_workspace; /* Workspace, crates/fe-fp4/sr
  * FE_FP4_GROUP sets the raster group height in row tiles (default 8, 0 = all). */
 int fe_fp4_kernels_load(fe_fp4_kernels **out);
 int fe_fp4_kernels_destroy(fe_fp4_kernels *k);
+/* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
+ * "group_m" (FE_FP4_GROUP), "gemv" 0/1 (FE_FP4_NO_GEMV), "gemv_sk" (FE_FP4_GEMV_SK; 0 = automatic), "xcd" -1/0/1
+ * (FE_FP4_XCD), "fp8_f16" 0/1 (FE_FP8_F16), "gemm_splits" (FE_GEMM_SPLITS). forward() reads no environment variable. No
+ * counterpart in the reference (its FE_FP4_GROUP is read at load too, crates/fe-fp4/src/lib.rs:31-32, 68). */
+int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value);
 
 /* HostLinear::upload (lib.rs:425-440) of an NVFP4 linear already fused on the host: codes [n][k/2], scales row-major
  * [n][k/16] (e4m3), alpha[n] = max(input_scale) * weight_scale_2 of the column's part, g = 1 / max(input_scale). */

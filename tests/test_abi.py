@@ -113,21 +113,21 @@ def test_plans():
     assert Plan.parse("2,8") == Plan(2, 8, 1, 0)
     assert Plan.parse("10,4,9,2") == Plan(10, 4, 9, 2)
     assert Plan.parse("x") is None
-    # every plan divides the K range into whole load steps of 64 channels (at least 8 a program, fewer only where K is
-    # shorter than 16 of them) and, among the split counts that do, takes the one whose program count is closest to the
-    # target as a ratio
-    import math
-    for k, n in [(5120, 17408), (17408, 5120), (5120, 5120), (5120, 1024), (128, 128), (1024, 256), (512, 384)]:
-        for blocks in (256, 704, 1024):
-            p = Linear.plan_for(k, n, 4, blocks)
-            steps = k // 64
-            least = min(8, max(2, steps // 2))
-            assert steps % p.sk == 0 and steps // p.sk >= min(least, steps) and p.ver in (1, 3)
-            miss = lambda d: abs(math.log(n // 128 * d / blocks))
-            fits = [d for d in range(1, steps + 1) if steps % d == 0 and steps // d >= least] or [1]
-            assert miss(p.sk) <= min(miss(d) for d in fits) + 1e-12
-    assert Linear.plan_for(5120, 17408, 4, 704).sk == 5 and Linear.plan_for(17408, 5120, 4, 704).sk == 17
-    assert Linear.plan_for(5120, 5120, 4, 704).sk == 10 and Linear.plan_for(5120, 1024, 4, 704).sk == 10
+    # plan_for: whole programs per CU (the target `blocks` rounded, 1..5 a CU; 256 CUs where no device is bound), runs
+    # of at least wk units of 128 channels x 128 columns, never more programs than that leaves; sk records the K splits
+    # per column block this amounts to. Shapes in the tuned table take its occ and wk instead.
+    os.environ["FE_EXL3_UNTUNED"] = "1"
+    try:
+        for k, n in [(5120, 17408), (17408, 5120), (5120, 5120), (5120, 1024), (128, 128), (1024, 256), (512, 384)]:
+            for blocks in (256, 704, 1024, 0):
+                p = Linear.plan_for(k, n, 4, blocks)
+                occ = min(5, max(1, (blocks + 128) // 256)) if blocks else 4
+                units, nb = (k // 128) * (n // 128), n // 128
+                programs = max(1, min(occ * 256, units // p.wk))
+                assert (p.ver, p.occ, p.wk) == (3, occ, 4) and p.sk == -(-programs // nb)
+        assert Linear.plan_for(5120, 17408, 4, 1024).sk == 8 and Linear.plan_for(5120, 1024, 4, 1024).sk == 10
+    finally:
+        del os.environ["FE_EXL3_UNTUNED"]
     os.environ["FE_EXL3_NOSPLIT"] = "1"
     try:
         assert Linear.plan_for(5120, 1024, 4, 1024).sk == 1

@@ -66,7 +66,7 @@ def call(torch, fn, kern, x, w, m, n, ldy=None, res=None, rows_alloc=None, lda=N
 
 @pytest.mark.parametrize("n,k,m", [(256, 512, 1), (1024, 1024, 3), (2048, 5120, 8), (96, 1024, 5), (48, 256, 1),
                                    (520, 768, 2), (1032, 2048, 7), (512, 512, 4), (528, 512, 6)])
-def test_gemv(env, oracle, monkeypatch, n, k, m):
+def test_gemv(env, oracle, n, k, m):
     torch, bf16, kern = env
     xb, wb = operands(n, k, m, 7 + n)
     x, w = dev_u16(torch, xb), dev_u16(torch, wb)
@@ -78,11 +78,11 @@ def test_gemv(env, oracle, monkeypatch, n, k, m):
     for r in {0, m - 1}:
         alone = call(torch, bf16.gemv, kern, x[r:r + 1].contiguous(), w, 1, n)
         assert np.array_equal(alone[0], got[r])
-    # nor on how many columns a program takes (FE_BF16_NC overrides the library's choice)
+    # nor on how many columns a program takes (the "nc" option overrides the library's choice)
     for nc in (1, 2, 4, 8):
-        monkeypatch.setenv("FE_BF16_NC", str(nc))
+        kern.set_option("nc", nc)
         assert np.array_equal(call(torch, bf16.gemv, kern, x, w, m, n), got), nc
-    monkeypatch.delenv("FE_BF16_NC")
+    kern.set_option("nc", -1)
     # residual: bf16(bf16(sum) + res), exact given the sums
     rb = bits(np.random.default_rng(3).normal(size=(m + 2, n)))
     with_res = call(torch, bf16.gemv, kern, x, w, m, n, res=dev_u16(torch, rb))
@@ -91,7 +91,7 @@ def test_gemv(env, oracle, monkeypatch, n, k, m):
 
 @pytest.mark.parametrize("n,k,m,lda", [(256, 512, 200, 512), (520, 768, 300, 776), (1024, 1024, 700, 1024), (96, 256, 33, 256),
                                        (768, 2048, 1, 2048)])
-def test_gemm_whole_and_cut(env, oracle, monkeypatch, n, k, m, lda):
+def test_gemm_whole_and_cut(env, oracle, n, k, m, lda):
     torch, bf16, kern = env
     xb, wb = operands(n, k, m, 11 + n, lda=lda)
     x, w = dev_u16(torch, xb), dev_u16(torch, wb)
@@ -101,9 +101,9 @@ def test_gemm_whole_and_cut(env, oracle, monkeypatch, n, k, m, lda):
 
     cut = run()
     assert np.array_equal(cut, run())  # deterministic
-    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    kern.set_option("gemm_splits", 1)
     whole = run()
-    monkeypatch.delenv("FE_GEMM_SPLITS")
+    kern.set_option("gemm_splits", 8)
     want, acc = oracle.bf16_linear_ref(xb[:, :k], wb)
     close(cut, acc)
     close(whole, acc)

@@ -140,24 +140,24 @@ def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
 
 
 @pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
-@pytest.mark.parametrize("ver", [1, 2])
+@pytest.mark.parametrize("ver", [1, 3])
 def test_gemv_all_bit_widths(env, oracle, bits, ver):
-    """ver 1: split-K programs per column block; ver 2: rows 1..16 streamed over the whole tensor."""
+    """ver 1: sk programs per column block; ver 3: occ programs per CU over the whole tensor."""
     torch, exl3, kern = env
     from ferrite_amd import synth
     t = synth.exl3_tensor(512, 256, bits, 20 + bits)
     check_linear(env, oracle, t, exl3.Plan(2, 4, ver, 2), strips=True, rows_list=[1, 5, 16, 17, 64])
 
 
-@pytest.mark.parametrize("programs,strips", [(1, True), (5, True), (7, False), (13, True), (48, False), (1000, True)])
-def test_streamed_gemv_any_partition(env, oracle, programs, strips, monkeypatch):
-    """The streamed GEMV cuts the tensor's 48 work units (3 column blocks x 16 load steps) into runs of any length:
-    runs that start and end inside a block, cover whole blocks, or are a single unit."""
+@pytest.mark.parametrize("programs,strips", [(1, True), (2, False), (5, True), (7, False), (13, True), (24, False), (1000, True)])
+def test_gemv_any_partition(env, oracle, programs, strips):
+    """The GEMV cuts the tensor's 24 work units (3 column blocks x 8 blocks of 128 channels) into runs of any length: runs
+    that start and end inside a column block, cover whole blocks or several, or are a single unit (plan ver 4: that many
+    programs; more programs than units: one a unit)."""
     torch, exl3, kern = env
     from ferrite_amd import synth
-    monkeypatch.setenv("FE_EXL3_PROGRAMS", str(programs))
     t = synth.exl3_tensor(1024, 384, 4, 77)
-    check_linear(env, oracle, t, exl3.Plan(4, 4, 2, 2), strips=strips, rows_list=[1, 2, 5, 8, 9, 16])
+    check_linear(env, oracle, t, exl3.Plan(programs, 4, 4, 0), strips=strips, rows_list=[1, 2, 5, 8, 9, 16, 17, 64])
 
 
 @pytest.mark.parametrize("sk,strips", [(1, True), (1, False), (4, True), (8, False), (16, True)])
@@ -182,10 +182,10 @@ def test_plan_for_default_and_determinism_with_shared_workspace(env, oracle):
     torch, exl3, kern = env
     from ferrite_amd import synth
     a = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, 256, 4, 1)), exl3.default_blocks(exl3.cu_count()))
-    b = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(512, 384, 3, 2)), exl3.default_blocks(exl3.cu_count()))
+    b = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, 384, 3, 2)), exl3.default_blocks(exl3.cu_count()))
     assert a.plan.sk > 1 and b.plan.sk > 1
     ws = exl3.Workspace([a, b], 16)
-    xa, xb = dev_u16(torch, synth.activations(16, 1024, 3)), dev_u16(torch, synth.activations(16, 512, 4))
+    xa, xb = dev_u16(torch, synth.activations(16, 1024, 3)), dev_u16(torch, synth.activations(16, 1024, 4))
     ya = torch.empty((16, 256), dtype=torch.float32, device="cuda")
     yb = torch.empty((16, 384), dtype=torch.float32, device="cuda")
     first = None
@@ -284,8 +284,8 @@ def test_argument_errors_are_results_not_crashes(env):
     assert torch.isfinite(y[:4]).all()
 
 
-def test_prefill_gemm_tiles_cut_or_whole(env, oracle, monkeypatch):
-    """Several 256 x 256 tiles with an odd count of 128-column blocks: computed whole (FE_GEMM_SPLITS=1) and cut along K
+def test_prefill_gemm_tiles_cut_or_whole(env, oracle):
+    """Several 256 x 256 tiles with an odd count of 128-column blocks: computed whole (option gemm_splits = 1) and cut along K
     with the reduce kernel (the default for a nearly empty last round)."""
     torch, exl3, kern = env
     from ferrite_amd import synth
@@ -307,8 +307,9 @@ def test_prefill_gemm_tiles_cut_or_whole(env, oracle, monkeypatch):
 
     cut = run()
     assert np.array_equal(cut, run())
-    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    kern.set_option("gemm_splits", 1)
     whole = run()
+    kern.set_option("gemm_splits", 8)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     rms = np.sqrt((ref ** 2).mean())
     assert np.abs(cut - ref).max() / rms < 1e-4
@@ -326,27 +327,26 @@ def test_tuner_returns_a_fitting_plan(env):
     from ferrite_amd import synth
     t = synth.exl3_tensor(1024, 512, 4, 3)
     best, table = exl3.tune(kern, t, iters=5, copies_bytes=1 << 20)
-    assert (t.k // 64) % best.sk == 0 and len(table) >= 4
+    assert best.ver == 3 and best.occ in (2, 3, 4, 5) and len(table) >= 4
     assert all(us1 > 0 and us16 > 0 for _, us1, us16 in table)
     lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), best)
-    assert lin.plan.sk == best.sk
+    assert lin.plan.occ == best.occ
 
 
-@pytest.mark.parametrize("k,sk,fits", [(1024, 1, True), (1024, 4, True), (2048, 16, True), (1024, 8, True), (1024, 16, False),
-                                       (1280, 2, True), (1280, 4, False)])
-def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, monkeypatch):
-    """forward() for few rows is one launch when every program's K range is whole 128-element blocks (the GEMV rotates
-    its own input and leaves it in the workspace), two launches otherwise. Both give the same bits, in y and in the
-    workspace's rotated input, for bf16 and f32 inputs."""
+@pytest.mark.parametrize("k,sk", [(1024, 1), (1024, 4), (2048, 16), (1024, 8), (1024, 16), (1280, 2), (1280, 4)])
+def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk):
+    """forward() for few rows is one launch (the GEMV rotates its own input and leaves it in the workspace) while a
+    program's share of the rotation stays small, two launches otherwise (and always with the "fused_rot" option off). Both
+    give the same bits, in y and in the workspace's rotated input, for bf16 and f32 inputs."""
     torch, exl3, kern = env
     from ferrite_amd import _lib, synth
     from ferrite_amd._lib import check
-    assert ((k // 64 // sk) % 2 == 0) == fits
     t = synth.exl3_tensor(k, 384, 4, 70 + sk)
     lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(sk=sk, wk=1, ver=1, occ=2))
-    # one launch when the K ranges fit and a program's share of the rotation stays small (rows x 128-blocks <= 32)
+    # one launch while a program's share of the rotation stays small: rows x 128-channel blocks of its run <= 16
+    programs = min(3 * sk, 3 * (k // 128))
     for rows in (1, 4, 7, 16, 33, 64, 65):
-        assert lin.forward_is_one_launch(rows) == (fits and rows <= 64 and rows * (k // 128 // sk) <= 32), rows
+        assert lin.forward_is_one_launch(rows) == (rows <= 64 and rows * -(-(3 * (k // 128)) // programs) <= 16), rows
     ws = exl3.Workspace([lin], 64)
     xb = synth.activations(64, k, 8, outliers=True)
     xd = dev_u16(torch, xb)
@@ -355,14 +355,13 @@ def test_forward_rotates_inside_the_gemv_or_before_it(env, oracle, k, sk, fits, 
         for x, xdt in ((xd, exl3.Dtype.Bf16), (xf, exl3.Dtype.F32)):
             out = {}
             for mode in ("fused", "separate"):
-                if mode == "separate":
-                    monkeypatch.setenv("FE_EXL3_NO_FUSED_ROT", "1")
+                kern.set_option("fused_rot", 0 if mode == "separate" else 1)
                 check(_lib.lib().fe_hip_memset_d8(ws.xh_ptr, 0x7e, 64 * k * 2, None))  # fp16 NaNs: stale inputs would show
                 y = torch.full((65, lin.n), float("nan"), dtype=torch.float32, device="cuda")
                 lin.forward(x, xdt, y, exl3.Dtype.F32, rows, ws)
                 torch.cuda.synchronize()
                 out[mode] = (y.cpu().numpy(), ws.xh(rows, k))
-                monkeypatch.delenv("FE_EXL3_NO_FUSED_ROT", raising=False)
+                kern.set_option("fused_rot", 1)
             assert np.array_equal(out["fused"][1], out["separate"][1]), (rows, xdt)
             assert np.array_equal(out["fused"][0][:rows].view(np.uint32), out["separate"][0][:rows].view(np.uint32)), (rows, xdt)
             assert np.isnan(out["fused"][0][rows:]).all()
@@ -414,7 +413,7 @@ def test_forward_on_swiglu_of_gate_and_up(env, k, sk):
 
 @pytest.mark.parametrize("bits,k,ns,sks", [(4, 1024, (384, 128, 256), (2, 4, 1)), (3, 1280, (256, 640), (2, 1)),
                                            (5, 1024, (128, 128, 384, 256), (8, 1, 2, 4)), (4, 2048, (512, 384), (16, 4))])
-def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sks, monkeypatch):
+def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sks):
     """Linears of one input (q, k, v; gate, up) in one GEMV launch: every member's programs are those of its own launch,
     so each output has the bits of the member's forward(), for every row count, input and output type, with the input
     rotated inside the GEMV (one launch) or by one launch for all members (two). Groups that cannot share a launch
@@ -457,13 +456,13 @@ def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sk
     torch.cuda.synchronize()
     assert all(torch.equal(a, b) for a, b in zip(y1, y2))
     # member by member: switched off, one member alone, a member of other bits, a workspace made for one small linear
-    monkeypatch.setenv("FE_EXL3_NO_GROUP", "1")
+    kern.set_option("group", 0)
     assert exl3.forward_group_launches(lins, 1, ws) == 0
     y3 = [torch.zeros((4, n), dtype=torch.float32, device="cuda") for n in ns]
     exl3.forward_group(lins, xd, exl3.Dtype.Bf16, y3, exl3.Dtype.F32, 4, ws)
     torch.cuda.synchronize()
     assert all(torch.equal(a, b) for a, b in zip(y1, y3))
-    monkeypatch.delenv("FE_EXL3_NO_GROUP")
+    kern.set_option("group", 1)
     assert exl3.forward_group_launches(lins[:1], 1, ws) == 0
     other = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, 128, bits + 1, 5)), exl3.Plan(sk=1, wk=1, ver=1, occ=2))
     mixed = [lins[0], other]
@@ -479,11 +478,11 @@ def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sk
 
 @pytest.mark.parametrize("bits,n,strips", [(2, 384, True), (3, 256, False), (4, 640, True), (5, 384, False), (6, 128, True),
                                            (8, 384, True), (4, 2304, True), (3, 4224, False)])
-def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracle, bits, n, strips, monkeypatch):
+def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracle, bits, n, strips):
     """Many rows: the trellis is decoded once into fp16 tiles (the GEMM's own LDS images) and the GEMM copies them instead
     of decoding per output tile row. Same fragments and MFMA order, so with whole tiles the same bits in every output
     mode; the two forms walk the tiles in different orders, so with a last round cut along K other tiles are the cut
-    ones and those differ by the order of their f32 sums. FE_EXL3_HAT_ROWS moves the row count from which this form
+    ones and those differ by the order of their f32 sums. The "hat_rows" option moves the row count from which this form
     runs (0: never). 2304 and 4224 columns: 9 and 17 column tiles, dealt to the XCDs in bands of 8."""
     torch, exl3, kern = env
     from ferrite_amd import synth
@@ -491,7 +490,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     t = synth.exl3_tensor(1024, n, bits, 90 + bits)
     xd = dev_u16(torch, synth.activations(m, t.k, 6, outliers=True))
     lin = exl3.Linear.new(kern, exl3.DeviceExl3(t, strips), 256)
-    monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+    kern.set_option("hat_rows", 65)
     ws = exl3.Workspace([lin], m)  # created for the decoded form
 
     def run(rows, dt, torch_dt, pre):
@@ -501,14 +500,13 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
         return y.view(torch.int16 if torch_dt == torch.bfloat16 else torch.int32).cpu().numpy()
 
     for splits in (None, "1"):
-        if splits:
-            monkeypatch.setenv("FE_GEMM_SPLITS", splits)
+        kern.set_option("gemm_splits", int(splits) if splits else 8)
         for rows in (65, 300, 600):
             for dt, tdt, pre in ((exl3.Dtype.F32, torch.float32, float("nan")), (exl3.Dtype.Bf16, torch.bfloat16, 7.0),
                                  (exl3.Dtype.Bf16Add, torch.bfloat16, 1.5), (exl3.Dtype.F32Add, torch.float32, 0.25)):
-                monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+                kern.set_option("hat_rows", 65)
                 tiles = run(rows, dt, tdt, pre)
-                monkeypatch.setenv("FE_EXL3_HAT_ROWS", "0")
+                kern.set_option("hat_rows", 0)
                 fused = run(rows, dt, tdt, pre)
                 if splits:
                     assert np.array_equal(tiles, fused), (splits, rows, dt)
@@ -518,18 +516,19 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
                     rms = np.sqrt((b ** 2).mean())
                     assert np.all(np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * rms), (rows, dt)
                 assert (tiles[rows:] == tiles[m]).all()  # rows past `rows` keep the prefill
-    monkeypatch.delenv("FE_GEMM_SPLITS", raising=False)
+    kern.set_option("gemm_splits", 8)
     # and against the oracle
-    monkeypatch.setenv("FE_EXL3_HAT_ROWS", "65")
+    kern.set_option("hat_rows", 65)
     y = torch.zeros((m, t.n), dtype=torch.float32, device="cuda")
     lin.forward(xd, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
     torch.cuda.synchronize()
     o = to_oracle(oracle, t)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
+    kern.set_option("hat_rows", 513)
 
 
-def test_prefill_over_kept_decoded_weights(env, oracle, monkeypatch):
+def test_prefill_over_kept_decoded_weights(env, oracle):
     """keep_decoded: the fp16 tiles stay with the linear, every call above 64 rows runs the GEMM over them (no decode
     launch, any workspace). Whole tiles have the bits of the decoding GEMM; decode-sized calls are untouched."""
     torch, exl3, kern = env
@@ -548,13 +547,13 @@ def test_prefill_over_kept_decoded_weights(env, oracle, monkeypatch):
         assert np.isnan(out[rows:]).all()
         return out[:rows]
 
-    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    kern.set_option("gemm_splits", 1)
     before = {rows: run(rows) for rows in (1, 16, 64, 65, 300)}
     lin.keep_decoded()
     lin.keep_decoded()  # a second call keeps what is there
     for rows, want in before.items():
         assert np.array_equal(run(rows).view(np.uint32), want.view(np.uint32)), rows
-    monkeypatch.delenv("FE_GEMM_SPLITS")
+    kern.set_option("gemm_splits", 8)
     cut = run(300)  # a last round cut along K: other tiles are the cut ones, sums in another order
     rms = np.sqrt((before[300].astype(np.float64) ** 2).mean())
     assert np.abs(cut.astype(np.float64) - before[300]).max() / rms < 1e-4

@@ -101,8 +101,8 @@ def test_fp4_linear(env, oracle, n, k, m, input_scale):
     assert np.array_equal(y3.view(torch.int16).cpu().numpy().view(np.uint16), yg)
 
 
-def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
-    """Several 256 x 256 output tiles with an odd count of 128-row weight tiles, computed whole (FE_GEMM_SPLITS=1), cut
+def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle):
+    """Several 256 x 256 output tiles with an odd count of 128-row weight tiles, computed whole (option gemm_splits = 1), cut
     along K with the reduce kernel (the default for a nearly empty last round), and from a row-major device view."""
     torch, fp4, kern = env
     from ferrite_amd import synth
@@ -123,12 +123,12 @@ def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
 
     cut = run(lin)
     assert np.array_equal(cut, run(lin))  # deterministic
-    monkeypatch.setenv("FE_GEMM_SPLITS", "1")
+    kern.set_option("gemm_splits", 1)
     whole = run(lin)
     view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), torch.from_numpy(host.sf).cuda(),
                                       torch.from_numpy(host.alpha).cuda(), host.g)
     assert np.array_equal(run(view), whole)
-    monkeypatch.delenv("FE_GEMM_SPLITS")
+    kern.set_option("gemm_splits", 8)
     assert np.array_equal(run(view), cut)
     # cut and whole differ only by the order of the f32 sums: at most one bf16 step
     a, b = bf16_to_f32(cut).astype(np.float64), bf16_to_f32(whole).astype(np.float64)
@@ -149,8 +149,8 @@ def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle, monkeypatch):
     assert np.array_equal(got, want)
 
 
-def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
-    """Up to 64 rows run the weight-read-bound GEMV (up to 48 rows a pass, K cut over several programs); FE_FP4_NO_GEMV
+def test_fp4_gemv_agrees_with_the_gemm(env, oracle):
+    """Up to 64 rows run the weight-read-bound GEMV (up to 48 rows a pass, K cut over several programs); option gemv = 0
     sends the same rows through the GEMM. Both sum the same exact products in f32, in different orders; within the GEMV a
     row's bits do not depend on the rows around it."""
     torch, fp4, kern = env
@@ -178,9 +178,9 @@ def test_fp4_gemv_agrees_with_the_gemm(env, oracle, monkeypatch):
         assert np.array_equal(gemv, run(lin)) and np.array_equal(gemv, run(view))
         with_res = run(lin, res)
         assert np.array_equal(with_res, bf16_bits(bf16_to_f32(gemv) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m])))
-        monkeypatch.setenv("FE_FP4_NO_GEMV", "1")
+        kern.set_option("gemv", 0)
         gemm = run(lin)
-        monkeypatch.delenv("FE_FP4_NO_GEMV")
+        kern.set_option("gemv", 1)
         a, b = bf16_to_f32(gemv).astype(np.float64), bf16_to_f32(gemm).astype(np.float64)
         assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all()
     # the same rows alone, in a pass of 16, 32 or 48 rows, and as the second pass of 64

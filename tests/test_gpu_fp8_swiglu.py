@@ -30,7 +30,7 @@ def bf16_bits(x):
 
 @pytest.mark.parametrize("n,k,m,input_scale", [(256, 512, 200, 0.05), (128, 1024, 1, 0.02), (640, 256, 300, 0.1),
                                                (384, 1152, 520, 0.05)])
-def test_fp8_linear(env, oracle, n, k, m, input_scale, monkeypatch):
+def test_fp8_linear(env, oracle, n, k, m, input_scale):
     torch, fp4, kern = env
     from ferrite_amd import synth
     host = synth.fp8_linear(n, k, 17, input_scale=input_scale, weight_scale=0.003)
@@ -76,13 +76,13 @@ def test_fp8_linear(env, oracle, n, k, m, input_scale, monkeypatch):
     assert np.array_equal(out2[:m], bf16_bits(bf16_to_f32(yg) + bf16_to_f32(res[:m]))) and np.array_equal(out2[m], res[m])
     assert np.array_equal(y3.view(torch.int16).cpu().numpy().view(np.uint16), yg)
 
-    # the default runs the 8-bit matrix instruction over the codes; FE_FP8_F16=1 the fp16 expansion of the same codes on
+    # the default runs the 8-bit matrix instruction over the codes; option fp8_f16 = 1 the fp16 expansion of the same codes on
     # the 16-bit instruction: the same exact products, summed in f32 in another order
-    monkeypatch.setenv("FE_FP8_F16", "1")
+    kern.set_option("fp8_f16", 1)
     y4 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     lin.forward(kern, ws, y4, n, xd, k, m)
     torch.cuda.synchronize()
-    monkeypatch.delenv("FE_FP8_F16")
+    kern.set_option("fp8_f16", 0)
     a = bf16_to_f32(y4.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
     b = bf16_to_f32(yg).astype(np.float64)
     assert np.all(np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * np.abs(b).max())

@@ -20,8 +20,8 @@ def test_forward_calls_replay_from_a_graph():
     lib, check = _lib.lib(), _lib.check
     kern, fk = exl3.Kernels.load(), fp4.Kernels.load()
     t = synth.exl3_tensor(1024, 384, 4, 5)
-    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 64)  # few programs per block: the K range is split
-    streamed = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(4, 4, 2, 2))
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 64)  # column blocks shared by several programs
+    streamed = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(7, 4, 4, 0))  # 7 uneven runs
     flin = synth.fp4_linear(384, 1024, 6).upload()
     # two more linears of the same input: with `lin` a grouped launch (the argument block is copied at capture)
     pair = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, n, 4, 30 + n)), 64) for n in (256, 128)]

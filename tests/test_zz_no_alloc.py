@@ -71,11 +71,12 @@ def test_sizes_beyond_the_array_are_errors():
         with pytest.raises(FeError) as e:
             lin.forward_static(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, rows)
         assert e.value.code == 10002  # FE_ERR_WORKSPACE
-    # partial sums of 16 splits x 16 rows x 16384 columns = 16 MiB: more than the array holds
-    t = synth.exl3_tensor(1024, 16384, 2, 15)
-    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(16))
+    # partial sums of 2048 programs over 256 column blocks at 16 rows: 2304 slots x 16 x 512 B = 18 MiB, more than the
+    # array holds
+    t = synth.exl3_tensor(1024, 32768, 2, 15)
+    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(8))
     x = torch.zeros((16, 1024), dtype=torch.bfloat16, device="cuda")
-    y = torch.zeros((16, 16384), dtype=torch.float32, device="cuda")
+    y = torch.zeros((16, 32768), dtype=torch.float32, device="cuda")
     with pytest.raises(FeError) as e:
         lin.forward_static(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 16)
     assert e.value.code == 10002 and "partial sums" in str(e.value)
