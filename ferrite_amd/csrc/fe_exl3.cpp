@@ -510,8 +510,11 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     // Exactly occ programs a CU: the dispatcher fills a CU as far as registers and LDS allow (5 programs) before it moves
     // on, which would leave CUs empty while others hold 5; an LDS request that fits occ times into the CU's 160 KB, and
     // not occ + 1 times, makes the CUs take occ each.
+    // (several linears: the most programs per CU any of them asks for)
     const fe_exl3_kernels *kern = ls[0]->kern;
-    if (const uint32_t occ = ls[0]->plan.occ; occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
+    uint32_t occ = 0;
+    for (size_t i = 0; i < count; i++) occ = std::max(occ, ls[i]->plan.occ);
+    if (occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
     uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld, inv_spb = 0xffffffffu / (k / 64);
     fe_devptr_t x = in.x, x2 = in.x2;
     void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb};
@@ -640,7 +643,7 @@ static bool group_fits(const fe_exl3_linear *const *ls, size_t count, uint32_t r
     bool f = true;
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = ls[i];
-        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern || l->plan.occ != ls[0]->plan.occ) return false;
+        if (!l || l->k != ls[0]->k || l->bits != ls[0]->bits || l->kern != ls[0]->kern) return false;
         f = f && fused_rotation_fits(l, rows);
         z += job_z(l, rows);
         nb += l->n / 128;

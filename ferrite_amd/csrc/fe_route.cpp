@@ -88,8 +88,9 @@ static int linear_forward(const fe_route_linear *l, const fe_route_ctx *c, uint3
         }
     }
     if (l->p && c->fp4()) return fe_fp4_linear_forward(l->p, c->fk, c->s, c->fws, y, ldy, x, lda, m, res);
-    if (l->q && c->x3() && m > FE_X3_ROWS) {
-        // no prompt weights: every row through the trellis linear (model.rs:305-309)
+    if (!l->w && l->q && c->x3() && m > FE_X3_ROWS) {
+        // no prompt weights and no bf16 weights: every row through the trellis linear (model.rs:305-309); with bf16
+        // weights beside the trellis the prompt rows take the bf16 GEMM below, as in the reference
         if (lda != l->k || ldy != l->n) return fail(FE_ERR_ARG, fn, l->name + ": the trellis linear needs lda == k and ldy == n");
         uint32_t ws_rows = 0;
         FE_TRY(fe_exl3_workspace_xh(c->xws, nullptr, &ws_rows, nullptr));

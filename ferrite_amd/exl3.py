@@ -341,13 +341,48 @@ class Workspace:
             self.h = None
 
 
-def tune(kern: Kernels, t: Exl3Tensor, iters: int = 50, w16: float = 0.25, copies_bytes: int = 600 << 20,
+def _graph_us(fn, inner: int, reps: int = 5) -> float:
+    """Microseconds per call of fn(stream) with `inner` calls captured into one HIP graph and the graph replayed: the
+    launches run back to back as they do under a captured decode step, with no host time between them."""
+    lib = _lib.lib()
+    s, a, b, g = C.c_void_p(), C.c_void_p(), C.c_void_p(), C.c_void_p()
+    check(lib.fe_hip_stream_create(C.byref(s)))
+    check(lib.fe_hip_event_create(C.byref(a)))
+    check(lib.fe_hip_event_create(C.byref(b)))
+    try:
+        fn(s)
+        check(lib.fe_hip_stream_sync(s))
+        check(lib.fe_hip_graph_begin(s))
+        for _ in range(inner):
+            fn(s)
+        check(lib.fe_hip_graph_end(s, C.byref(g)))
+        check(lib.fe_hip_graph_launch(g, s))
+        best = float("inf")
+        for _ in range(3):
+            check(lib.fe_hip_event_record(a, s))
+            for _ in range(reps):
+                check(lib.fe_hip_graph_launch(g, s))
+            check(lib.fe_hip_event_record(b, s))
+            check(lib.fe_hip_event_sync(b))
+            ms = C.c_float()
+            check(lib.fe_hip_event_elapsed_ms(C.byref(ms), a, b))
+            best = min(best, ms.value * 1e3 / (reps * inner))
+        check(lib.fe_hip_graph_destroy(g))
+        return best
+    finally:
+        lib.fe_hip_event_destroy(a)
+        lib.fe_hip_event_destroy(b)
+        lib.fe_hip_stream_destroy(s)
+
+
+def tune(kern: Kernels, t: Exl3Tensor, iters: int = 5, w16: float = 0.25, copies_bytes: int = 600 << 20,
          occs=(2, 3, 4, 5), min_units=(2, 4, 8)):
     """Times every candidate plan on one tensor shape at 1 and 16 rows and returns (best plan, table), the table a list of
     (plan, us at 1 row, us at 16 rows) sorted by us1 + w16 * us16 (the measure of
     crates/fe-exl3/src/bin/exl3-tune.rs:75-118). Launches cycle over enough copies of the weights that none is served
-    from a cache. Candidates: occ programs per CU, each a run of at least wk units of 128 channels x 128 columns; plans
-    that come to the same program count are timed once."""
+    from a cache and are replayed from a graph, `iters` replays of two passes over the copies. Candidates: occ programs
+    per CU, each a run of at least wk units of 128 channels x 128 columns; plans that come to the same program count are
+    timed once."""
     import torch
     copies = max(2, min(64, copies_bytes // max(1, t.trellis_bytes()) + 1))
     devs = [DeviceExl3.upload_strips(t) for _ in range(copies)]
@@ -366,15 +401,12 @@ def tune(kern: Kernels, t: Exl3Tensor, iters: int = 50, w16: float = 0.25, copie
             ws = Workspace(lins[:1], 16)
             us = []
             for rows in (1, 16):
-                for lin in lins[:2]:
-                    lin.forward(x, Dtype.Bf16, y, Dtype.Bf16, rows, ws)
-                a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                a.record()
-                for i in range(iters):
-                    lins[i % copies].forward(x, Dtype.Bf16, y, Dtype.Bf16, rows, ws)
-                b.record()
-                torch.cuda.synchronize()
-                us.append(a.elapsed_time(b) * 1e3 / iters)
+                at = [0]
+
+                def fn(s):
+                    lins[at[0] % copies].forward(x, Dtype.Bf16, y, Dtype.Bf16, rows, ws, stream=s)
+                    at[0] += 1
+                us.append(_graph_us(fn, 2 * copies, iters))
             table.append((p, us[0], us[1]))
     table.sort(key=lambda e: e[1] + w16 * e[2])
     return table[0][0], table

@@ -46,7 +46,9 @@ int fe_route_ctx_set_x3_gemm(fe_route_ctx *c, int on);
  * Borrowed. */
 int fe_route_linear_create(fe_route_linear **out, const char *name, uint32_t n, uint32_t k, const fe_exl3_linear *q,
                            const fe_fp4_linear *p);
-/* Linear::w (model.rs:265): bf16 weights [n][k] on the device (0 = none), used where neither q nor p applies. Borrowed. */
+/* Linear::w (model.rs:265): bf16 weights [n][k] on the device (0 = none). They take the rows that neither the trellis GEMV
+ * (decode rows of a linear with q) nor p takes; a linear that holds q and w (the loader's bf16 + exl3_decode form,
+ * model.rs:664-684) never sends prompt rows back through the trellis (model.rs:305). Borrowed. */
 int fe_route_linear_set_bf16(fe_route_linear *l, fe_devptr_t w);
 int fe_route_linear_destroy(fe_route_linear *l);
 /* Linear::forward (model.rs:275-346): y (row stride ldy) = x (row stride lda) . W^T for m rows; with res (stride ldy):

@@ -96,8 +96,20 @@ def check(got, got_bf16, ref, f32_bound):
     assert (np.abs(got_bf16 - ref) / np.maximum(np.abs(ref), rms)).max() < 1e-2
 
 
-@pytest.mark.parametrize("shape,bits", [("qo", 4), ("kv", 4), ("gate_up", 3), ("gate_up", 4), ("gate_up", 5), ("down", 4),
-                                        ("lm_head", 6)])
+def end_to_end(oracle, layer, xd, rows, got_rows):
+    """The whole linear against the reference's f64 linear on the bf16 inputs themselves (crates/fe-exl3/src/cpu.rs:180-215)
+    for a subset of the rows: max |y - ref| / rms(ref). What separates the two is the fp16 rounding of the rotated inputs
+    (the reference's GPU path has it too) and f32 sums."""
+    t = layer.t
+    o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+    xb = xd.cpu().numpy().view(np.uint16)[rows]
+    x64 = (xb.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    ref = oracle.linear_f64(o, x64, threads=oracle.default_threads(16))
+    return np.abs(got_rows - ref).max() / np.sqrt((ref ** 2).mean())
+
+
+@pytest.mark.parametrize("shape,bits", [("qo", 4), ("kv", 4), ("gate_up", 3), ("gate_up", 4), ("gate_up", 5), ("down", 3),
+                                        ("down", 4), ("down", 5), ("lm_head", 6)])
 def test_exl3_decode_rows_at_full_size(env, oracle, shape, bits):
     torch, exl3, kern = env
     k, n = SHAPES[shape]
@@ -106,6 +118,8 @@ def test_exl3_decode_rows_at_full_size(env, oracle, shape, bits):
     for m in (1, 4, 8, 16):
         xd, xh, got, got_bf16, ws = run_rows(env, layer, m, 9)
         check(got, got_bf16, layer.reference(torch, xh, torch.float64), 1e-4)
+        if m == 1 and shape != "lm_head":  # end to end against the reference's CPU linear
+            assert end_to_end(oracle, layer, xd, [0], got[:1]) < 2e-3
         if m == 16:  # each row of the batch has the bits of the single-row call
             for r in (0, 7, 15):
                 y1 = torch.zeros((1, n), dtype=torch.float32, device="cuda")
@@ -174,15 +188,22 @@ def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
 
 
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
-def test_exl3_prefill_at_full_size(env, oracle, shape):
-    """M = 2048, 1 % outlier channels x20: the MFMA GEMM, including the tiles cut along K and the reduce kernel."""
+@pytest.mark.parametrize("m", [128, 300, 512, 2048])
+def test_exl3_prefill_at_full_size(env, oracle, shape, m):
+    """Prompt rows with 1 % outlier channels x20 through the MFMA GEMM, including the tiles cut along K and the reduce
+    kernel: 2048 rows run over tiles decoded once per call, 128, 300 and 512 rows (the chunks a prompt usually comes in)
+    decode inside the GEMM, at the real strides and with the K cut the launcher picks for one or two rows of output tiles.
+    Stage by stage against the GPU's own rotated input (1e-4 of the rms), and end to end against the reference's f64
+    linear on the bf16 inputs for the reference's row sample (crates/fe-fp4/src/bin/fp4-check.rs:96)."""
     torch, exl3, kern = env
     k, n = SHAPES[shape]
     layer = Layer(env, oracle, k, n, 4, 77)
-    xd, xh, got, got_bf16, ws = run_rows(env, layer, 2048, 11, outliers=True)
+    xd, xh, got, got_bf16, ws = run_rows(env, layer, m, 11, outliers=True)
     check(got, got_bf16, layer.reference(torch, xh, torch.float32), 1e-4)
-    again = run_rows(env, layer, 2048, 11, outliers=True)[2]
+    again = run_rows(env, layer, m, 11, outliers=True)[2]
     assert np.array_equal(again, got)  # deterministic
+    rows = sorted({0, 1, 17, 127, min(128, m - 1), m // 2, m - 1})
+    assert end_to_end(oracle, layer, xd, rows, got[rows]) < 2e-3
 
 
 @pytest.mark.parametrize("m", [1, 16, 2048])

@@ -164,6 +164,47 @@ def test_linear_without_prompt_weights(env):
         route.Linear("bad", HIDDEN, HIDDEN, q=e.q_down)
 
 
+def test_linear_with_trellis_and_bf16_weights(env):
+    """model.rs:305, 664-684: a linear that holds the trellis (q) and plain bf16 weights (w): decode rows take the trellis
+    GEMV, the prompt rows after them the bf16 linear, never the trellis again."""
+    e = env
+    torch, route = e.torch, e.route
+    from ferrite_amd import bf16
+    bk = bf16.Kernels.load()
+    wb = bf16_bits(np.random.default_rng(5).normal(size=(HIDDEN, INTER)) / 32)
+    w = dev_u16(torch, wb)
+    lin = route.Linear("down", HIDDEN, INTER, q=e.q_down, w=w)
+    c = e.ctx
+    c.set_bf16(bk)
+    try:
+        m, dec = 150, 5
+        x = dev_u16(torch, e.synth.activations(m, INTER, 9))
+        c.dec = dec
+        y = torch.zeros((m, HIDDEN), dtype=torch.bfloat16, device="cuda")
+        lin.forward(c, y, HIDDEN, x, INTER, m)
+        torch.cuda.synchronize()
+        got = bits(y)
+        assert np.array_equal(got[:dec], x3_direct(e, e.q_down, x, dec))
+        want = torch.zeros((m - dec, HIDDEN), dtype=torch.bfloat16, device="cuda")
+        bf16.forward(bk, want, HIDDEN, x[dec:], INTER, w, m - dec, dec=0)
+        torch.cuda.synchronize()
+        assert np.array_equal(got[dec:], bits(want))
+        # no decode rows announced: all 150 rows are prompt rows of the bf16 linear
+        c.dec = 0
+        lin.forward(c, y, HIDDEN, x, INTER, m)
+        allw = torch.zeros((m, HIDDEN), dtype=torch.bfloat16, device="cuda")
+        bf16.forward(bk, allw, HIDDEN, x, INTER, w, m, dec=0)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y), bits(allw))
+        # a small batch is all decode rows: the trellis
+        lin.forward(c, y, HIDDEN, x, INTER, 7)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits(y)[:7], x3_direct(e, e.q_down, x, 7))
+    finally:
+        c.dec = 0
+        c.set_bf16(None)
+
+
 def test_proj_places_parts_as_the_reference(env):
     e = env
     torch, route = e.torch, e.route

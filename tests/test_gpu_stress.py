@@ -1,0 +1,108 @@
+"""Stress of the EXL3 decode path, bounded so that it runs in seconds: random shapes, bit widths, plans, layouts and row
+counts against the oracle (each case stops at its first mismatch and names itself), and thousands of random
+(linear, rows) calls on one shared workspace without a synchronization in between, every one compared bit for bit with
+the first result of its kind (the role of crates/fe-exl3/src/bin/exl3-stress.rs:62-98, which runs 256k such calls)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROWS = [1, 2, 3, 4, 5, 8, 15, 16, 17, 31, 33, 48, 63, 64]
+
+
+def dev_u16(torch, a):
+    return torch.from_numpy(np.ascontiguousarray(a).view(np.int16)).cuda()
+
+
+def random_plan(rng, exl3, k, n):
+    kind = int(rng.integers(0, 3))
+    if kind == 0:  # sk programs per column block
+        steps = k // 64
+        return exl3.Plan(int(rng.choice([d for d in range(1, steps + 1) if steps % d == 0])), 1, 1, 0)
+    if kind == 1:  # occ programs per CU, runs of at least wk units
+        return exl3.Plan(1, int(rng.choice([1, 2, 4])), 3, int(rng.integers(1, 6)))
+    return exl3.Plan(int(rng.integers(1, (k // 128) * (n // 128) + 3)), 1, 4, 0)  # that many programs in all
+
+
+def test_random_shapes_against_the_oracle(oracle):
+    import torch
+    from ferrite_amd import exl3, route, synth
+    kern = exl3.Kernels.load()
+    rng = np.random.default_rng(20251)
+    for case in range(48):
+        k = int(rng.integers(1, 17)) * 128
+        bits = int(rng.choice([2, 3, 4, 5, 6, 8]))
+        ns = [int(rng.integers(1, 7)) * 128 for _ in range(int(rng.integers(1, 4)))]
+        rows = int(rng.choice(ROWS))
+        lins, ts = [], []
+        for i, n in enumerate(ns):
+            t = synth.exl3_tensor(k, n, bits, 1000 + case * 10 + i)
+            strips = bool(rng.integers(0, 2))
+            lins.append(exl3.Linear.with_plan(kern, exl3.DeviceExl3(t, strips), random_plan(rng, exl3, k, n)))
+            ts.append(t)
+        ws = exl3.Workspace(lins, 64)
+        xb = synth.activations(rows, k, case, outliers=bool(rng.integers(0, 2)))
+        x = dev_u16(torch, xb)
+        what = f"case {case}: k {k} bits {bits} ns {ns} plans {[l.plan for l in lins]} rows {rows}"
+        ys = [torch.full((rows + 1, n), float("nan"), dtype=torch.float32, device="cuda") for n in ns]
+        for l, y in zip(lins, ys):
+            l.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, rows, ws)
+        torch.cuda.synchronize()
+        for l, t, y in zip(lins, ts, ys):
+            o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+            l.rotate_input(x, exl3.Dtype.Bf16, rows, ws)
+            torch.cuda.synchronize()
+            ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(rows, k))
+            got = y.cpu().numpy()
+            assert np.abs(got[:rows] - ref).max() / max(np.sqrt((ref ** 2).mean()), 1e-30) < 1e-4, what
+            assert np.isnan(got[rows]).all(), what
+        if len(lins) >= 2:  # the same linears as one launch: the bits of each one's own forward
+            gs = [torch.full((rows + 1, n), float("nan"), dtype=torch.float32, device="cuda") for n in ns]
+            exl3.forward_group(lins, x, exl3.Dtype.Bf16, gs, exl3.Dtype.F32, rows, ws)
+            torch.cuda.synchronize()
+            for a, b in zip(ys, gs):
+                assert torch.equal(a[:rows].view(torch.int32), b[:rows].view(torch.int32)) and torch.isnan(b[rows]).all(), what
+        # SwiGLU of two arrays as the input: the bits of fe_silu_mul followed by forward
+        gu = dev_u16(torch, synth.activations(rows, 2 * k, case + 7))
+        act = torch.zeros((rows, k), dtype=torch.bfloat16, device="cuda")
+        route.silu_mul(act, gu.data_ptr(), gu.data_ptr() + 2 * k, 2 * k, k, rows)
+        a = torch.zeros((rows, ns[0]), dtype=torch.float32, device="cuda")
+        b = torch.zeros_like(a)
+        lins[0].forward(act.view(torch.int16), exl3.Dtype.Bf16, a, exl3.Dtype.F32, rows, ws)
+        lins[0].forward_swiglu(gu.data_ptr(), gu.data_ptr() + 2 * k, 2 * k, b, exl3.Dtype.F32, rows, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), what
+
+
+def test_random_calls_on_a_shared_workspace_repeat_their_bits():
+    import torch
+    from ferrite_amd import exl3, synth
+    kern = exl3.Kernels.load()
+    blocks = exl3.default_blocks(exl3.cu_count())
+    shapes = [(1024, 2048, 4), (2048, 1024, 3), (5120, 1024, 4), (1024, 384, 5), (3072, 640, 2), (512, 4096, 6)]
+    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, n, b, 70 + i)), blocks)
+            for i, (k, n, b) in enumerate(shapes)]
+    ws = exl3.Workspace(lins, 64)
+    xs = [dev_u16(torch, synth.activations(64, k, 80 + i)) for i, (k, n, b) in enumerate(shapes)]
+    rows_list = [1, 2, 4, 8, 16, 17, 33, 64]
+    want = {}
+    for li, l in enumerate(lins):
+        for m in rows_list:
+            y = torch.zeros((m, l.n), dtype=torch.float32, device="cuda")
+            l.forward(xs[li], exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+            want[(li, m)] = y
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(7)
+    calls, batches, bad = 400, 24, 0
+    for bi in range(batches):
+        picks = [(int(rng.integers(0, len(lins))), int(rng.choice(rows_list))) for _ in range(calls)]
+        outs = []
+        for li, m in picks:
+            y = torch.empty((m, lins[li].n), dtype=torch.float32, device="cuda")
+            lins[li].forward(xs[li], exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+            outs.append(y)
+        torch.cuda.synchronize()
+        for (li, m), y in zip(picks, outs):
+            if not torch.equal(y.view(torch.int32), want[(li, m)].view(torch.int32)):
+                bad += 1
+        assert bad == 0, f"batch {bi}: {bad} of {calls} calls differ from their first result"
