@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized-linear hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-prefill] [--no-sweep]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-prefill] [--no-sweep] [--no-configs]
 
 Workload (BASELINE.json configs[1]): the EXL3 decode MLP of a Qwen3.8-27B-shaped layer at M = 1, at 3, 4 and 5 bits per
 weight: gate and up are K=5120 N=17408, down is K=17408 N=5120. One step = the forward (input rotation + trellis GEMV)
@@ -11,13 +11,18 @@ Linear::forward. `value` is the trellis bytes streamed per second (the reference
 crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step, launch gaps and input rotations included. The nine
 weight sets total 401 MB, more than L2 plus the 256 MB Infinity Cache, so every step streams its weights from HBM.
 
-`roofline` is the dominant kernel alone (the grouped 4-bit GEMV of the two 5120x17408 projections): its trellis bytes
+`roofline` is the dominant kernel alone (the 4-bit GEMV launch of the two 5120x17408 projections): its trellis bytes
 over its average launch duration, measured with HIP event pairs on the launch stream around its launches inside the
 timed region (the other launches of the timed region carry no events: every record is a packet of its own on the queue;
-a pass after the timed region brackets all six launches for `per_launch`).
-`cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host.
+a pass after the timed region brackets all six launches for `per_launch`). It also carries the single 5120x17408 linear
+the target names and the measured decode-only ceiling of the vector ALUs (`alu_ceiling_GBs`), which splits the distance to
+the HBM roofline into "ceiling against HBM" and "kernel against ceiling".
+`cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host;
+`configs` holds, per BASELINE configuration, a CPU figure of the same kind and the parity of the GPU result against it
+(W_hat mismatches on sampled tiles, max |y - ref| / rms(ref), max relative error with the denominator floored at the rms).
 `m2048` reports the prefill GEMMs (EXL3 4-bit and NVFP4, 5120x17408, M = 2048) in TFLOP/s against the bf16/f16 MFMA
-peak; it is measured after the timed region and is not part of `value`.
+peak; it is measured after the timed region and is not part of `value`. Every timed figure cycles over enough copies of
+its weights (at least 512 MB) that none is served from L2 or the Infinity Cache.
 """
 from __future__ import annotations
 
@@ -33,14 +38,17 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
-# `bench.py --traffic-pass` (profiles/exl3_gemv_group_b4_m1_hbm_traffic.md): 45202 KiB fetched x 2.0 (the factor that
-# makes the counter read a streaming read and an elementwise update of known size correctly) + 799 KiB written x 1.0
-ROOFLINE_TRAFFIC_BYTES = int((45202 * 2.0 + 799 * 1.0) * 1024)
+# `bench.py --traffic-pass`: KiB fetched x 2.0 (the factor that makes the counter read a streaming read and an
+# elementwise update of known size correctly) + KiB written x 1.0
+ROOFLINE_TRAFFIC_BYTES = int((46793 * 2.0 + 1218 * 1.0) * 1024)
+ROOFLINE_TRAFFIC_SOURCE = "profiles/exl3_gemvb_b4_gate_up_m1_hbm_traffic.md (rocprofv3 --pmc, not measured by this run)"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA peak of MI355X
 SEED = 20251
 MLP = [("gate", 5120, 17408), ("up", 5120, 17408), ("down", 17408, 5120)]
 BITS = [3, 4, 5]
+COLD_BYTES = 512 << 20  # weights a timed loop cycles through: past the 256 MB Infinity Cache
+ROW_SAMPLE = lambda m: sorted({0, 1, 17, 127, min(128, m - 1), m // 2, m - 1})  # crates/fe-fp4/src/bin/fp4-check.rs:96
 
 
 class Events:
@@ -63,6 +71,20 @@ class Events:
         self.check(self.lib.fe_hip_event_elapsed_ms(C.byref(out), a, b))
         return out.value
 
+    def loop_us(self, stream, fn, reps):
+        """Microseconds per call of fn() over `reps` back-to-back calls between one pair of recorded events."""
+        fn()
+        a, b = self.new(), self.new()
+        self.record(a, stream)
+        for _ in range(reps):
+            fn()
+        self.record(b, stream)
+        return self.ms(a, b) * 1e3 / reps
+
+
+def bf16_to_f64(np, bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
 
 def cpu_baseline(reps=12):
     """The CPU oracle on the workload's 4-bit MLP (gate, up, down at M = 1), all host cores, `reps` passes: a bounded
@@ -75,20 +97,66 @@ def cpu_baseline(reps=12):
     for name, k, n in MLP:
         t = synth.exl3_tensor(k, n, 4, SEED, name)
         o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
-        x = (synth.activations(1, k, SEED).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        x = bf16_to_f64(np, synth.activations(1, k, SEED))
         layers.append((o, x))
         nbytes += t.trellis_bytes()
-    y_gate = None
     t0 = time.perf_counter()
     for _ in range(reps):
-        for i, (o, x) in enumerate(layers):
-            y = oracle.linear_f64(o, x, threads=cores)
-            if i == 0:
-                y_gate = y
+        for o, x in layers:
+            oracle.linear_f64(o, x, threads=cores)
     dt = time.perf_counter() - t0
     return {"value": round(reps * nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
             "sample": f"oracle linear_f64 (decode_tile + f64 factored linear, threaded over 128-column blocks) on the 4-bit "
-                      f"gate, up and down projections at M=1, {reps} passes, {dt:.2f} s"}, y_gate
+                      f"gate, up and down projections at M=1, {reps} passes, {dt:.2f} s"}
+
+
+def cold_copies(torch, exl3, kern, lin_sets, total=COLD_BYTES):
+    """lin_sets: a list of linears that one timed call uses together. Returns a list of such lists, the first the given
+    one, the others over device copies of the same weights (plans and bits unchanged), enough of them that a loop over
+    the list touches at least `total` bytes of trellis before it comes back to the first."""
+    per = sum(l.weight_bytes() for l in lin_sets)
+    out, keep = [list(lin_sets)], []
+    while per * len(out) < total:
+        cp = []
+        for l in lin_sets:
+            tr = torch.empty(l.weight_bytes() // 4, dtype=torch.int32, device="cuda")
+            _copy_dtod(tr.data_ptr(), l.view.trellis, l.weight_bytes())
+            v = exl3.Exl3View(l.k, l.n, l.bits, tr.data_ptr(), l.view.suh, l.view.svh, l.view.strips)
+            cp.append(exl3.Linear.from_view(kern, l.name, v, l.plan))
+            keep.append(tr)
+        out.append(cp)
+    return out, keep
+
+
+def _copy_dtod(dst, src, nbytes):
+    from ferrite_amd import _lib
+    _lib.check(_lib.lib().fe_hip_memcpy_dtod_async(dst, src, nbytes, None))
+    _lib.check(_lib.lib().fe_hip_synchronize())
+
+
+def exl3_parity(torch, np, oracle, exl3, kern, t, x_bits, y_rows, rows, tiles=64):
+    """Parity of one EXL3 linear on the GPU against the reference's CPU path restated in oracle/: W_hat on `tiles` sampled
+    16x16 tiles, bit for bit, against decode_tile; outputs y_rows (f64, the rows `rows` of the batch x_bits) against
+    linear_f64 on the same bf16 inputs. Returns the parity triple and the seconds the CPU linear took."""
+    stored = exl3.DeviceExl3.upload(t)
+    w = torch.zeros((t.k, t.n), dtype=torch.int16, device="cuda")
+    kern.reconstruct_hat_f16(stored.view, w)
+    torch.cuda.synchronize()
+    rng = np.random.default_rng([SEED, t.k, t.n, t.bits])
+    bad = 0
+    for kt, nt in zip(rng.integers(0, t.k // 16, tiles), rng.integers(0, t.n // 16, tiles)):
+        want = oracle.decode_tile(t.tile(int(kt), int(nt)), t.bits)
+        got = w[kt * 16:kt * 16 + 16, nt * 16:nt * 16 + 16].cpu().numpy().view(np.uint16)
+        bad += int((got != want).sum())
+    del w, stored
+    o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+    t0 = time.perf_counter()
+    ref = oracle.linear_f64(o, bf16_to_f64(np, x_bits[rows]), threads=oracle.default_threads(64))
+    dt = time.perf_counter() - t0
+    rms = float(np.sqrt((ref ** 2).mean()))
+    err = np.abs(y_rows - ref)
+    return {"w_hat_mismatches": bad, "w_hat_values_checked": tiles * 256, "max_err_over_rms": round(float(err.max() / rms), 6),
+            "max_rel_floored_at_rms": round(float((err / np.maximum(np.abs(ref), rms)).max()), 6), "rows_checked": len(rows)}, dt
 
 
 def main():
@@ -98,6 +166,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--no-configs", action="store_true", help="leave out the per-configuration CPU figures and parity")
     ap.add_argument("--bracket-events", action="store_true",
                     help="time the roofline kernel with events recorded before and after its launch instead of events attached to its dispatch")
     ap.add_argument("--no-sweep", action="store_true", help="leave out the M = 1, 4, 8, 16 sweep (for a kernel trace of the step alone)")
@@ -116,9 +185,7 @@ def main():
         sys.exit("bench.py: no GPU")
     if args.traffic_pass:
         return traffic_pass(torch, np, exl3, synth)
-    cpu = None
-    if not args.no_cpu:
-        cpu, y_cpu = cpu_baseline()  # first, as the configuration asks
+    cpu = None if args.no_cpu else cpu_baseline()  # first, as the configuration asks
 
     kern = exl3.Kernels.load()
     lib = _lib.lib()
@@ -127,25 +194,17 @@ def main():
     blocks = exl3.default_blocks(exl3.cu_count())
 
     # the nine linears, one device copy each
-    linears = []
+    linears, tensors = [], {}
     for bits in BITS:
         for name, k, n in MLP:
             t = synth.exl3_tensor(k, n, bits, SEED, name)
+            tensors[(name, bits)] = t
             lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), blocks)
             x = torch.from_numpy(synth.activations(1, k, SEED).view(np.int16)).cuda()
             y = torch.zeros((1, n), dtype=torch.bfloat16, device="cuda")
             linears.append((name, bits, lin, x, y))
     ws = exl3.Workspace([l[2] for l in linears], 1)
     total_bytes = sum(l[2].weight_bytes() for l in linears)
-
-    if cpu is not None:  # parity of the sampled layer on the GPU against the CPU result just computed
-        name, bits, lin, x, _ = next(l for l in linears if l[0] == "gate" and l[1] == 4)
-        yf = torch.zeros((1, lin.n), dtype=torch.float32, device="cuda")
-        lin.forward(x, exl3.Dtype.Bf16, yf, exl3.Dtype.F32, 1, ws)
-        torch.cuda.synchronize()
-        got = yf.cpu().numpy().astype(np.float64)
-        rel = float(np.abs(got - y_cpu).max() / np.sqrt((y_cpu ** 2).mean()))
-        cpu["gpu_vs_cpu_max_err_over_rms"] = round(rel, 6)
 
     # The step's launches: per bit width, gate + up of one input as a grouped call, then down. Every argument of the calls
     # into the C ABI is prepared once.
@@ -214,25 +273,9 @@ def main():
         if la[2]:
             dom_ms += [ev.ms(*events[i][li]) for i in range(args.steps)]
             dom_bytes = la[1]
-            dom_kernel = "exl3_gemv_group_b4"
+    dom_kernel = "exl3_gemvb_b4_r1"
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
-
-    # the dominant launch alone, back to back between one pair of events: its duration without the event packets and the
-    # other launches' gaps (what a kernel trace reports for it inside the step; here the same 89 MB are read every time
-    # and stay in the Infinity Cache, which does not help a kernel bound by its decode instructions)
-    dom = next(la for la in launches if la[2])
-    a, b = ev.new(), ev.new()
-    rc = 0
-    for fn, aa in dom[4]:
-        rc |= fn(*aa)
-    ev.record(a, stream)
-    for _ in range(args.steps):
-        for fn, aa in dom[4]:
-            rc |= fn(*aa)
-    ev.record(b, stream)
-    _lib.check(rc)
-    dom_b2b_us = ev.ms(a, b) * 1e3 / args.steps
 
     per, reps = {}, max(args.steps, 5)
     acc = [0.0] * len(launches)
@@ -244,6 +287,42 @@ def main():
         us = acc[li] / reps * 1e3
         per[la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
 
+    # The dominant launch and the single linear the target names, each alone and back to back between one pair of
+    # events, cycling over weight copies past the caches: the kernel's duration plus the gap between two launches.
+    g4, u4 = by[("gate", 4)][0], by[("up", 4)][0]
+    x4 = by[("gate", 4)][1]
+    pair_sets, keep1 = cold_copies(torch, exl3, kern, [g4, u4])
+    ws_pair = exl3.Workspace([g4, u4], 1)
+    ys_pair = [by[("gate", 4)][2], by[("up", 4)][2]]
+    at = [0]
+
+    def dom_call():
+        exl3.forward_group(pair_sets[at[0] % len(pair_sets)], x4, exl3.Dtype.Bf16, ys_pair, exl3.Dtype.Bf16, 1, ws_pair, stream=stream)
+        at[0] += 1
+
+    dom_b2b_us = ev.loop_us(stream, dom_call, 4 * len(pair_sets))
+
+    def single_call():
+        pair_sets[at[0] % len(pair_sets)][0].forward(x4, exl3.Dtype.Bf16, ys_pair[0], exl3.Dtype.Bf16, 1, ws_pair, stream=stream)
+        at[0] += 1
+
+    single_us = ev.loop_us(stream, single_call, 8 * len(pair_sets))
+    # ... and its kernel alone, by events attached to the dispatch (what a kernel trace reports)
+    one_pairs = [(ev.new(), ev.new()) for _ in range(2 * len(pair_sets))]
+    for a, b in one_pairs:
+        _lib.check(f_time_next(a, b))
+        single_call()
+    single_kernel_us = sum(ev.ms(a, b) for a, b in one_pairs) / len(one_pairs) * 1e3
+    single_bytes = g4.weight_bytes()
+    del pair_sets, keep1
+
+    # the decode-only ceiling of the vector ALUs: the GEMV's decode at the GEMV's occupancy with no memory traffic
+    ceiling = {}
+    for bits in BITS:
+        grid, iters = 4 * exl3.cu_count(), 256
+        ms = kern.probe_decode(bits, grid, iters, 5)
+        ceiling[f"b{bits}"] = round(grid * 256 * 32 * iters * bits / 8 / (ms * 1e-3) / 1e9, 1)
+
     out = {
         "metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -252,21 +331,155 @@ def main():
         "config": {"workload": "EXL3 decode MLP, Qwen3.8-27B-shaped layer, M=1, 3/4/5 bpw (gate, up 5120x17408; down 17408x5120)",
                    "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
                    "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
-        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (gate + up, 5120x17408 each, M=1)", "achieved": round(achieved, 2),
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": ROOFLINE_TRAFFIC_BYTES,
+        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (gate + up in one launch, 5120x17408 each, 4 bits, M=1)",
+                     "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": ROOFLINE_TRAFFIC_BYTES, "traffic_source": ROOFLINE_TRAFFIC_SOURCE,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms),
-                     "back_to_back_us": round(dom_b2b_us, 3),
-                     "events": "recorded around the launch" if args.bracket_events else "attached to the kernel's dispatch"},
+                     "back_to_back_cold_us": round(dom_b2b_us, 3),
+                     "events": "recorded around the launch" if args.bracket_events else "attached to the kernel's dispatch",
+                     "alu_ceiling_GBs": ceiling,
+                     "frac_of_alu_ceiling": round(achieved / ceiling["b4"], 4),
+                     "single_linear_5120x17408_b4_m1": {
+                         "kernel_us": round(single_kernel_us, 3), "GB/s": round(single_bytes / single_kernel_us / 1e3, 1),
+                         "frac": round(single_bytes / single_kernel_us / 1e3 / HBM_PEAK_GBS, 4),
+                         "back_to_back_cold_us": round(single_us, 3), "bytes_per_launch": single_bytes}},
         "cpu_baseline": cpu,
         "per_launch": per,
     }
 
     out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup)
+    if not args.no_configs and not args.no_cpu:
+        out["configs"] = configs(torch, np, exl3, fp4, synth, kern, ev, stream, tensors, by, ws)
     if not args.no_sweep:
-        out["rows_sweep_b4"] = rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears)
+        out["rows_sweep_b4"] = rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, _lib.check, linears)
     if not args.no_prefill:
         out["m2048"] = prefill(torch, np, exl3, fp4, synth, kern, ev, stream)
     print(json.dumps(out))
+
+
+def configs(torch, np, exl3, fp4, synth, kern, ev, stream, tensors, by, ws):
+    """Per BASELINE configuration: the CPU path (oracle/: the reference's CPU dequant + matmul restated) timed on the host
+    cores, run before the GPU figure it stands beside, and the parity of the GPU result against it."""
+    import oracle
+    cores = oracle.default_threads(64)
+    res = {"cpu_cores": cores}
+    blocks = exl3.default_blocks(exl3.cu_count())
+
+    # configs[0]: EXL3 4 bpw, K = N = 5120, M = 1; the CPU path first
+    t = synth.exl3_tensor(5120, 5120, 4, SEED, "c1")
+    xb = synth.activations(1, 5120, SEED)
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), blocks)
+    w1 = exl3.Workspace([lin], 1)
+    x = torch.from_numpy(xb.view(np.int16)).cuda()
+    y = torch.zeros((1, 5120), dtype=torch.float32, device="cuda")
+    o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+    t0 = time.perf_counter()
+    for _ in range(5):
+        oracle.linear_f64(o, bf16_to_f64(np, xb), threads=cores)
+    cpu_s = (time.perf_counter() - t0) / 5
+    lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 1, w1)
+    torch.cuda.synchronize()
+    par, _ = exl3_parity(torch, np, oracle, exl3, kern, t, xb, y.cpu().numpy().astype(np.float64), [0])
+    sets, keep = cold_copies(torch, exl3, kern, [lin])
+    yb = torch.zeros((1, 5120), dtype=torch.bfloat16, device="cuda")
+    at = [0]
+
+    def call():
+        sets[at[0] % len(sets)][0].forward(x, exl3.Dtype.Bf16, yb, exl3.Dtype.Bf16, 1, w1, stream=stream)
+        at[0] += 1
+
+    us = ev.loop_us(stream, call, 2 * len(sets))
+    nbytes = lin.weight_bytes()
+    res["c1_exl3_b4_5120x5120_m1"] = {
+        "cpu": {"seconds": round(cpu_s, 4), "GB/s": round(nbytes / cpu_s / 1e9, 4), "cores": cores, "kind": "port",
+                "sample": "oracle linear_f64, whole linear, 5 passes"},
+        "gpu": {"us": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)},
+        "gpu_over_cpu": round(cpu_s * 1e6 / us, 1), "parity": par}
+    del sets, keep, lin, w1
+
+    # configs[1]: every linear of the timed step against the CPU linear on the same input
+    c2 = {}
+    for (name, bits), t in tensors.items():
+        lin, x, _ = by[(name, bits)]
+        y = torch.zeros((1, t.n), dtype=torch.float32, device="cuda")
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, 1, ws)
+        torch.cuda.synchronize()
+        par, cpu_s = exl3_parity(torch, np, oracle, exl3, kern, t, synth.activations(1, t.k, SEED), y.cpu().numpy().astype(np.float64), [0])
+        par["cpu_linear_f64_seconds"] = round(cpu_s, 4)
+        c2[f"{name}_b{bits}"] = par
+    res["c2_decode_mlp_m1"] = c2
+
+    # configs[3]: EXL3 4 bpw prefill, M = 2048, activations with 1 % outlier channels x20. The CPU figure is the f64 linear on
+    # the reference's row sample and on one row: T(m) = a + b m (decode once, then the products), evaluated at 2048 rows.
+    m = 2048
+    c4 = {}
+    for name, k, n in (("gate_up", 5120, 17408), ("down", 17408, 5120)):
+        t = tensors[("gate" if name == "gate_up" else "down", 4)]
+        xb = synth.activations(m, k, SEED, outliers=True)
+        rows = ROW_SAMPLE(m)
+        o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+        t0 = time.perf_counter()
+        oracle.linear_f64(o, bf16_to_f64(np, xb[:1]), threads=cores)
+        t1 = time.perf_counter() - t0
+        lin = by[("gate" if name == "gate_up" else "down", 4)][0]
+        wsm = exl3.Workspace([lin], m)
+        x = torch.from_numpy(xb.view(np.int16)).cuda()
+        y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.Bf16, m, wsm)
+        torch.cuda.synchronize()
+        got = y[rows].float().cpu().numpy().astype(np.float64)
+        par, t7 = exl3_parity(torch, np, oracle, exl3, kern, t, xb, got, rows, tiles=16)
+        b = max(t7 - t1, 0.0) / (len(rows) - 1)
+        cpu_s = t1 + b * (m - 1)
+        flops = 2.0 * m * n * k
+        c4[f"exl3_b4_{k}x{n}"] = {
+            "cpu": {"seconds_extrapolated": round(cpu_s, 2), "GFLOP/s": round(flops / cpu_s / 1e9, 2), "cores": cores, "kind": "port",
+                    "sample": f"oracle linear_f64 on 1 row ({t1:.2f} s) and on rows {rows} ({t7:.2f} s), extrapolated linearly to {m} rows"},
+            "parity": par}
+        del wsm, x, y
+    res["c4_exl3_prefill_m2048"] = c4
+
+    # configs[4]: NVFP4, K = 5120, N = 17408, M = 1 and 2048: quantize the activations, dequantize both operands, f64 dot
+    # products (crates/fe-fp4/src/format.rs:72-90, 136-142, 151-181), on the row sample; parity as fp4-check.rs:134-144
+    k, n = 5120, 17408
+    host = synth.fp4_linear(n, k, SEED, input_scale=1.0)
+    fk = fp4.Kernels.load()
+    flin = host.upload()
+    t0 = time.perf_counter()
+    wdq = oracle.dequant_fp4(host.codes, host.sf, 1.0)
+    t_w = time.perf_counter() - t0
+    c5 = {}
+    for m in (1, 2048):
+        xb = synth.activations(m, k, SEED)
+        rows = ROW_SAMPLE(m) if m > 1 else [0]
+        t0 = time.perf_counter()
+        codes, sf = oracle.quant_fp4(xb[rows], host.g)
+        ref = oracle.ref_gemm(oracle.dequant_fp4(codes, sf, 1.0), wdq).astype(np.float64) * host.alpha.astype(np.float64)
+        t_rows = time.perf_counter() - t0
+        cpu_s = t_w + t_rows / len(rows) * m
+        fws = fp4.Workspace(m, k)
+        x = torch.from_numpy(xb.view(np.int16)).cuda()
+        y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+        flin.forward(fk, fws, y, n, x, k, m)
+        torch.cuda.synchronize()
+        got = y[rows].float().cpu().numpy().astype(np.float64)
+        gc, gsf_t = fws.read(m, k)
+        gsf = oracle.untile_scales(gsf_t, m, k // 16).reshape(m, k // 16)
+        scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+        flops = 2.0 * m * n * k
+        c5[f"m{m}"] = {
+            "cpu": {"seconds" + ("_extrapolated" if m > 1 else ""): round(cpu_s, 3), "GFLOP/s": round(flops / cpu_s / 1e9, 2),
+                    "cores": cores, "kind": "port",
+                    "sample": f"oracle quant_fp4_row + dequant_fp4_row + ref_gemm on rows {rows} ({t_rows:.2f} s) plus the weight "
+                              f"dequantization ({t_w:.2f} s)" + (f", scaled to {m} rows" if m > 1 else "")},
+            "parity": {"activation_code_bytes_differing": int((gc[rows] != codes).sum()),
+                       "activation_scale_bytes_differing": int((gsf[rows] != sf).sum()),
+                       "max_err_over_row_max": round(float((np.abs(got - ref) / scale).max()), 6),
+                       "max_rel_floored_at_1e-2_row_max": round(float((np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max()), 6),
+                       "rows_checked": len(rows)}}
+        del fws, x, y
+    res["c5_nvfp4_5120x17408"] = c5
+    return res
 
 
 def traffic_pass(torch, np, exl3, synth):
@@ -290,77 +503,91 @@ def traffic_pass(torch, np, exl3, synth):
         exl3.forward_group(lins, x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, 1, ws)
     torch.cuda.synchronize()
     print(json.dumps({"exl3_probe_v4_reads_KiB": nbytes / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
-                      "roofline_kernel": "exl3_gemv_group_b4", "algorithmic_KiB": nbytes / 1024}))
+                      "roofline_kernel": "exl3_gemvb_b4_r1", "algorithmic_KiB": nbytes / 1024}))
 
 
-def rows_sweep(torch, np, exl3, synth, kern, ev, stream, linears, reps=20):
-    """The 4-bit MLP at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts): microseconds per linear,
-    launched back to back as the step launches them (gate + up grouped, then down), so that no weight is served from
-    cache. Not part of `value`."""
+def graph_us(lib, check, ev, fn, inner, reps=5):
+    """Microseconds per call of fn(stream) with `inner` calls captured into one HIP graph on a stream of its own and the
+    graph replayed `reps` times."""
+    s, g = C.c_void_p(), C.c_void_p()
+    check(lib.fe_hip_stream_create(C.byref(s)))
+    fn(s)
+    check(lib.fe_hip_stream_sync(s))
+    check(lib.fe_hip_graph_begin(s))
+    for _ in range(inner):
+        fn(s)
+    check(lib.fe_hip_graph_end(s, C.byref(g)))
+    check(lib.fe_hip_graph_launch(g, s))
+    a, b = ev.new(), ev.new()
+    ev.record(a, s)
+    for _ in range(reps):
+        check(lib.fe_hip_graph_launch(g, s))
+    ev.record(b, s)
+    us = ev.ms(a, b) * 1e3 / (reps * inner)
+    check(lib.fe_hip_graph_destroy(g))
+    check(lib.fe_hip_stream_destroy(s))
+    return us
+
+
+def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
+    """The 4-bit MLP and the attention projections at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts):
+    microseconds per linear, launched back to back as the step launches them (gate + up grouped, then down; q, k, v grouped,
+    then o), cycling over weight copies of at least 512 MB in all, eagerly launched and replayed from a graph. Not part of
+    `value`."""
     four = {name: lin for name, bits, lin, x, y in linears if bits == 4}
     g, u, d = four["gate"], four["up"], four["down"]
-    res = {}
+    mlp_sets, keep_a = cold_copies(torch, exl3, kern, [g, u, d])
+    blocks = exl3.default_blocks(exl3.cu_count())
+    q, kk, v, o = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, n, 4, SEED, name)), blocks)
+                   for name, n in (("q", 5120), ("k", 1024), ("v", 1024), ("o", 5120)))
+    attn_sets, keep_b = cold_copies(torch, exl3, kern, [q, kk, v, o])
+    abytes = sum(l.weight_bytes() for l in (q, kk, v, o))
+    nbytes = (g.weight_bytes() + u.weight_bytes() + d.weight_bytes()) / 3
+    res = {"weight_copies_cycled": {"mlp": len(mlp_sets), "attn": len(attn_sets)}}
     for m in (1, 4, 8, 16):
-        ws = exl3.Workspace([g, u, d], m)
+        ws = exl3.Workspace([g, u, d, q, kk, v, o], m)
         x = torch.from_numpy(synth.activations(m, g.k, SEED).view(np.int16)).cuda()
         xd = torch.from_numpy(synth.activations(m, d.k, SEED).view(np.int16)).cuda()
         yg, yu = (torch.zeros((m, g.n), dtype=torch.bfloat16, device="cuda") for _ in range(2))
         yd = torch.zeros((m, d.n), dtype=torch.bfloat16, device="cuda")
-
-        def mlp():
-            exl3.forward_group([g, u], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=stream)
-            d.forward(xd, exl3.Dtype.Bf16, yd, exl3.Dtype.Bf16, m, ws, stream=stream)
-
-        mlp()
-        a, b = ev.new(), ev.new()
-        ev.record(a, stream)
-        for _ in range(reps):
-            mlp()
-        ev.record(b, stream)
-        us = ev.ms(a, b) * 1e3 / (reps * 3)
-        nbytes = (g.weight_bytes() + u.weight_bytes() + d.weight_bytes()) / 3
-        res[f"m{m}"] = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1),
-                        "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-                        "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
-        # the MLP block as the model runs it: down reads SwiGLU(gate, up) of the grouped launch's outputs and adds
-        # into the residual stream
         resid = torch.zeros((m, d.n), dtype=torch.bfloat16, device="cuda")
-
-        def block():
-            exl3.forward_group([g, u], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=stream)
-            d.forward_swiglu(yg, yu, g.n, resid, exl3.Dtype.Bf16Add, m, ws, stream=stream)
-
-        block()
-        a, b = ev.new(), ev.new()
-        ev.record(a, stream)
-        for _ in range(reps):
-            block()
-        ev.record(b, stream)
-        res[f"m{m}"]["mlp_block_us"] = round(ev.ms(a, b) * 1e3 / reps, 2)
-    # the attention projections of the same layer (40 heads of 128, 8 KV heads): q, k, v of one input grouped, then o
-    blocks = exl3.default_blocks(exl3.cu_count())
-    q, kk, v, o = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, n, 4, SEED, name)), blocks)
-                   for name, n in (("q", 5120), ("k", 1024), ("v", 1024), ("o", 5120)))
-    abytes = sum(l.weight_bytes() for l in (q, kk, v, o))
-    for m in (1, 4, 8, 16):
-        ws = exl3.Workspace([q, kk, v, o], m)
-        x = torch.from_numpy(synth.activations(m, 5120, SEED).view(np.int16)).cuda()
         ys = [torch.zeros((m, l.n), dtype=torch.bfloat16, device="cuda") for l in (q, kk, v)]
         yo = torch.zeros((m, 5120), dtype=torch.bfloat16, device="cuda")
+        at = [0]
 
-        def attn():
-            exl3.forward_group([q, kk, v], x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, m, ws, stream=stream)
-            o.forward(x, exl3.Dtype.Bf16, yo, exl3.Dtype.Bf16, m, ws, stream=stream)
+        def mlp(s=stream):
+            gg, uu, dd = mlp_sets[at[0] % len(mlp_sets)]
+            at[0] += 1
+            exl3.forward_group([gg, uu], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=s)
+            dd.forward(xd, exl3.Dtype.Bf16, yd, exl3.Dtype.Bf16, m, ws, stream=s)
 
-        attn()
-        a, b = ev.new(), ev.new()
-        ev.record(a, stream)
-        for _ in range(reps):
-            attn()
-        ev.record(b, stream)
-        us = ev.ms(a, b) * 1e3 / reps
-        res[f"m{m}"]["attn_qkv_o_us"] = round(us, 2)
-        res[f"m{m}"]["attn_GB/s"] = round(abytes / us / 1e3, 1)
+        # the MLP block as the model runs it: down reads SwiGLU(gate, up) of the grouped launch's outputs and adds into the
+        # residual stream
+        def block(s=stream):
+            gg, uu, dd = mlp_sets[at[0] % len(mlp_sets)]
+            at[0] += 1
+            exl3.forward_group([gg, uu], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=s)
+            dd.forward_swiglu(yg, yu, g.n, resid, exl3.Dtype.Bf16Add, m, ws, stream=s)
+
+        def attn(s=stream):
+            qq, k2, vv, oo = attn_sets[at[0] % len(attn_sets)]
+            at[0] += 1
+            exl3.forward_group([qq, k2, vv], x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, m, ws, stream=s)
+            oo.forward(x, exl3.Dtype.Bf16, yo, exl3.Dtype.Bf16, m, ws, stream=s)
+
+        us = ev.loop_us(stream, mlp, 3 * len(mlp_sets)) / 3
+        r = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+             "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
+        r["mlp_block_us"] = round(ev.loop_us(stream, block, 3 * len(mlp_sets)), 2)
+        r["mlp_block_graph_us"] = round(graph_us(lib, check, ev, block, 2 * len(mlp_sets)), 2)
+        a_us = ev.loop_us(stream, attn, 2 * len(attn_sets))
+        r["attn_qkv_o_us"] = round(a_us, 2)
+        r["attn_GB/s"] = round(abytes / a_us / 1e3, 1)
+        a_g = graph_us(lib, check, ev, attn, 2 * len(attn_sets))
+        r["attn_qkv_o_graph_us"] = round(a_g, 2)
+        r["attn_graph_GB/s"] = round(abytes / a_g / 1e3, 1)
+        res[f"m{m}"] = r
+    del mlp_sets, attn_sets, keep_a, keep_b
     return res
 
 
@@ -393,6 +620,10 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     res = {}
     flops = 2.0 * m * n * k
     reps = 10
+
+    def timed(fn, reps=10):
+        return ev.loop_us(stream, fn, reps) / 1e3
+
     # EXL3
     t = synth.exl3_tensor(k, n, 4, SEED, "gate")
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 1024)
@@ -400,30 +631,13 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     x = torch.from_numpy(synth.activations(m, k, SEED, outliers=True).view(np.int16)).cuda()
     y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     lin.rotate_input(x, exl3.Dtype.Bf16, m, ws)
-    lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
-    a, b = ev.new(), ev.new()
-    ev.record(a, stream)
-    for _ in range(reps):
-        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
-    ev.record(b, stream)
-    ms = ev.ms(a, b) / reps
-    a2, b2 = ev.new(), ev.new()
-    ev.record(a2, stream)
-    for _ in range(reps):
-        lin.rotate_input(x, exl3.Dtype.Bf16, m, ws)
-    ev.record(b2, stream)
-    rot_ms = ev.ms(a2, b2) / reps
+    ms = timed(lambda: lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws))
+    rot_ms = timed(lambda: lin.rotate_input(x, exl3.Dtype.Bf16, m, ws))
     res["exl3_b4_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                                  "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "rot_in_ms": round(rot_ms, 4)}
     # the same with the weights decoded once and kept with the linear (2 bytes a weight): no decode launch per call
     lin.keep_decoded()
-    lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
-    a3, b3 = ev.new(), ev.new()
-    ev.record(a3, stream)
-    for _ in range(reps):
-        lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws)
-    ev.record(b3, stream)
-    ms = ev.ms(a3, b3) / reps
+    ms = timed(lambda: lin.gemv_rotated(ws.xh_ptr, y, exl3.Dtype.Bf16, m, ws))
     res["exl3_b4_5120x17408_decoded_kept"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                                               "kept_bytes": ((n // 128 + 1) // 2) * 256 * k * 2}
@@ -435,47 +649,32 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     xf = torch.from_numpy(synth.activations(m, k, SEED).view(np.int16)).cuda()
     yf = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     flin.forward(fk, fws, yf, n, xf, k, m)
-    a, b = ev.new(), ev.new()
-    ev.record(a, stream)
-    for _ in range(reps):
-        flin.gemm(fk, fws, yf, n, m)
-    ev.record(b, stream)
-    ms = ev.ms(a, b) / reps
-    a2, b2 = ev.new(), ev.new()
-    ev.record(a2, stream)
-    for _ in range(reps):
-        flin.quantize(fk, fws, xf, k, m)
-    ev.record(b2, stream)
-    q_ms = ev.ms(a2, b2) / reps
+    ms = timed(lambda: flin.gemm(fk, fws, yf, n, m))
+    q_ms = timed(lambda: flin.quantize(fk, fws, xf, k, m))
     res["nvfp4_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
-                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "quant_ms": round(q_ms, 4)}
-    # NVFP4 at M = 1: the weight-read-bound GEMV over the same linear (codes + block scales = 9/16 byte a weight)
-    flin.quantize(fk, fws, xf, k, 1)
-    reps = 50
-    pairs = [(ev.new(), ev.new()) for _ in range(reps)]
-    flin.gemm(fk, fws, yf, n, 1)
-    for a, b in pairs:
-        ev.record(a, stream)
-        flin.gemm(fk, fws, yf, n, 1)
-        ev.record(b, stream)
-    us = sum(ev.ms(a, b) for a, b in pairs) / reps * 1e3
+                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "quant_ms": round(q_ms, 4),
+                               # the quantizer leaves the activations as codes + scales (the format) and as the fp16 operand
+                               # 2 * value * scale the GEMM reads: 2 bytes an element against the format's 9/16
+                               "activation_operand_bytes": m * k * 2, "activation_format_bytes": m * k // 2 + m * k // 16}
+    # NVFP4 at M = 1: the weight-read-bound GEMV over the same linear (codes + block scales = 9/16 byte a weight), cycling
+    # over weight copies past the caches
+    host1 = synth.fp4_linear(n, k, SEED, input_scale=1.0)
     wbytes = n * k // 2 + n * k // 16
+    copies = [flin] + [host1.upload() for _ in range(max(1, COLD_BYTES // wbytes))]
+    flin.quantize(fk, fws, xf, k, 1)
+    at = [0]
+
+    def gemv1():
+        copies[at[0] % len(copies)].gemm(fk, fws, yf, n, 1)
+        at[0] += 1
+
+    us = ev.loop_us(stream, gemv1, 4 * len(copies))
     res["nvfp4_5120x17408_m1"] = {"gemv_us": round(us, 2), "GB/s": round(wbytes / us / 1e3, 1),
-                                  "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
-    del flin, yf
+                                  "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_cycled": len(copies)}
+    del copies, flin, yf, host1
     # the layer's other prefill shape, down (17408 x 5120): the same two GEMMs
     kd, nd = n, k
     flops_d = 2.0 * m * nd * kd
-
-    def timed(fn):
-        fn()
-        a, b = ev.new(), ev.new()
-        ev.record(a, stream)
-        for _ in range(10):
-            fn()
-        ev.record(b, stream)
-        return ev.ms(a, b) / 10
-
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(kd, nd, 4, SEED, "down")), 1024)
     ws = exl3.Workspace([lin], m)
     x = torch.from_numpy(synth.activations(m, kd, SEED, outliers=True).view(np.int16)).cuda()
@@ -494,30 +693,18 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     del flin_d, fws_d, x, y
     # the two neighbours of that GEMM in the prompt path: the fused gate|up front (SwiGLU + NVFP4 re-quantization in the
     # epilogue, 2 x 17408 output columns) and an FP8 linear of the same shape
-    reps = 5
     gate, up = synth.fp4_linear(n, k, SEED, name="gate"), synth.fp4_linear(n, k, SEED + 1, name="up")
     pair = fp4.HostLinear.fuse([("gate", gate.codes, gate.sf, 1.0, 1.0), ("up", up.codes, up.sf, 1.0, 1.0)]).into_swiglu().upload()
     del gate, up
     act = fp4.Workspace(m, n)
-    pair.forward_swiglu(fk, fws, act, xf, k, m, 1.0)
-    a, b = ev.new(), ev.new()
-    ev.record(a, stream)
-    for _ in range(reps):
-        pair.forward_swiglu(fk, fws, act, xf, k, m, 1.0)
-    ev.record(b, stream)
-    ms = ev.ms(a, b) / reps
+    ms = timed(lambda: pair.forward_swiglu(fk, fws, act, xf, k, m, 1.0), 5)
     res["nvfp4_swiglu_front_5120x34816"] = {"quant_plus_gemm_ms": round(ms, 4), "TFLOP/s": round(2 * flops / ms / 1e9, 1),
                                             "frac_mfma_peak": round(2 * flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
     del pair, act
     f8 = synth.fp8_linear(n, k, SEED).upload()
     y8 = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
     f8.forward(fk, fws, y8, n, xf, k, m)
-    a, b = ev.new(), ev.new()
-    ev.record(a, stream)
-    for _ in range(reps):
-        f8.gemm(fk, fws, y8, n, m)
-    ev.record(b, stream)
-    ms = ev.ms(a, b) / reps
+    ms = timed(lambda: f8.gemm(fk, fws, y8, n, m), 5)
     res["fp8_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1), "mfma": "f32_32x32x64_f8f6f4 (e4m3 x e4m3)",
                              "frac_mfma_fp8_peak": round(flops / ms / 1e9 / MFMA_FP8_PEAK_TFLOPS, 4)}
     del f8, y8
@@ -532,21 +719,14 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     ms = timed(lambda: bf16.gemm(bk, yb, n, xf, k, ws_b[0], m))
     res["bf16_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
-    wi = bf16.interleave_gu(bk, ws_b[0], ws_b[1])
-    actb = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
-    ms = timed(lambda: bf16.gemm_swiglu(bk, actb, xf, k, wi, m))
-    res["bf16_swiglu_front_5120x34816"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(2 * flops / ms / 1e9, 1),
-                                           "frac_mfma_peak": round(2 * flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
-    del wi, actb
     for rows in (1, 8):
-        reps = 30
-        pairs = [(ev.new(), ev.new()) for _ in range(reps)]
-        bf16.gemv(bk, yb, n, xf, k, ws_b[0], rows)
-        for i, (a, b) in enumerate(pairs):
-            ev.record(a, stream)
-            bf16.gemv(bk, yb, n, xf, k, ws_b[i % 3], rows)
-            ev.record(b, stream)
-        us = sum(ev.ms(a, b) for a, b in pairs) / reps * 1e3
+        at = [0]
+
+        def gv():
+            bf16.gemv(bk, yb, n, xf, k, ws_b[at[0] % 3], rows)
+            at[0] += 1
+
+        us = ev.loop_us(stream, gv, 30)
         res[f"bf16_5120x17408_m{rows}"] = {"gemv_us": round(us, 2), "GB/s": round(2.0 * n * k / us / 1e3, 1),
                                           "frac_hbm_peak": round(2.0 * n * k / us / 1e3 / HBM_PEAK_GBS, 4)}
     return res

@@ -1035,31 +1035,36 @@ extern "C" __global__ __launch_bounds__(256) void exl3_probe_v4(const u32x4* in,
     if (x == 0x9e3779b9u) out[0] = x;  // practically never: keeps the loads alive without a store stream
 }
 
-// Decode-only probe: every lane decodes `iters` load steps of synthetic words (no memory traffic, no MFMA): the ALU
-// ceiling of the trellis decode in weights per second. out receives a checksum.
+// Decode-only probe: every lane decodes `iters` load steps of synthetic words and feeds them to the matrix instruction as
+// the GEMV does (no memory traffic, no LDS): the ALU ceiling of the trellis decode in weights per second at the GEMV's
+// occupancy (launch 4 programs a CU). The words change from step to step by additions that do not depend on the results,
+// as words from memory would not. out receives a checksum.
 template <int BITS>
 __device__ __forceinline__ void probe_decode_body(uint32_t* out, uint32_t iters, uint32_t seed) {
     LaneWords<BITS> lw;
 #pragma unroll
-    for (int i = 0; i <= BITS; i++) lw.w[i] = seed * (threadIdx.x + 1) + i * 0x9e3779b9u;
-    uint32_t acc = 0;
+    for (int i = 0; i <= BITS; i++) lw.w[i] = (seed + i) * 0x9e3779b9u * (threadIdx.x + 1 + blockIdx.x * 256);
+    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+    const f16x8 xb = {1, 1, 1, 1, 1, 1, 1, 1};
     for (uint32_t it = 0; it < iters; it++) {
         f16x8 op[2][2];
         decode_lane<BITS>(lw, op);
-        u32x4 a = __builtin_bit_cast(u32x4, op[0][0]) ^ __builtin_bit_cast(u32x4, op[0][1]) ^
-                  __builtin_bit_cast(u32x4, op[1][0]) ^ __builtin_bit_cast(u32x4, op[1][1]);
-        acc ^= a[0] ^ a[1] ^ a[2] ^ a[3];
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][0], xb, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][0], xb, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[0][1], xb, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(op[1][1], xb, acc1, 0, 0, 0);
 #pragma unroll
-        for (int i = 0; i <= BITS; i++) lw.w[i] += acc | 1;
+        for (int i = 0; i <= BITS; i++) lw.w[i] += 0x9e3779b9u + i;
     }
-    if (acc == seed) out[blockIdx.x * blockDim.x + threadIdx.x] = acc;
+    const float sum = acc0[0] + acc0[1] + acc0[2] + acc0[3] + acc1[0] + acc1[1] + acc1[2] + acc1[3];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = __float_as_uint(sum);
 }
-extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b3(uint32_t* out, uint32_t iters, uint32_t seed) {
+extern "C" __global__ __launch_bounds__(256, 4) void exl3_probe_decode_b3(uint32_t* out, uint32_t iters, uint32_t seed) {
     probe_decode_body<3>(out, iters, seed);
 }
-extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b4(uint32_t* out, uint32_t iters, uint32_t seed) {
+extern "C" __global__ __launch_bounds__(256, 4) void exl3_probe_decode_b4(uint32_t* out, uint32_t iters, uint32_t seed) {
     probe_decode_body<4>(out, iters, seed);
 }
-extern "C" __global__ __launch_bounds__(256) void exl3_probe_decode_b5(uint32_t* out, uint32_t iters, uint32_t seed) {
+extern "C" __global__ __launch_bounds__(256, 4) void exl3_probe_decode_b5(uint32_t* out, uint32_t iters, uint32_t seed) {
     probe_decode_body<5>(out, iters, seed);
 }
