@@ -642,6 +642,17 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
                                               "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
                                               "kept_bytes": ((n // 128 + 1) // 2) * 256 * k * 2}
     del lin, ws, y
+    # yardstick: the vendor library's f16 GEMM (torch.matmul -> hipBLASLt) of the same shape on this box, same timing loop.
+    # Launches of this size run against the board's power limit, not the MFMA's issue rate: the figure says what a tuned
+    # plain GEMM sustains here.
+    a16 = torch.randn((m, k), device="cuda", dtype=torch.float16)
+    w16 = torch.randn((n, k), device="cuda", dtype=torch.float16)
+    y16 = torch.empty((m, n), device="cuda", dtype=torch.float16)
+    ms = timed(lambda: torch.matmul(a16, w16.T, out=y16))
+    res["vendor_f16_gemm_5120x17408"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops / ms / 1e9, 1),
+                                         "frac_mfma_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                                         "what": "torch.matmul (hipBLASLt), f16 x f16^T, random normal operands"}
+    del a16, w16, y16
     # NVFP4
     fk = fp4.Kernels.load()
     flin = synth.fp4_linear(n, k, SEED, input_scale=1.0).upload()
