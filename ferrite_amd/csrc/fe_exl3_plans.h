@@ -12,13 +12,13 @@ struct FeTunedPlan {
 // clang-format off
 static const FeTunedPlan kFeTunedPlans[] = {
     // MI355X, 256 CUs: us at 1 row / 16 rows of the best candidates (graph-replayed, weights cycled past the caches)
-    {5120, 17408, 3, 256, 4, 2},  // occ 4 wk 2: 17.7 / 24.9; occ 3 wk 8: 18.2 / 23.8; occ 4 wk 8: 18.2 / 23.7
-    {17408, 5120, 3, 256, 3, 2},  // occ 3 wk 2: 19.3 / 26.7; occ 3 wk 8: 19.6 / 27.2; occ 4 wk 8: 19.6 / 27.2
-    {5120, 17408, 4, 256, 4, 2},  // occ 4 wk 2: 18.0 / 25.4; occ 5 wk 8: 18.5 / 24.2; occ 4 wk 8: 18.5 / 24.2
-    {17408, 5120, 4, 256, 3, 2},  // occ 3 wk 2: 19.7 / 27.1; occ 4 wk 8: 20.0 / 27.9; occ 5 wk 8: 20.0 / 28.0
-    {5120, 17408, 5, 256, 3, 8},  // occ 3 wk 8: 23.8 / 30.5; occ 2 wk 2: 24.0 / 29.9; occ 5 wk 8: 23.9 / 30.5
-    {17408, 5120, 5, 256, 2, 2},  // occ 2 wk 2: 24.0 / 30.5; occ 5 wk 8: 24.7 / 34.0; occ 3 wk 8: 24.7 / 33.9
-    {5120, 5120, 4, 256, 4, 4},   // occ 4 wk 4: 10.9 / 14.9; occ 5 wk 4: 10.9 / 15.0; occ 3 wk 4: 10.9 / 14.9
-    {5120, 1024, 4, 256, 4, 4},   // occ 3 wk 4: 8.2 / 12.1; occ 4 wk 4: 8.2 / 12.2; occ 2 wk 4: 8.2 / 12.2
+    {5120, 17408, 3, 256, 4, 2},  // occ 4 wk 2: 17.3 / 24.0; occ 3 wk 8: 18.0 / 23.2; occ 4 wk 8: 18.0 / 23.2
+    {17408, 5120, 3, 256, 3, 8},  // occ 3..5 wk 8 (680 programs, 17 a column block): 18.9 / 26.3; occ 3 wk 2: 19.1 / 26.0
+    {5120, 17408, 4, 256, 4, 2},  // occ 4 wk 2: 17.7 / 24.6; occ 4 wk 8: 18.3 / 23.6; occ 3 wk 8: 18.4 / 23.6
+    {17408, 5120, 4, 256, 3, 8},  // occ 3..5 wk 8: 19.1 / 26.7; occ 3 wk 2: 19.5 / 26.7
+    {5120, 17408, 5, 256, 3, 8},  // occ 3 wk 8: 20.1 / 25.8; occ 4 wk 8: 20.3 / 25.9; occ 4 wk 2: 20.1 / 27.4
+    {17408, 5120, 5, 256, 3, 8},  // occ 3..5 wk 8: 21.1 / 29.0; occ 3 wk 2: 21.3 / 28.7
+    {5120, 5120, 4, 256, 4, 4},   // occ 2..5 wk 4 (400 programs): 10.7 / 14.6
+    {5120, 1024, 4, 256, 4, 4},   // occ 2..5 wk 4 (80 programs): 8.1 / 11.9
 };
 // clang-format on

@@ -396,19 +396,6 @@ __device__ __forceinline__ uint32_t udiv_inv(uint32_t x, uint32_t d, uint32_t in
     return q + ((q + 1) * d <= x ? 1u : 0u);
 }
 
-// FE_STAMP builds (timeline probes, never the shipped code object) take one more kernel argument: 16 slots per program,
-// wall-clock stamps (100 MHz) written by thread 0 and the hardware id of the CU.
-#ifdef FE_STAMP
-#define FE_STAMP_ARG , uint64_t* stamps
-#define FE_STAMP_PASS , stamps
-#define FE_STAMP_AT(i) \
-    if (threadIdx.x == 0) stamps[(size_t)blockIdx.x * 16 + (i)] = __builtin_amdgcn_s_memrealtime()
-#else
-#define FE_STAMP_ARG
-#define FE_STAMP_PASS
-#define FE_STAMP_AT(i)
-#endif
-
 // The ring of load steps turned left by `phase` slots (phase < DEPTH), so that the oldest step in flight sits in slot 0
 // again: one pass of moves whatever the phase.
 template <int BITS, int DEPTH>
@@ -426,6 +413,15 @@ __device__ __forceinline__ void ring_turn(LaneWords<BITS> (&ring)[DEPTH], uint32
     }
 }
 
+// The word before a lane's run is the last word of the run of lane q - 1 of the same tile (q = lane & 7; for q = 0 the
+// tile's last word, lane q = 7): a move across lanes instead of a second load per step. The 16 lanes of a DPP row are the
+// two tiles of one k step, so lane i takes lane i - 1 (row_shr:1) or, at q = 0, lane i + 7 (row_ror:9).
+__device__ __forceinline__ uint32_t lane_prev_word(uint32_t last) {
+    const uint32_t shr = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)last, 0x111, 0xf, 0xf, false);
+    const uint32_t ror = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)last, 0x129, 0xf, 0xf, false);
+    return (threadIdx.x & 7) ? shr : ror;
+}
+
 // A lane's words of one load step through a buffer resource over the whole trellis: the lane's byte offsets (run, word
 // before the run) are loop constants in vector registers and the step's position is a scalar offset, so walking the run
 // costs no vector instructions; reads past the end of the trellis return zero instead of faulting. Streaming (nt) loads.
@@ -434,7 +430,8 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words_buf(__amdgpu_buffer_r
                                                                uint32_t soff) {
     constexpr int NT = 2;
     LaneWords<BITS> r;
-    r.w[0] = __builtin_amdgcn_raw_buffer_load_b32(rs, prev_b, soff, NT);
+    (void)prev_b;
+    r.w[0] = 0;  // the word before the run comes from the neighbouring lane when the step is decoded (lane_prev_word)
     if constexpr (BITS == 1) {
         r.w[1] = __builtin_amdgcn_raw_buffer_load_b32(rs, run_b, soff, NT);
     } else if constexpr (BITS == 2) {
@@ -464,18 +461,9 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words_buf(__amdgpu_buffer_r
 
 template <int BITS, int RG>
 __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uint32_t k, uint32_t m, uint32_t y_mode,
-                                           uint32_t chunk, uint32_t inv_spb, const RotSrc src FE_STAMP_ARG) {
+                                           uint32_t chunk, uint32_t inv_spb, const RotSrc src) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
-    FE_STAMP_AT(0);
-#ifdef FE_STAMP
-    if (threadIdx.x == 0) {
-        uint32_t hw = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_REG_HW_ID
-        uint32_t xcc = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // HW_REG_XCC_ID
-        stamps[(size_t)blockIdx.x * 16 + 8] = ((uint64_t)xcc << 32) | hw;
-        stamps[(size_t)blockIdx.x * 16 + 9] = __builtin_amdgcn_s_memtime();
-    }
-#endif
     constexpr uint32_t tw = 8 * BITS;
     constexpr int DEPTH = 4;  // load steps in flight per lane (8 measured slower: 22.9 against 20.7 us)
     constexpr int GROUP = 8;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
@@ -560,6 +548,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
 
     auto one = [&](LaneWords<BITS>& slot, uint32_t t) {  // t: load step within the staged chunk
         f16x8 op[2][2];
+        slot.w[0] = lane_prev_word(slot.w[BITS]);
         decode_lane<BITS>(slot, op);
         issue(slot);
         // keep the refill where it is issued: left alone, the scheduler sinks the loads to the end of the group, right in
@@ -590,7 +579,6 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
     // The segment of column block fnb that ends here: its sums meet in LDS, and then either are the block's sums (the
     // block lies in this run alone) or go to z for the program that arrives last at the block.
     auto flush = [&](uint32_t fnb) {
-        FE_STAMP_AT(2);
         __syncthreads();  // the previous segment's readers are done with `red`
         // rows 4 g .. 4 g + 3 of A are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32 (tile g >> 1 of
         // its pair, n = 4 (g & 1) + i + 8 h): a lane's four sums of either half are four neighbouring columns
@@ -628,16 +616,13 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
         float* zseg = mb.z + (size_t)(p + fnb) * m * 128;
         for (uint32_t row = hw; row < m; row += 8)
             store_agent_f32x4(zseg + row * 128 + 4 * l32, *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32));
-        FE_STAMP_AT(3);
         agent_stores_wait();
         __syncthreads();
-        FE_STAMP_AT(4);
         if (tid == 0) {
             uint32_t old = __hip_atomic_fetch_add(&mb.counters[fnb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             last_flag = (old == last_prog - first_prog);
         }
         __syncthreads();
-        FE_STAMP_AT(5);
         if (last_flag) {
             // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB segments each, 8 or 12 agent-scope
             // loads in flight (each takes a trip to memory: the trips overlap); every row's segments are added in program
@@ -682,7 +667,6 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
             else
                 rows_of(std::integral_constant<int, 2>{});
             if (tid == 0) __hip_atomic_store(&mb.counters[fnb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            FE_STAMP_AT(6);
         }
     };
 
@@ -731,7 +715,6 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
             }
         }
         __syncthreads();
-        if (c0 == 0) { FE_STAMP_AT(1); }
         // the chunk's load steps, segment by segment (a segment ends with its column block or with the chunk)
         uint32_t i = 0;
         while (i < cs) {
@@ -760,21 +743,17 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
         }
     }
     if (st) flush(nb);
-    FE_STAMP_AT(7);
-#ifdef FE_STAMP
-    if (threadIdx.x == 0) stamps[(size_t)blockIdx.x * 16 + 10] = __builtin_amdgcn_s_memtime();
-#endif
 }
 
 // (second launch bound: wavefronts per SIMD the registers must allow. Four programs a CU for up to 16 rows.)
 #define GEMVB_KERNEL(BITS, RG)                                                                                        \
-    extern "C" __global__ __launch_bounds__(256, RG == 1 ? 4 : 2) void exl3_gemvb_b##BITS##_r##RG(                                   \
+    extern "C" __global__ __launch_bounds__(256, RG == 1 ? 4 : 2) void exl3_gemvb_b##BITS##_r##RG(                    \
         GemvJob job, const void* x, const void* x2, uint32_t x_mode, uint32_t ldx, uint32_t k, uint32_t m,             \
-        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb FE_STAMP_ARG) {                                             \
+        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb) {                                                           \
         uint32_t i = 0;                                                                                               \
         while (i + 1 < job.count && blockIdx.x >= job.first[i + 1]) i++;                                              \
         gemvb_body<BITS, RG>(job.m[i], blockIdx.x - job.first[i], k, m, y_mode, chunk, inv_spb,                       \
-                             RotSrc{x, x2, x_mode, ldx} FE_STAMP_PASS);                                               \
+                             RotSrc{x, x2, x_mode, ldx});                                                             \
     }
 #define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
 GEMVB_FAMILY(2)
