@@ -46,6 +46,7 @@ struct fe_exl3_options {
     uint32_t group = 1;            // linears of one input share a launch (FE_EXL3_NO_GROUP=1: one launch each)
     uint32_t hat_rows = kHatRows;  // rows from which the prefill decodes once (FE_EXL3_HAT_ROWS; 0: never)
     uint32_t lds_pad = 1;          // LDS request that pins the programs per CU to the plan's occ (FE_EXL3_NO_LDS_PAD=1: off)
+    uint32_t fuse = 1;             // consecutive programs share a workgroup when a launch has more than the CUs hold (FE_EXL3_NO_FUSE=1: off)
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
 };
@@ -148,6 +149,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     o.group = env_u32("FE_EXL3_NO_GROUP", 0) ? 0 : 1;
     if (getenv("FE_EXL3_HAT_ROWS")) fe_exl3_kernels_set_option(k, "hat_rows", (uint32_t)std::max(0, atoi(getenv("FE_EXL3_HAT_ROWS"))));
     o.lds_pad = env_u32("FE_EXL3_NO_LDS_PAD", 0) ? 0 : 1;
+    o.fuse = env_u32("FE_EXL3_NO_FUSE", 0) ? 0 : 1;
     o.gemm_group_m = env_u32("FE_EXL3_GROUP", o.gemm_group_m);
     o.gemm_splits = env_u32("FE_GEMM_SPLITS", o.gemm_splits);
     if (!c) {
@@ -179,6 +181,7 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     else if (nm == "group") o.group = value;
     else if (nm == "hat_rows") o.hat_rows = value == 0 ? 0xffffffffu : std::max(value, kMaxRowsPerPass + 1);
     else if (nm == "lds_pad") o.lds_pad = value;
+    else if (nm == "fuse") o.fuse = value;
     else if (nm == "gemm_group_m") o.gemm_group_m = value;
     else if (nm == "gemm_splits") o.gemm_splits = value;
     else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
@@ -478,7 +481,17 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
                       int y_dtype, uint32_t rows, const fe_exl3_workspace *ws, const RotInput &in, const char *fn) {
     GemvJobArgs g{};
     g.count = (uint32_t)count;
-    uint32_t programs = 0, run_steps = 0;
+    const fe_exl3_kernels *kern = ls[0]->kern;
+    // Programs of the partition a workgroup runs one after the other (`fuse`): when the members' programs together are
+    // more than the CUs hold at once, consecutive programs share a workgroup instead of waiting for a free place, which
+    // saves the second one's start-up. The partition, and with it every sum, stays the member's own.
+    uint32_t occ = 0, total = 0;
+    for (size_t i = 0; i < count; i++) occ = std::max(occ, ls[i]->plan.occ), total += ls[i]->programs;
+    const uint32_t places = std::max(1u, (occ ? occ : 4) * std::max(kern->cus, 1u));
+    // (measured on gate + up, 4 bits: 34.1 against 35.6 us at 1 row, 36.8 / 38.2 at 4, even at 8, 44.8 / 41.9 at 16, where the
+    // longer run's inputs no longer fit the staging buffer in one piece: up to 4 rows)
+    uint32_t fuse = kern->opt.fuse && rows <= 4 ? std::min(4u, std::max(1u, (total + places - 1) / places)) : 1;
+    uint32_t programs = 0, run_steps = 0;  // (programs: workgroups of the launch)
     size_t z_at = 0, cnt_at = 0;
     char msg[200];
     for (size_t i = 0; i < count; i++) {
@@ -494,12 +507,12 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
         m.n = l->n, m.programs = l->programs;
         view_strides(l->view, &m.stride_k, &m.stride_nb);
         g.first[i] = programs;
-        programs += l->programs;
+        programs += (l->programs + fuse - 1) / fuse;
         z_at += job_z(l, rows), cnt_at += l->n / 128;
         const uint32_t units = (l->k / 128) * (l->n / 128);
         m.base = units / l->programs, m.rem = units % l->programs;
         m.inv_base = 0xffffffffu / m.base, m.inv_base1 = 0xffffffffu / (m.base + 1);
-        run_steps = std::max(run_steps, 2 * ((units + l->programs - 1) / l->programs));
+        run_steps = std::max(run_steps, 2 * fuse * ((units + l->programs - 1) / l->programs));
     }
     for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
     // staged inputs: the whole run where the LDS budget holds it for `rows` rows, else chunks of a multiple of 4 load steps
@@ -511,13 +524,10 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     // on, which would leave CUs empty while others hold 5; an LDS request that fits occ times into the CU's 160 KB, and
     // not occ + 1 times, makes the CUs take occ each.
     // (several linears: the most programs per CU any of them asks for)
-    const fe_exl3_kernels *kern = ls[0]->kern;
-    uint32_t occ = 0;
-    for (size_t i = 0; i < count; i++) occ = std::max(occ, ls[i]->plan.occ);
     if (occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
     uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld, inv_spb = 0xffffffffu / (k / 64);
     fe_devptr_t x = in.x, x2 = in.x2;
-    void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb};
+    void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb, &fuse};
     return fe_hip_launch(kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 

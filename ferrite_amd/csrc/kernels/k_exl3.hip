@@ -386,7 +386,7 @@ struct GemvMember {
     uint32_t inv_base, inv_base1;  // floor((2^32 - 1) / base), floor((2^32 - 1) / (base + 1))
 };
 struct GemvJob {
-    uint32_t count, first[FE_EXL3_GROUP_MAX + 1];  // member i owns programs first[i] .. first[i + 1] - 1 of the grid
+    uint32_t count, first[FE_EXL3_GROUP_MAX + 1];  // member i owns workgroups first[i] .. first[i + 1] - 1 of the grid
     GemvMember m[FE_EXL3_GROUP_MAX];
 };
 
@@ -460,7 +460,7 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words_buf(__amdgpu_buffer_r
 }
 
 template <int BITS, int RG>
-__device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uint32_t k, uint32_t m, uint32_t y_mode,
+__device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, uint32_t np, uint32_t k, uint32_t m, uint32_t y_mode,
                                            uint32_t chunk, uint32_t inv_spb, const RotSrc src) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
@@ -471,9 +471,15 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
     const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
     const uint32_t n = mb.n, spb = k / 64, upb = spb / 2;  // load steps, units a column block
     const uint32_t base = mb.base, rem = mb.rem;
-    const uint32_t u0 = p * base + (p < rem ? p : rem);
-    const uint32_t S = 2 * (base + (p < rem ? 1 : 0));  // load steps of this run
+    // This workgroup runs the programs p0 .. p0 + np - 1 of the partition one after the other. Their runs are contiguous, so
+    // to the loads and the staging they are one run; where one program's run ends its sums are flushed as that program's
+    // (its own slot in z, its own arrival), exactly as if it had been launched on its own: the same sums in the same
+    // order, without a second start-up.
+    auto run_start = [&](uint32_t q) { return q * base + (q < rem ? q : rem); };
+    const uint32_t u0 = run_start(p0);
+    const uint32_t S = 2 * (run_start(p0 + np) - u0);  // load steps of this workgroup's run
     if (S == 0) return;
+    uint32_t pl = p0, lend = 2 * (run_start(p0 + 1) - u0);  // the program at work and the load step at which its run ends
     uint32_t nb = udiv_inv(2 * u0, spb, inv_spb), st = 2 * u0 - nb * spb;  // where the run stands: column block, load step
     const uint32_t nb_run0 = nb, st_run0 = st;
 
@@ -578,7 +584,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
 
     // The segment of column block fnb that ends here: its sums meet in LDS, and then either are the block's sums (the
     // block lies in this run alone) or go to z for the program that arrives last at the block.
-    auto flush = [&](uint32_t fnb) {
+    auto flush = [&](uint32_t fnb, uint32_t p) {
         __syncthreads();  // the previous segment's readers are done with `red`
         // rows 4 g .. 4 g + 3 of A are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32 (tile g >> 1 of
         // its pair, n = 4 (g & 1) + i + 8 h): a lane's four sums of either half are four neighbouring columns
@@ -715,10 +721,11 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
             }
         }
         __syncthreads();
-        // the chunk's load steps, segment by segment (a segment ends with its column block or with the chunk)
+        // the chunk's load steps, segment by segment (a segment ends with its column block, with the chunk ...
         uint32_t i = 0;
         while (i < cs) {
-            const uint32_t seg = cs - i < spb - st ? cs - i : spb - st;
+            uint32_t seg = cs - i < spb - st ? cs - i : spb - st;
+            seg = seg < lend - (c0 + i) ? seg : lend - (c0 + i);  // ... or with the program's run
             // Whole groups of GROUP steps run as straight-line code: no branches inside, and the refill of a ring slot is
             // unconditional, so each load lands straight in the slot its words were just decoded from and only that
             // slot's next use waits for it. The wait at the top of a group has to cover every load in flight (the
@@ -735,24 +742,28 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p, uin
             }
             ring_turn<BITS, DEPTH>(ring, seg % DEPTH);
             i += seg, st += seg;
-            if (st == spb) {
-                flush(nb);
-                nb++, st = 0;
-                if (c0 + i < S) sv = *(const u32x2*)(mb.svh + nb * 128 + 4 * l32);  // the next block's output scales
+            const bool block_end = st == spb, run_end = c0 + i == lend;
+            if (block_end || run_end) {
+                flush(nb, pl);
+                if (block_end) {
+                    nb++, st = 0;
+                    if (c0 + i < S) sv = *(const u32x2*)(mb.svh + nb * 128 + 4 * l32);  // the next block's output scales
+                }
+                if (run_end) pl++, lend = 2 * (run_start(pl + 1) - u0);
             }
         }
     }
-    if (st) flush(nb);
 }
 
 // (second launch bound: wavefronts per SIMD the registers must allow. Four programs a CU for up to 16 rows.)
 #define GEMVB_KERNEL(BITS, RG)                                                                                        \
     extern "C" __global__ __launch_bounds__(256, RG == 1 ? 4 : 2) void exl3_gemvb_b##BITS##_r##RG(                    \
         GemvJob job, const void* x, const void* x2, uint32_t x_mode, uint32_t ldx, uint32_t k, uint32_t m,             \
-        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb) {                                                           \
+        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb, uint32_t fuse) {                                            \
         uint32_t i = 0;                                                                                               \
         while (i + 1 < job.count && blockIdx.x >= job.first[i + 1]) i++;                                              \
-        gemvb_body<BITS, RG>(job.m[i], blockIdx.x - job.first[i], k, m, y_mode, chunk, inv_spb,                       \
+        const uint32_t p0 = (blockIdx.x - job.first[i]) * fuse, left = job.m[i].programs - p0;                        \
+        gemvb_body<BITS, RG>(job.m[i], p0, left < fuse ? left : fuse, k, m, y_mode, chunk, inv_spb,                   \
                              RotSrc{x, x2, x_mode, ldx});                                                             \
     }
 #define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
