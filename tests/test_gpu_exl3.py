@@ -122,12 +122,10 @@ def check_linear(env, oracle, t, plan, strips, rows_list=ROWS, seed=1):
         if rows < 64:
             assert np.isnan(y[rows:]).all()
         if rows >= 5:  # row invariance (exl3-gemvcheck.rs:124-141): a row's bits do not depend on the row count
-            # (plan ver 2 sums rows 1..16 in the streamed order and 17..64 in the split order: invariant within each)
-            regime = 1 if (plan.ver == 2 and rows <= 16) else 0
-            if regime not in first5:
-                first5[regime] = y[:5].copy()
+            if 0 not in first5:
+                first5[0] = y[:5].copy()
             else:
-                assert np.array_equal(first5[regime].view(np.uint64), y[:5].view(np.uint64)), rows
+                assert np.array_equal(first5[0].view(np.uint64), y[:5].view(np.uint64)), rows
     # fused residual add: y (bf16, prefilled with 1.5) += x @ W, 5 rows (exl3-gemvcheck.rs:142-168)
     rows = 5
     pre = torch.full((mr, t.n), 1.5, dtype=torch.bfloat16, device="cuda")
@@ -447,7 +445,7 @@ def test_group_forward_has_the_bits_of_each_members_forward(env, bits, k, ns, sk
     """Linears of one input (q, k, v; gate, up) in one GEMV launch: every member's programs are those of its own launch,
     so each output has the bits of the member's forward(), for every row count, input and output type, with the input
     rotated inside the GEMV (one launch) or by one launch for all members (two). Groups that cannot share a launch
-    (different bits, a streamed plan, a workspace without the room) run member by member."""
+    (different bits, a workspace without the room) run member by member."""
     torch, exl3, kern = env
     from ferrite_amd import synth
     lins = []

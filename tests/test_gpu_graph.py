@@ -21,13 +21,13 @@ def test_forward_calls_replay_from_a_graph():
     kern, fk = exl3.Kernels.load(), fp4.Kernels.load()
     t = synth.exl3_tensor(1024, 384, 4, 5)
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 64)  # column blocks shared by several programs
-    streamed = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(7, 4, 4, 0))  # 7 uneven runs
+    uneven = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(7, 4, 4, 0))  # 7 uneven runs
     flin = synth.fp4_linear(384, 1024, 6).upload()
     # two more linears of the same input: with `lin` a grouped launch (the argument block is copied at capture)
     pair = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(1024, n, 4, 30 + n)), 64) for n in (256, 128)]
     group = [lin] + pair
     rows = [1, 16, 40, 300]
-    ws = exl3.Workspace([lin, streamed] + pair, max(rows))
+    ws = exl3.Workspace([lin, uneven] + pair, max(rows))
     assert exl3.forward_group_launches(group, 1, ws) in (1, 2) and exl3.forward_group_launches(group, 16, ws) in (1, 2)
     fws = fp4.Workspace(max(rows), 1024)
     xs = {m: dev_u16(torch, synth.activations(m, 1024, m)) for m in rows}
@@ -36,7 +36,7 @@ def test_forward_calls_replay_from_a_graph():
         for m in rows:
             lin.forward(xs[m], exl3.Dtype.Bf16, outs[("e", m)], exl3.Dtype.F32, m, ws, stream=stream)
             flin.forward(fk, fws, outs[("f", m)], 384, xs[m], 1024, m, stream=stream)
-        streamed.forward(xs[16], exl3.Dtype.Bf16, outs[("s", 16)], exl3.Dtype.F32, 16, ws, stream=stream)
+        uneven.forward(xs[16], exl3.Dtype.Bf16, outs[("s", 16)], exl3.Dtype.F32, 16, ws, stream=stream)
         for m in (1, 16):
             exl3.forward_group(group, xs[m], exl3.Dtype.Bf16, [outs[("g", m, i)] for i in range(3)], exl3.Dtype.F32, m, ws, stream=stream)
 
