@@ -12,9 +12,9 @@ crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step, launch gaps and i
 weight sets total 401 MB, more than L2 plus the 256 MB Infinity Cache, so every step streams its weights from HBM.
 
 `roofline` is the dominant kernel alone (the 4-bit GEMV launch of the two 5120x17408 projections): its trellis bytes
-over its average launch duration, measured with HIP event pairs on the launch stream around its launches inside the
-timed region (the other launches of the timed region carry no events: every record is a packet of its own on the queue;
-a pass after the timed region brackets all six launches for `per_launch`). It also carries the single 5120x17408 linear
+over its average launch duration, measured with HIP event pairs on the launch stream in a second pass of the same K
+steps in which every launch carries such a pair (which is also where `per_launch` comes from; `value` is taken from the
+first pass, without events: a pair costs the eager step 3.5 us a launch). It also carries the single 5120x17408 linear
 the target names and the measured decode-only ceiling of the vector ALUs (`alu_ceiling_GBs`), which splits the distance to
 the HBM roofline into "ceiling against HBM" and "kernel against ceiling".
 `cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host;
@@ -229,15 +229,15 @@ def main():
                      (f_rotated, (d.h, stream, ws.xh_ptr, yd.data_ptr(), bf16, 1, ws.h))]
         launches.append((f"down_b{bits}", d.weight_bytes(), False, len(calls), calls, None))
 
-    # Event pairs on the launch stream. In the timed region only the dominant kernel's launches carry them; one more pass
-    # after the timed region times every launch for the per-launch table. A pair is attached to the dispatch of the
-    # launch's last kernel (the GEMV), so it reads that kernel's own begin and end as a kernel trace does
-    # (fe_hip_time_next_launch); with --bracket-events it is recorded before and after the launch instead, each record
-    # a packet of its own on the queue, which adds the dispatch gap and the packets to the reading.
+    # Event pairs on the launch stream, one per launch of a second pass of the same K steps. A pair is attached to the dispatch of the
+    # launch's last kernel (the GEMV), so it reads that kernel's own begin and end as a kernel trace does and puts no
+    # packets of its own on the queue (fe_hip_time_next_launch); every launch carries one, because a timed dispatch that
+    # follows an untimed one takes its start when it is accepted, while the launch before it still drains (3-4 us too
+    # long). With --bracket-events the pairs are recorded before and after the launch instead, each record a packet
+    # of its own on the queue, which adds the dispatch gap and the packets to the reading.
     attached = not args.bracket_events
     f_time_next = lib.fe_hip_time_next_launch
-    events = [[(ev.new(), ev.new()) if la[2] else None for la in launches] for _ in range(args.steps)]
-    table_events = [(ev.new(), ev.new()) for _ in launches]
+    events = [[(ev.new(), ev.new()) for _ in launches] for _ in range(args.steps)]
 
     def step(pairs=None):
         rc = 0
@@ -262,11 +262,18 @@ def main():
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step(events[i])
+        step()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     ms_per_step = dt * 1e3 / args.steps
     value = total_bytes / (dt / args.steps) / 1e9
+    # the same K steps once more with an event pair on every launch, for the roofline kernel's own duration and the
+    # per-launch table (the pairs cost the eager step 3.5 us a launch, so `value` is taken without them)
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    ms_per_step_timed = (time.perf_counter() - t0) * 1e3 / args.steps
 
     dom_ms = []
     for li, la in enumerate(launches):
@@ -277,14 +284,9 @@ def main():
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
 
-    per, reps = {}, max(args.steps, 5)
-    acc = [0.0] * len(launches)
-    for _ in range(reps):  # after the timed region: every launch bracketed
-        step(table_events)
-        for li in range(len(launches)):
-            acc[li] += ev.ms(*table_events[li])
-    for li, la in enumerate(launches):
-        us = acc[li] / reps * 1e3
+    per = {}
+    for li, la in enumerate(launches):  # every launch of the timed region, by its own events
+        us = sum(ev.ms(*events[i][li]) for i in range(args.steps)) / args.steps * 1e3
         per[la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
 
     # The dominant launch and the single linear the target names, each alone and back to back between one pair of
@@ -335,6 +337,7 @@ def main():
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": ROOFLINE_TRAFFIC_BYTES, "traffic_source": ROOFLINE_TRAFFIC_SOURCE,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms),
+                     "timed_in": f"a second pass of the {args.steps} steps with an event pair on every launch ({ms_per_step_timed:.5f} ms a step)",
                      "back_to_back_cold_us": round(dom_b2b_us, 3),
                      "events": "recorded around the launch" if args.bracket_events else "attached to the kernel's dispatch",
                      "alu_ceiling_GBs": ceiling,
