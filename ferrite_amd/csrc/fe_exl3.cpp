@@ -16,7 +16,7 @@
 namespace {
 
 constexpr uint32_t kMaxRowsPerPass = 64;       // 4 row groups of 16
-constexpr uint32_t kHatRows = 513;             // rows from which the prefill decodes once into fp16 tiles (3 output tile rows)
+constexpr uint32_t kHatRows = 2048;            // rows from which the prefill decodes once into fp16 tiles (8 output tile rows)
 constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
 constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH

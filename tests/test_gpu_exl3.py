@@ -553,7 +553,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     o = to_oracle(oracle, t)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
-    kern.set_option("hat_rows", 513)
+    kern.set_option("hat_rows", 2048)
 
 
 def test_prefill_over_kept_decoded_weights(env, oracle):
