@@ -49,6 +49,7 @@ struct fe_exl3_options {
     uint32_t fuse = 1;             // consecutive programs share a workgroup when a launch has more than the CUs hold (FE_EXL3_NO_FUSE=1: off)
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
+    uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
 };
 
 struct fe_exl3_kernels {
@@ -58,10 +59,10 @@ struct fe_exl3_kernels {
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemvb[6][4] = {};                               // the decode GEMV, [bits slot][row groups - 1]
     uint32_t cus = 0;
-    fe_function_t gemm[6] = {};
+    fe_function_t gemm[6] = {}, gemm_sk[6] = {};  // decode inside the GEMM: one piece a program / stream-K
     fe_function_t gemm_reduce = nullptr;
     fe_function_t hat_tiles[6] = {};  // trellis -> fp16 weights as the GEMM's LDS images
-    fe_function_t gemm_hat = nullptr; // the GEMM over them
+    fe_function_t gemm_hat = nullptr, gemm_hat_sk = nullptr;  // the GEMM over them
     fe_exl3_options opt;
 };
 
@@ -137,12 +138,17 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
+        snprintf(nm, sizeof nm, "exl3_gemm_b%d_sk", kBits[i]);
+        get(&k->gemm_sk[i], nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm_sk[i], kGemmLds);
         snprintf(nm, sizeof nm, "exl3_hat_tiles_b%d", kBits[i]);
         get(&k->hat_tiles[i], nm);
         if (i == 0) get(&k->gemm_reduce, "exl3_gemm_reduce");
     }
     get(&k->gemm_hat, "exl3_gemm_hat");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm_hat, kGemmLds);
+    get(&k->gemm_hat_sk, "exl3_gemm_hat_sk");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm_hat_sk, kGemmLds);
     fe_exl3_options &o = k->opt;
     o.fused_rot = env_u32("FE_EXL3_NO_FUSED_ROT", 0) ? 0 : 1;
     o.fused_rot_pairs = env_u32("FE_EXL3_FUSED_ROT_PAIRS", o.fused_rot_pairs);
@@ -152,6 +158,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     o.fuse = env_u32("FE_EXL3_NO_FUSE", 0) ? 0 : 1;
     o.gemm_group_m = env_u32("FE_EXL3_GROUP", o.gemm_group_m);
     o.gemm_splits = env_u32("FE_GEMM_SPLITS", o.gemm_splits);
+    o.gemm_sk = env_u32("FE_GEMM_SK", o.gemm_sk);
     if (!c) {
         int cus = 0;
         c = fe_hip_cu_count(&cus);
@@ -184,6 +191,7 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     else if (nm == "fuse") o.fuse = value;
     else if (nm == "gemm_group_m") o.gemm_group_m = value;
     else if (nm == "gemm_splits") o.gemm_splits = value;
+    else if (nm == "gemm_sk") o.gemm_sk = value;
     else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
     return 0;
 }
@@ -358,13 +366,14 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     };
     const uint32_t gemv_rows = std::min(max_rows, kMaxRowsPerPass);
     ws->z_len = std::max<size_t>(top(zs) * gemv_rows, 4);
-    ws->counters_len = std::max<size_t>(top(nbs), 1);
+    int cus = 0, c = 0;
+    if (max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
+    // arrival counters: a word a column block of the linears of one launch (GEMV); a word an output tile (stream-K GEMM)
+    ws->counters_len = std::max<size_t>({top(nbs), (size_t)4 * cus, 1});
     // (rotated inputs: one linear's at max_rows, or those of the linears of one launch at up to 64 rows each)
-    int c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * gemv_rows) * max_k * 2);
+    if (!c) c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * gemv_rows) * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
-    int cus = 0;
-    if (!c && max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
     if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes);
     // zeroed once: the unused half of the last tile of an odd count of column blocks is read (and its sums discarded)
     if (!c && max_rows >= hat_rows && max_hat) c = ws->hat.zeroed(max_hat);
@@ -432,24 +441,24 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear_gemv_rotated", "rotated input of 4 GB or more");
     const uint32_t tiles_m = (rows + 255) / 256, tiles_n = (n / 128 + 1) / 2;
     if (group == 0 || group > tiles_m) group = tiles_m;
-    FeGemmSplit g = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes),
-                                  kern->opt.gemm_splits);
-    uint32_t full = g.full, splits = g.splits;
+    FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
+                                          ws->counters_len, kern->opt.gemm_splits, kern->opt.gemm_sk);
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
     const bool kept = l->hat.bytes != 0;  // decoded once and kept: any row count above the GEMV's runs over it
     if (kept || (rows >= kern->opt.hat_rows && ws->hat.bytes >= hat_bytes(l))) {
         fe_devptr_t hat = kept ? l->hat.p : ws->hat.p;
         if (!kept) FE_TRY(launch_decode(l, s, hat));
         group = 0;  // the raster that deals column tiles to the XCDs: each decoded weight panel goes through one L2
-        void *args[] = {&xh, &hat, &svh, &y, &n, &k, &rows, &mode, &group, &full, &splits, &part};
-        FE_TRY(fe_hip_launch(kern->gemm_hat, g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+        void *args[] = {&xh, &hat, &svh, &y, &n, &k, &rows, &mode, &group, &sch.args};
+        FE_TRY(fe_hip_launch(sch.stream_k ? kern->gemm_hat_sk : kern->gemm_hat, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     } else {
-        void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &full, &splits, &part};
-        FE_TRY(fe_hip_launch(kern->gemm[bits_slot(l->bits)], g.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+        void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &sch.args};
+        FE_TRY(fe_hip_launch((sch.stream_k ? kern->gemm_sk : kern->gemm)[bits_slot(l->bits)], sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     }
-    if (!g.cut()) return 0;
+    if (sch.stream_k || !sch.split.cut()) return 0;
+    uint32_t full = sch.split.full, splits = sch.split.splits;
     void *rargs[] = {&part, &svh, &y, &n, &rows, &mode, &group, &full, &splits};
-    return fe_hip_launch(kern->gemm_reduce, g.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
+    return fe_hip_launch(kern->gemm_reduce, sch.split.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 // The GEMV can rotate its own input: every program rotates the channels of its own run, (row, 128-channel block) pairs,

@@ -23,6 +23,7 @@ struct fe_fp4_kernels {
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4[3] = {nullptr, nullptr, nullptr};
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
+    fe_function_t gemm4_sk = nullptr, gemm8_sk = nullptr, gemm8c_sk = nullptr;  // the same on the stream-K schedule
     uint32_t cus = 0;
     // Switches of the launch paths: read from the environment once, at load; fe_fp4_kernels_set_option changes them
     // afterwards. No forward call reads the environment.
@@ -32,6 +33,7 @@ struct fe_fp4_kernels {
     int32_t xcd = -1;          // column tiles dealt to the XCDs: -1 = where the weights are the larger operand (FE_FP4_XCD)
     uint32_t fp8_f16 = 0;      // FP8 linears as fp16 expansion on the 16-bit matrix instruction (FE_FP8_F16=1)
     uint32_t gemm_splits = 8;  // most pieces a cut output tile takes (FE_GEMM_SPLITS; 1: never cut)
+    int32_t gemm_sk = 1;       // stream-K schedule of the GEMMs: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
 };
 
 struct fe_fp4_linear {
@@ -72,6 +74,12 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->gemm8c, k->module, "fe_gemm_fp8_codes");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8c, kGemmLds);
+    struct { fe_function_t *f; const char *nm; } sks[] = {
+        {&k->gemm4_sk, "fe_gemm_nvfp4_sk"}, {&k->gemm8_sk, "fe_gemm_fp8_sk"}, {&k->gemm8c_sk, "fe_gemm_fp8_codes_sk"}};
+    for (auto &e : sks) {
+        if (!c) c = fe_hip_module_get_function(e.f, k->module, e.nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(*e.f, kGemmLds);
+    }
     if (!c) c = fe_hip_module_get_function(&k->swiglu4, k->module, "fe_gemm_nvfp4_swiglu");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->swiglu4, kGemmLds);
     if (!c) c = fe_hip_module_get_function(&k->swiglu_reduce4, k->module, "fe_gemm_nvfp4_swiglu_reduce");
@@ -84,6 +92,7 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (const char *e = getenv("FE_FP4_XCD")) k->xcd = atoi(e) ? 1 : 0;
     if (const char *e = getenv("FE_FP8_F16")) k->fp8_f16 = atoi(e) ? 1 : 0;
     if (const char *e = getenv("FE_GEMM_SPLITS")) k->gemm_splits = (uint32_t)atoi(e);
+    if (const char *e = getenv("FE_GEMM_SK")) k->gemm_sk = atoi(e);
     if (c) {
         fe_fp4_kernels_destroy(k);
         return c;
@@ -108,6 +117,7 @@ int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value
     else if (nm == "xcd") k->xcd = value;
     else if (nm == "fp8_f16") k->fp8_f16 = value ? 1 : 0;
     else if (nm == "gemm_splits") k->gemm_splits = (uint32_t)value;
+    else if (nm == "gemm_sk") k->gemm_sk = value;
     else return fe_set_error(FE_ERR_ARG, "fe_fp4_kernels_set_option", name);
     return 0;
 }
@@ -331,26 +341,29 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     // FP8 runs on the 8-bit matrix instruction over the codes of both operands, k tiles of 128 (FE_FP8_F16=1: the fp16
     // expansion on the 16-bit instruction, k tiles of 64; same products, another order of the f32 sums)
     const bool codes8 = l->fp8 && !kern->fp8_f16;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes),
-                                   kern->gemm_splits);
-    uint32_t full = gs.full, splits = gs.splits;
-    fe_devptr_t part = ws->part.p;
+    FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, ws->part.p, ws->part.bytes,
+                                          ws->counters.p, kGemvCounters, kern->gemm_splits, kern->gemm_sk);
+    // stream-K programs sit at different depths of K: one row tile at a time (column tiles fastest) keeps those that are
+    // in step on one panel of activations
+    if (sch.stream_k && kern->xcd < 0) group = 1;
     float scale = l->fp8 ? 1.0f : 0.0625f;  // what the fp16 expansions of the two operands carry (FP4_OPERAND_SCALE)
     if (codes8) {
         fe_devptr_t codes = ws->codes.p;
-        void *args8[] = {&y, &codes, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &full, &splits, &part};
-        FE_TRY(fe_hip_launch(kern->gemm8c, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args8));
+        void *args8[] = {&y, &codes, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &sch.args};
+        FE_TRY(fe_hip_launch(sch.stream_k ? kern->gemm8c_sk : kern->gemm8c, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args8));
     } else if (l->fp8) {
-        void *args8[] = {&y, &aq, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &full, &splits, &part};
-        FE_TRY(fe_hip_launch(kern->gemm8, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args8));
+        void *args8[] = {&y, &aq, &w, &alpha, &res, &m, &n, &k, &ldy, &group, &w_snt, &w_skt, &w_sr, &sch.args};
+        FE_TRY(fe_hip_launch(sch.stream_k ? kern->gemm8_sk : kern->gemm8, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args8));
     } else {
-        void *args[] = {&y,     &aq,    &w,    &sw,    &alpha, &res,  &m,      &n,   &k, &ldy,
-                        &group, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr, &full, &splits, &part};
-        FE_TRY(fe_hip_launch(kern->gemm4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
+        void *args[] = {&y,     &aq,    &w,     &sw,   &alpha, &res,   &m,    &n,       &k,
+                        &ldy,   &group, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr, &sch.args};
+        FE_TRY(fe_hip_launch(sch.stream_k ? kern->gemm4_sk : kern->gemm4, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     }
-    if (!gs.cut()) return 0;
+    if (sch.stream_k || !sch.split.cut()) return 0;
+    uint32_t full = sch.split.full, splits = sch.split.splits;
+    fe_devptr_t part = ws->part.p;
     void *rargs[] = {&y, &part, &alpha, &res, &m, &n, &ldy, &group, &full, &splits, &scale};
-    return fe_hip_launch(kern->reduce4, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
+    return fe_hip_launch(kern->reduce4, sch.split.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }
 
 int fe_fp4_linear_forward(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_stream_t s, const fe_fp4_workspace *ws,
@@ -381,12 +394,14 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
     fe_devptr_t aq = ws->aq.p, w = l->w.p, sw = l->sw.p, alpha = l->alpha.p, part = ws->part.p;
     fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
-    FeGemmSplit gs = fe_gemm_split(tiles_m * tiles_n, k / 64, kern->cus, (uint32_t)(ws->part.bytes / kFeGemmPartBytes), kern->gemm_splits);
+    FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
+                                          kGemvCounters, kern->gemm_splits, 0);  // (this kernel has the one-piece form only)
+    void *args[] = {&aq,    &w,     &sw,    &alpha, &m,       &n,       &k,    &group, &w_snt, &w_skt,
+                    &w_sr,  &s_snt, &s_skt, &s_sr,  &sch.args, &q_codes, &q_sf, &q_aq,  &down_g};
+    FE_TRY(fe_hip_launch(kern->swiglu4, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
+    if (sch.stream_k || !sch.split.cut()) return 0;
+    const FeGemmSplit &gs = sch.split;
     uint32_t full = gs.full, splits = gs.splits;
-    void *args[] = {&aq,    &w,     &sw,   &alpha, &m,    &n,      &k,    &group,   &w_snt, &w_skt, &w_sr,
-                    &s_snt, &s_skt, &s_sr, &full,  &splits, &part, &q_codes, &q_sf, &q_aq,  &down_g};
-    FE_TRY(fe_hip_launch(kern->swiglu4, gs.programs(), 1, 1, 256, 1, 1, kGemmLds, s, args));
-    if (!gs.cut()) return 0;
     void *rargs[] = {&part, &alpha, &m, &n, &group, &full, &splits, &q_codes, &q_sf, &q_aq, &down_g};
     return fe_hip_launch(kern->swiglu_reduce4, gs.cut() * 64, 1, 1, 256, 1, 1, 0, s, rargs);
 }

@@ -113,3 +113,53 @@ inline FeGemmSplit fe_gemm_split(uint32_t tiles, uint32_t ktiles, uint32_t cus, 
     g.splits = best;
     return g;
 }
+
+// The schedule argument of the GEMM kernels (GemmSched of kernels/gemm_core.h) and what to launch with it.
+struct FeGemmSchedArgs {
+    uint32_t full_tiles, splits, sk_base, sk_rem;
+    fe_devptr_t part;
+    uint32_t part_bytes, pad_;
+    fe_devptr_t counters;
+};
+struct FeGemmSchedule {
+    FeGemmSplit split;     // the one-piece schedule (when !stream_k): its cut tiles need the reduce launch
+    FeGemmSchedArgs args;
+    uint32_t programs = 0;
+    bool stream_k = false;
+};
+// mode 0: always one piece a program. mode 2: stream-K wherever the workspace allows (tests). mode 1: stream-K where
+// it is the faster schedule, as measured (MI355X, NVFP4 and EXL3, 20..1088 tiles): all of
+//  * fewer tiles than CUs, and the best cut of the one-piece schedule leaves a partly filled round (160 tiles on 256
+//    CUs: three pieces a tile are 480 programs; with 128, 192 or 224 tiles a cut fills its rounds and stream-K has
+//    nothing to gain);
+//  * at most three pieces a tile (runs of at least half a tile): the piece that arrives last adds the others alone,
+//    which takes about 5 us a piece;
+//  * equal runs, and programs 8 apart (the same XCD) in step, i.e. at the same depth of K at the same time: they then
+//    share operand panels in their L2. Without it every program streams its own operands past the L2 and the GEMM runs
+//    10..25 % slower than the one-piece schedule, whose programs all walk K in step (240 tiles: 579 against 479 us).
+// 160 tiles (2048 rows x 5120 columns): 5..14 % faster than the one-piece schedule. With a whole round or more of tiles
+// the one-piece schedule wins (5120 x 17408 at 2048 rows: 2..10 %). Needs two partial slots a program and a zeroed
+// counter a tile.
+constexpr uint32_t kFeXcds = 8;
+inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t cus, fe_devptr_t part, size_t part_bytes,
+                                       fe_devptr_t counters, size_t counters_len, uint32_t cap, int mode) {
+    FeGemmSchedule r;
+    const uint32_t slots = (uint32_t)(part_bytes / kFeGemmPartBytes);
+    r.split = fe_gemm_split(tiles, ktiles, cus, slots, cap);
+    r.programs = r.split.programs();
+    r.args = {r.split.full, r.split.splits, 0, 0, part, (uint32_t)std::min<size_t>(part_bytes, 0xffffffffu), 0, counters};
+    const uint64_t units = (uint64_t)tiles * ktiles;
+    const uint32_t programs = (uint32_t)std::min<uint64_t>({cus, units, slots / 2});
+    if (!mode || !programs || !counters || tiles > counters_len || units >= (1ull << 31) ||
+        (size_t)programs * 2 * kFeGemmPartBytes > 0xffffffffu)
+        return r;
+    const uint32_t base = (uint32_t)(units / programs), rem = (uint32_t)(units % programs);
+    if (mode == 1 && !(tiles < cus && rem == 0 && 2 * base >= ktiles && (kFeXcds * base) % ktiles == 0 &&
+                       (r.split.cut() * r.split.splits) % cus != 0))
+        return r;
+    if (base >= ktiles && rem == 0 && base % ktiles == 0) return r;  // whole tiles only: nothing to gain
+    r.stream_k = true;
+    r.programs = programs;
+    r.args.sk_base = base, r.args.sk_rem = rem;
+    return r;
+}

@@ -462,3 +462,135 @@ __device__ __forceinline__ void gemm_reduce_rows(const float* __restrict__ part,
     float v[4] = {sum[0], sum[1], sum[2], sum[3]};
     fn(t, row, cb, l32, v);
 }
+
+// ---- Stream-K schedule -------------------------------------------------------------------------------------------------
+// The tiles' k tiles, laid end to end in raster order (tile-major, K ascending), are one sequence of units; program p of P
+// takes the contiguous run of base = units / P of them (+ 1 for the first units % P programs), so every program does the
+// same work to within one k tile whatever the tile count, and there is no mostly empty last round and no reduce launch.
+// A run crosses tile boundaries: each piece of a tile (segment) is one pass of the main loop. A tile that lies in one
+// run is finished there. Otherwise its pieces meet through the workspace: a piece that is not the last to arrive leaves
+// its accumulators in a slot (two slots a program: one for a run's first segment, one for its last) and bumps the tile's
+// arrival counter; the piece whose arrival completes the count adds the pieces in piece order, starting from zero, with
+// its own accumulators in their place, and finishes the tile: the sums do not depend on which piece came last. The
+// hand-off is the decode GEMV's: write-through stores, acknowledged, then a relaxed agent-scope atomic; the reader's loads
+// bypass its L2; counters return to zero.
+#define GM_PART_BYTES (GM_PART_FLOATS * 4)
+
+__device__ __forceinline__ uint32_t sk_start(uint32_t p, uint32_t base, uint32_t rem) { return p * base + (p < rem ? p : rem); }
+// the program whose run holds unit u
+__device__ __forceinline__ uint32_t sk_owner(uint32_t u, uint32_t base, uint32_t rem) {
+    const uint32_t big = rem * (base + 1);
+    return u < big ? u / (base + 1) : rem + (u - big) / base;
+}
+
+// Program p has worked through k tiles of tile `tile` (units t0 .. t0 + ktiles - 1) that other programs share. Returns
+// true if this program finishes the tile, with the sum of all pieces in acc; false if it has left its piece in the
+// workspace. Every branch is uniform over the workgroup. lds: free (the main loop ended with a barrier).
+__device__ __forceinline__ bool gemm_sk_meet(f32x16 (&acc)[4][4], uint32_t p, uint32_t tile, uint32_t t0, uint32_t ktiles,
+                                             uint32_t base, uint32_t rem, float* part, uint32_t part_bytes, uint32_t* counters,
+                                             unsigned char* lds) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t first = sk_owner(t0, base, rem), last = sk_owner(t0 + ktiles - 1, base, rem);
+    const uint32_t n = last - first + 1, me = p - first;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)part, 0, part_bytes, 0x00020000);
+    volatile uint32_t* flag = (volatile uint32_t*)lds;
+    uint32_t* cnt = counters + tile;
+    // a run's piece of a tile in which the run does not begin is the run's last segment
+    auto slot_of = [&](uint32_t q) { return 2 * q + (sk_start(q, base, rem) < t0 ? 1u : 0u); };
+    if (tid == 0) *flag = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    uint32_t seen = *flag;
+    __syncthreads();
+    if (seen != n - 1) {  // someone is still at work: leave the piece
+        const uint32_t so = slot_of(p) * GM_PART_BYTES;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const f32x4 v = {acc[i][j][4 * e], acc[i][j][4 * e + 1], acc[i][j][4 * e + 2], acc[i][j][4 * e + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, v), rs, tid * 16,
+                                                           so + ((i * 4 + j) * 4 + e) * 4096, 16);
+                }
+        agent_stores_wait();
+        __syncthreads();
+        if (tid == 0) *flag = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        seen = *flag;
+        __syncthreads();
+        if (seen != n - 1) return false;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f32x4 t[16];
+#pragma unroll
+        for (int c = 0; c < 16; c++) t[c] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (uint32_t q = 0; q < n; q++) {
+            if (q == me) {
+#pragma unroll
+                for (int c = 0; c < 16; c++)
+                    t[c] += (f32x4){acc[i][c >> 2][4 * (c & 3)], acc[i][c >> 2][4 * (c & 3) + 1], acc[i][c >> 2][4 * (c & 3) + 2],
+                                    acc[i][c >> 2][4 * (c & 3) + 3]};
+            } else {
+                const uint32_t so = slot_of(first + q) * GM_PART_BYTES + i * 16 * 4096;
+                f32x4 ld[16];
+#pragma unroll
+                for (int c = 0; c < 16; c++) ld[c] = load_agent_f32x4(rs, tid * 16, so + c * 4096);
+#pragma unroll
+                for (int c = 0; c < 16; c++) t[c] += ld[c];
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 16; c++)
+#pragma unroll
+            for (int x = 0; x < 4; x++) acc[i][c >> 2][4 * (c & 3) + x] = t[c][x];
+    }
+    if (tid == 0) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
+// How a GEMM launch is spread over its programs. sk_base == 0: one piece a program (gemm_work: whole tiles, then the
+// cut tiles, whose partials a reduce kernel adds). Otherwise stream-K: grid = the programs, runs of sk_base (+ 1 for the
+// first sk_rem) k tiles; part holds two slots a program, counters one word a tile, zero at rest.
+struct GemmSched {
+    uint32_t full_tiles, splits, sk_base, sk_rem;
+    float* part;
+    uint32_t part_bytes;
+    uint32_t* counters;
+};
+
+// Runs the program's share of the schedule: main(tm, tn, kt0, ktn, acc) is one pass of the main loop over k tiles
+// kt0 .. kt0 + ktn - 1 of tile (tm, tn), finish(tm, tn, acc) the tile's epilogue. One call site of each, whatever the
+// schedule. SK picks the schedule at compile time (a kernel that holds both spills around its 256 accumulators):
+// sc.sk_base must be nonzero exactly when SK.
+template <bool SK, class Main, class Finish>
+__device__ __forceinline__ void gemm_schedule(const GemmSched& sc, uint32_t tiles_m, uint32_t tiles_n, uint32_t group,
+                                              uint32_t ktiles, unsigned char* lds, Main main, Finish finish) {
+    const uint32_t p = blockIdx.x;
+    f32x16 acc[4][4];
+    if constexpr (!SK) {
+        const GemmWork wk = gemm_work(p, tiles_m, tiles_n, group, ktiles, sc.full_tiles, sc.splits);
+        main(wk.tm, wk.tn, wk.kt0, wk.ktn, acc);
+        if (wk.partial)
+            gemm_store_partial(acc, lds, sc.part + (size_t)wk.slot * GM_PART_FLOATS);
+        else
+            finish(wk.tm, wk.tn, acc);
+    } else {
+        uint32_t u = sk_start(p, sc.sk_base, sc.sk_rem);
+        const uint32_t uend = sk_start(p + 1, sc.sk_base, sc.sk_rem);
+        while (u < uend) {
+            const uint32_t tile = u / ktiles, t0 = tile * ktiles, kt0 = u - t0;
+            const uint32_t ktn = ktiles - kt0 < uend - u ? ktiles - kt0 : uend - u;
+            uint32_t tm, tn;
+            gemm_raster(tile, tiles_m, tiles_n, group, tm, tn);
+            __syncthreads();  // the epilogue of the segment before is done with the LDS
+            main(tm, tn, kt0, ktn, acc);
+            bool fin = true;
+            if (ktn != ktiles)
+                fin = gemm_sk_meet(acc, p, tile, t0, ktiles, sc.sk_base, sc.sk_rem, sc.part, sc.part_bytes, sc.counters, lds);
+            if (fin) finish(tm, tn, acc);
+            u += ktn;
+        }
+    }
+}

@@ -812,64 +812,62 @@ struct Exl3Producer {
 
 // y[m][n] (+)= H(xh @ W_hat) * svh / sqrt(128) for prefill-sized m: xh fp16 [m][k] (rotated inputs), 256 x 256 output
 // tiles; a wavefront's 128 columns are exactly one Hadamard block, so the output rotation is local to the wavefront.
-// grid full_tiles + (tiles - full_tiles) * splits with tiles = ceil(m / 256) * ceil(n / 256) (grouped raster), 256
-// threads, dynamic LDS GM_LDS_TILES (the epilogue reuses it). Tiles past full_tiles leave partials in `part` for
-// exl3_gemm_reduce. make_producer(tn) builds the weight producer of 256-column tile tn.
-template <class MakeProducer>
+// Tiles = ceil(m / 256) * ceil(n / 256) (grouped raster), spread over the grid as sc says (gemm_schedule): one piece a
+// program, the cut tiles finished by exl3_gemm_reduce, or stream-K. 256 threads, dynamic LDS GM_LDS_TILES (the epilogue
+// reuses it). make_producer(tn) builds the weight producer of 256-column tile tn.
+template <bool SK, class MakeProducer>
 __device__ __forceinline__ void exl3_gemm_tile(const _Float16* __restrict__ xh, const uint16_t* __restrict__ svh, void* y,
                                                uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, uint32_t group_m,
-                                               uint32_t full_tiles, uint32_t splits, float* part,
-                                               MakeProducer make_producer) {
+                                               const GemmSched& sched, MakeProducer make_producer) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t nbs = n / 128;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nbs + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
-    const uint32_t m0 = wk.tm * GM_BM, tn = wk.tn;
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    auto prod = make_producer(tn);
-    f32x16 acc[4][4];
-    gemm_mainloop(xh, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
-    if (wk.partial) {
-        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
-        return;
-    }
-    const uint32_t nb = 2 * tn + wn;
-    if (nb >= nbs) return;
-    const uint32_t col = nb * 128 + 4 * (lane & 31);
-    const f32x4 sc = row_scales(svh, col);
-    // one copy of the epilogue per output mode, so that the row loop has no mode branches
-    auto run = [&](auto mode_tag) {
-        constexpr uint32_t MODE = decltype(mode_tag)::value;
-        gemm_epilogue(
-            acc, lds,
-            [&](float (&v)[4][4], uint32_t l32) {
-                fwht128_half_wave_rows(v, l32);
+    gemm_schedule<SK>(
+        sched, (m + GM_BM - 1) / GM_BM, (nbs + 1) / 2, group_m, k / GM_BK, lds,
+        [&](uint32_t tm, uint32_t tn, uint32_t kt0, uint32_t ktn, f32x16(&acc)[4][4]) {
+            auto prod = make_producer(tn);
+            gemm_mainloop(xh, k, m, kt0, ktn, tm * GM_BM, prod, lds, acc);
+        },
+        [&](uint32_t tm, uint32_t tn, f32x16(&acc)[4][4]) {
+            const uint32_t m0 = tm * GM_BM, nb = 2 * tn + wn;
+            if (nb >= nbs) return;
+            const uint32_t col = nb * 128 + 4 * (lane & 31);
+            const f32x4 sc = row_scales(svh, col);
+            // one copy of the epilogue per output mode, so that the row loop has no mode branches
+            auto run = [&](auto mode_tag) {
+                constexpr uint32_t MODE = decltype(mode_tag)::value;
+                gemm_epilogue(
+                    acc, lds,
+                    [&](float (&v)[4][4], uint32_t l32) {
+                        fwht128_half_wave_rows(v, l32);
 #pragma unroll
-                for (int u = 0; u < 4; u++)
+                        for (int u = 0; u < 4; u++)
 #pragma unroll
-                    for (int e = 0; e < 4; e++) v[u][e] = v[u][e] * FE_HAD_SCALE * sc[e];  // finish_row's products
-            },
-            [&](uint32_t row, uint32_t, float (&v)[4]) {
-                uint32_t grow = m0 + wm * 128 + row;
-                if (grow < m) store4(y, MODE, (size_t)grow * n + col, v);
-            });
-    };
-    if (y_mode == 0)
-        run(std::integral_constant<uint32_t, 0>{});
-    else if (y_mode == 1)
-        run(std::integral_constant<uint32_t, 1>{});
-    else if (y_mode == 2)
-        run(std::integral_constant<uint32_t, 2>{});
-    else
-        run(std::integral_constant<uint32_t, 3>{});
+                            for (int e = 0; e < 4; e++) v[u][e] = v[u][e] * FE_HAD_SCALE * sc[e];  // finish_row's products
+                    },
+                    [&](uint32_t row, uint32_t, float (&v)[4]) {
+                        uint32_t grow = m0 + wm * 128 + row;
+                        if (grow < m) store4(y, MODE, (size_t)grow * n + col, v);
+                    });
+            };
+            if (y_mode == 0)
+                run(std::integral_constant<uint32_t, 0>{});
+            else if (y_mode == 1)
+                run(std::integral_constant<uint32_t, 1>{});
+            else if (y_mode == 2)
+                run(std::integral_constant<uint32_t, 2>{});
+            else
+                run(std::integral_constant<uint32_t, 3>{});
+        });
 }
 
 // The GEMM decoding the trellis itself: every 256-row tile of the output decodes its weights again.
-template <int BITS>
+template <int BITS, bool SK>
 __device__ __forceinline__ void exl3_gemm_body(const _Float16* __restrict__ xh, const uint32_t* __restrict__ trellis,
                                                const uint16_t* __restrict__ svh, void* y, uint32_t n, uint32_t k, uint32_t m,
                                                uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m,
-                                               uint32_t full_tiles, uint32_t splits, float* part) {
-    exl3_gemm_tile(xh, svh, y, n, k, m, y_mode, group_m, full_tiles, splits, part, [&](uint32_t tn) {
+                                               const GemmSched& sched) {
+    exl3_gemm_tile<SK>(xh, svh, y, n, k, m, y_mode, group_m, sched, [&](uint32_t tn) {
         constexpr uint32_t tw = 8 * BITS;
         const uint32_t lane = threadIdx.x & 63, nbs = n / 128;
         Exl3Producer<BITS> prod;
@@ -957,15 +955,23 @@ struct HatProducer {
     }
 };
 
-extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_hat(const _Float16* xh, const unsigned char* hat,
-                                                                   const uint16_t* svh, void* y, uint32_t n, uint32_t k,
-                                                                   uint32_t m, uint32_t y_mode, uint32_t group_m,
-                                                                   uint32_t full_tiles, uint32_t splits, float* part) {
-    exl3_gemm_tile(xh, svh, y, n, k, m, y_mode, group_m, full_tiles, splits, part, [&](uint32_t tn) {
+// (every GEMM kernel comes as NAME, one piece a program, and NAME_sk, stream-K, with the same parameters)
+#define HAT_GEMM_PARAMS                                                                                                  \
+    const _Float16 *xh, const unsigned char *hat, const uint16_t *svh, void *y, uint32_t n, uint32_t k, uint32_t m, uint32_t y_mode, \
+        uint32_t group_m, GemmSched sched
+template <bool SK>
+__device__ __forceinline__ void exl3_gemm_hat_kernel(HAT_GEMM_PARAMS) {
+    exl3_gemm_tile<SK>(xh, svh, y, n, k, m, y_mode, group_m, sched, [&](uint32_t tn) {
         HatProducer prod;
         prod.base = hat + (size_t)tn * (k / GM_BK) * GM_B_BYTES + 16 * threadIdx.x;
         return prod;
     });
+}
+extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_hat(HAT_GEMM_PARAMS) {
+    exl3_gemm_hat_kernel<false>(xh, hat, svh, y, n, k, m, y_mode, group_m, sched);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_hat_sk(HAT_GEMM_PARAMS) {
+    exl3_gemm_hat_kernel<true>(xh, hat, svh, y, n, k, m, y_mode, group_m, sched);
 }
 
 // Finishes the tiles that exl3_gemm_b* cut along K: sums their partial slots and applies the output rotation and scale.
@@ -982,14 +988,15 @@ extern "C" __global__ __launch_bounds__(256) void exl3_gemm_reduce(const float* 
     });
 }
 
-#define GEMM_KERNEL(BITS)                                                                                              \
-    extern "C" __global__ __launch_bounds__(256, 1) void exl3_gemm_b##BITS(                                            \
+#define GEMM_KERNEL_(NAME, BITS, SK)                                                                                   \
+    extern "C" __global__ __launch_bounds__(256, 1) void NAME(                                                         \
         const _Float16* xh, const uint32_t* trellis, const uint16_t* svh, void* y, uint32_t n, uint32_t k, uint32_t m,  \
-        uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m, uint32_t full_tiles, uint32_t splits, \
-        float* part) {                                                                                                 \
-        exl3_gemm_body<BITS>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m, full_tiles, splits,    \
-                             part);                                                                                    \
+        uint32_t y_mode, uint32_t stride_k, uint32_t stride_nb, uint32_t group_m, GemmSched sched) {                    \
+        exl3_gemm_body<BITS, SK>(xh, trellis, svh, y, n, k, m, y_mode, stride_k, stride_nb, group_m, sched);           \
     }
+#define GEMM_KERNEL(BITS)                       \
+    GEMM_KERNEL_(exl3_gemm_b##BITS, BITS, false) \
+    GEMM_KERNEL_(exl3_gemm_b##BITS##_sk, BITS, true)
 #define HAT_KERNEL(BITS)                                                                                      \
     extern "C" __global__ __launch_bounds__(256) void exl3_hat_tiles_b##BITS(                                 \
         const uint32_t* trellis, unsigned char* hat, uint32_t k, uint32_t stride_k, uint32_t stride_nb) {     \

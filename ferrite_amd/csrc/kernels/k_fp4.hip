@@ -358,29 +358,33 @@ __device__ __forceinline__ void fp_store_piece(const FpOut& o, const float (&v)[
 }
 
 // C[M][ldc] = bf16((A_q . W_q^T) * alpha[n]) (+ res: bf16(bf16(.) + res)); A_q = the fp16 operand of the quantizer,
-// W_q expanded by the producer; `scale` = 1 / (the factors the two fp16 expansions carry). grid full_tiles +
-// (tiles - full_tiles) * splits with tiles = ceil(M / 256) * ceil(N / 256) (grouped raster), 256 threads, dynamic LDS
-// GM_LDS_TILES. Tiles past full_tiles leave partials in `part` for the reduce kernel. N % 128 == 0, K % 128 == 0.
-// (kernels/k-fp4/src/lib.rs:285-470)
-template <class Producer, bool SWIGLU>
-__device__ __forceinline__ void fp_gemm_body(Producer& prod, const FpOut& out, const _Float16* aq, const float* alpha,
-                                             float scale, uint32_t m, uint32_t n, uint32_t k, const GemmWork& wk, float* part) {
+// W_q expanded by the producer make_prod(tn) of 256-column tile tn; `scale` = 1 / (the factors the two fp16 expansions
+// carry). Tiles = ceil(M / 256) * ceil(N / 256) (grouped raster), spread over the grid as sc says (gemm_schedule): one
+// piece a program, the cut tiles finished by the reduce kernel, or stream-K. 256 threads, dynamic LDS GM_LDS_TILES.
+// N % 128 == 0, K % 128 == 0. (kernels/k-fp4/src/lib.rs:285-470)
+template <bool SWIGLU, bool SK, class MakeProd>
+__device__ __forceinline__ void fp_gemm_body(MakeProd make_prod, const FpOut& out, const _Float16* aq, const float* alpha,
+                                             float scale, uint32_t m, uint32_t n, uint32_t k, uint32_t group_m,
+                                             const GemmSched& sc) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-    const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
     const uint32_t tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    f32x16 acc[4][4];
-    gemm_mainloop(aq, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
-    if (wk.partial) {
-        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
-        return;
-    }
-    const uint32_t colb = n0 + wn * 128;
-    if (colb >= n) return;
-    const uint32_t col = colb + 4 * (tid & 31);
-    const f32x4 al = *(const f32x4*)(alpha + col) * scale;
-    gemm_epilogue(
-        acc, lds, [](float (&)[4][4], uint32_t) {},
-        [&](uint32_t row, uint32_t l32, float (&v)[4]) { fp_store_piece<SWIGLU>(out, v, al, l32, m0 + wm * 128 + row, m, col, n); });
+    gemm_schedule<SK>(
+        sc, (m + GM_BM - 1) / GM_BM, (n / 128 + 1) / 2, group_m, k / GM_BK, lds,
+        [&](uint32_t tm, uint32_t tn, uint32_t kt0, uint32_t ktn, f32x16(&acc)[4][4]) {
+            auto prod = make_prod(tn);
+            gemm_mainloop(aq, k, m, kt0, ktn, tm * GM_BM, prod, lds, acc);
+        },
+        [&](uint32_t tm, uint32_t tn, f32x16(&acc)[4][4]) {
+            const uint32_t m0 = tm * GM_BM, colb = tn * GM_BN + wn * 128;
+            if (colb >= n) return;
+            const uint32_t col = colb + 4 * (tid & 31);
+            const f32x4 al = *(const f32x4*)(alpha + col) * scale;
+            gemm_epilogue(
+                acc, lds, [](float (&)[4][4], uint32_t) {},
+                [&](uint32_t row, uint32_t l32, float (&v)[4]) {
+                    fp_store_piece<SWIGLU>(out, v, al, l32, m0 + wm * 128 + row, m, col, n);
+                });
+        });
 }
 
 // Finishes the tiles that a GEMM kernel cut along K. grid (tiles - full_tiles) * 64, 256 threads.
@@ -414,18 +418,23 @@ __device__ __forceinline__ Fp4Producer fp4_producer(const uint8_t* w, const uint
 
 // NVFP4: the codes of row r = 128 nt + i, k tile kt are 32 bytes at w + nt * w_snt + kt * w_skt + i * w_sr, its 4 scales
 // at sw + nt * s_snt + kt * s_skt + i * s_sr.
-extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(uint16_t* c, const _Float16* aq, const uint8_t* w,
-                                                                   const uint8_t* sw, const float* alpha, const uint16_t* res,
-                                                                   uint32_t m, uint32_t n, uint32_t k, uint32_t ldc,
-                                                                   uint32_t group_m, uint32_t w_snt, uint32_t w_skt,
-                                                                   uint32_t w_sr, uint32_t s_snt, uint32_t s_skt,
-                                                                   uint32_t s_sr, uint32_t full_tiles, uint32_t splits,
-                                                                   float* part) {
-    const uint32_t nts = n / 128;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
-    Fp4Producer prod = fp4_producer(w, sw, wk.tn, nts, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
+// Every GEMM kernel comes in two forms, NAME (one piece a program) and NAME_sk (stream-K), with the same parameters.
+#define FP4_GEMM_PARAMS                                                                                                    \
+    uint16_t *c, const _Float16 *aq, const uint8_t *w, const uint8_t *sw, const float *alpha, const uint16_t *res, uint32_t m, \
+        uint32_t n, uint32_t k, uint32_t ldc, uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, \
+        uint32_t s_skt, uint32_t s_sr, GemmSched sc
+template <bool SK>
+__device__ __forceinline__ void gemm_nvfp4_kernel(FP4_GEMM_PARAMS) {
     FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
-    fp_gemm_body<Fp4Producer, false>(prod, out, aq, alpha, FP4_OPERAND_SCALE, m, n, k, wk, part);
+    fp_gemm_body<false, SK>(
+        [&](uint32_t tn) { return fp4_producer(w, sw, tn, n / 128, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr); }, out, aq, alpha,
+        FP4_OPERAND_SCALE, m, n, k, group_m, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4(FP4_GEMM_PARAMS) {
+    gemm_nvfp4_kernel<false>(c, aq, w, sw, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_sk(FP4_GEMM_PARAMS) {
+    gemm_nvfp4_kernel<true>(c, aq, w, sw, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr, sc);
 }
 
 extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t* c, const float* part, const float* alpha,
@@ -442,12 +451,11 @@ extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t*
 extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_swiglu(
     const _Float16* aq, const uint8_t* w, const uint8_t* sw, const float* alpha, uint32_t m, uint32_t n, uint32_t k,
     uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt, uint32_t s_sr,
-    uint32_t full_tiles, uint32_t splits, float* part, uint8_t* q_codes, uint8_t* q_sf, _Float16* q_aq, float qg) {
-    const uint32_t nts = n / 128;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
-    Fp4Producer prod = fp4_producer(w, sw, wk.tn, nts, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
+    GemmSched sc, uint8_t* q_codes, uint8_t* q_sf, _Float16* q_aq, float qg) {  // (one piece a program only)
     FpOut out = {nullptr, nullptr, 0, q_codes, q_sf, q_aq, qg};
-    fp_gemm_body<Fp4Producer, true>(prod, out, aq, alpha, FP4_OPERAND_SCALE, m, n, k, wk, part);
+    fp_gemm_body<true, false>(
+        [&](uint32_t tn) { return fp4_producer(w, sw, tn, n / 128, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr); }, out, aq, alpha,
+        FP4_OPERAND_SCALE, m, n, k, group_m, sc);
 }
 
 extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_swiglu_reduce(const float* part, const float* alpha, uint32_t m,
@@ -460,21 +468,30 @@ extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_swiglu_reduce(co
 
 // FP8: the 64 codes of row r = 128 nt + i, k tile kt are at w + nt * w_snt + kt * w_skt + i * w_sr; both fp16 expansions
 // are the values themselves. Finished by fe_gemm_nvfp4_reduce with scale 1. (kernels/k-fp4/src/lib.rs:472-484)
-extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8(uint16_t* c, const _Float16* aq, const uint8_t* w,
-                                                                 const float* alpha, const uint16_t* res, uint32_t m, uint32_t n,
-                                                                 uint32_t k, uint32_t ldc, uint32_t group_m, uint32_t w_snt,
-                                                                 uint32_t w_skt, uint32_t w_sr, uint32_t full_tiles,
-                                                                 uint32_t splits, float* part) {
+#define FP8_GEMM_PARAMS                                                                                                     \
+    uint16_t *c, const _Float16 *aq, const uint8_t *w, const float *alpha, const uint16_t *res, uint32_t m, uint32_t n, uint32_t k, \
+        uint32_t ldc, uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, GemmSched sc
+template <bool SK>
+__device__ __forceinline__ void gemm_fp8_kernel(FP8_GEMM_PARAMS) {
     const uint32_t nts = n / 128, tid = threadIdx.x;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / GM_BK, full_tiles, splits);
-    uint32_t nt = 2 * wk.tn + (tid >> 7);
-    nt = nt < nts ? nt : nts - 1;
-    Fp8Producer prod;
-    prod.row = tid;
-    prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
-    prod.w_skt = w_skt;
     FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
-    fp_gemm_body<Fp8Producer, false>(prod, out, aq, alpha, 1.0f, m, n, k, wk, part);
+    fp_gemm_body<false, SK>(
+        [&](uint32_t tn) {
+            uint32_t nt = 2 * tn + (tid >> 7);
+            nt = nt < nts ? nt : nts - 1;
+            Fp8Producer prod;
+            prod.row = tid;
+            prod.w = w + (size_t)nt * w_snt + (size_t)(tid & 127) * w_sr;
+            prod.w_skt = w_skt;
+            return prod;
+        },
+        out, aq, alpha, 1.0f, m, n, k, group_m, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8(FP8_GEMM_PARAMS) {
+    gemm_fp8_kernel<false>(c, aq, w, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_sk(FP8_GEMM_PARAMS) {
+    gemm_fp8_kernel<true>(c, aq, w, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, sc);
 }
 
 // The same linear on the 8-bit matrix instruction: activations are the quantizer's e4m3 codes [M][K], weights stay codes
@@ -508,38 +525,45 @@ struct Fp8CodeProducer {
     }
 };
 
-extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_codes(uint16_t* c, const uint8_t* aq, const uint8_t* w,
-                                                                       const float* alpha, const uint16_t* res, uint32_t m,
-                                                                       uint32_t n, uint32_t k, uint32_t ldc, uint32_t group_m,
-                                                                       uint32_t w_snt, uint32_t w_skt, uint32_t w_sr,
-                                                                       uint32_t full_tiles, uint32_t splits, float* part) {
+#define FP8C_GEMM_PARAMS                                                                                                   \
+    uint16_t *c, const uint8_t *aq, const uint8_t *w, const float *alpha, const uint16_t *res, uint32_t m, uint32_t n, uint32_t k, \
+        uint32_t ldc, uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, GemmSched sc
+template <bool SK>
+__device__ __forceinline__ void gemm_fp8_codes_kernel(FP8C_GEMM_PARAMS) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const uint32_t nts = n / 128, tid = threadIdx.x, wave = tid >> 6, wm = wave >> 1, wn = wave & 1;
-    const GemmWork wk = gemm_work(blockIdx.x, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / 128, full_tiles, splits);
-    const uint32_t m0 = wk.tm * GM_BM, n0 = wk.tn * GM_BN;
-    Fp8CodeProducer prod;
-    const uint32_t chunk = tid & 7, row = tid >> 3;
-#pragma unroll
-    for (int b = 0; b < 2; b++) {
-        uint32_t nt = 2 * wk.tn + b;
-        nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program copies its first tile twice
-        prod.w[b] = w + (size_t)nt * w_snt + (size_t)(chunk >> 2) * w_skt + (size_t)row * w_sr + (chunk & 3) * 16;
-    }
-    prod.w_skt = w_skt, prod.w_sr = w_sr, prod.st = gm_swz(row, chunk);
-    f32x16 acc[4][4];
-    gemm_mainloop_f8(aq, k, m, wk.kt0, wk.ktn, m0, prod, lds, acc);
-    if (wk.partial) {
-        gemm_store_partial(acc, lds, part + (size_t)wk.slot * GM_PART_FLOATS);
-        return;
-    }
-    const uint32_t colb = n0 + wn * 128;
-    if (colb >= n) return;
-    const uint32_t col = colb + 4 * (tid & 31);
-    const f32x4 al = *(const f32x4*)(alpha + col);
     FpOut out = {c, res, ldc, nullptr, nullptr, nullptr, 0.f};
-    gemm_epilogue(
-        acc, lds, [](float (&)[4][4], uint32_t) {},
-        [&](uint32_t r, uint32_t l32, float (&v)[4]) { fp_store_piece<false>(out, v, al, l32, m0 + wm * 128 + r, m, col, n); });
+    gemm_schedule<SK>(
+        sc, (m + GM_BM - 1) / GM_BM, (nts + 1) / 2, group_m, k / 128, lds,
+        [&](uint32_t tm, uint32_t tn, uint32_t kt0, uint32_t ktn, f32x16(&acc)[4][4]) {
+            Fp8CodeProducer prod;
+            const uint32_t chunk = tid & 7, row = tid >> 3;
+#pragma unroll
+            for (int b = 0; b < 2; b++) {
+                uint32_t nt = 2 * tn + b;
+                nt = nt < nts ? nt : nts - 1;  // an odd count of 128-row tiles: the last program copies its first tile twice
+                prod.w[b] = w + (size_t)nt * w_snt + (size_t)(chunk >> 2) * w_skt + (size_t)row * w_sr + (chunk & 3) * 16;
+            }
+            prod.w_skt = w_skt, prod.w_sr = w_sr, prod.st = gm_swz(row, chunk);
+            gemm_mainloop_f8(aq, k, m, kt0, ktn, tm * GM_BM, prod, lds, acc);
+        },
+        [&](uint32_t tm, uint32_t tn, f32x16(&acc)[4][4]) {
+            const uint32_t m0 = tm * GM_BM, colb = tn * GM_BN + wn * 128;
+            if (colb >= n) return;
+            const uint32_t col = colb + 4 * (tid & 31);
+            const f32x4 al = *(const f32x4*)(alpha + col);
+            gemm_epilogue(
+                acc, lds, [](float (&)[4][4], uint32_t) {},
+                [&](uint32_t r, uint32_t l32, float (&v)[4]) {
+                    fp_store_piece<false>(out, v, al, l32, m0 + wm * 128 + r, m, col, n);
+                });
+        });
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_codes(FP8C_GEMM_PARAMS) {
+    gemm_fp8_codes_kernel<false>(c, aq, w, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_fp8_codes_sk(FP8C_GEMM_PARAMS) {
+    gemm_fp8_codes_kernel<true>(c, aq, w, alpha, res, m, n, k, ldc, group_m, w_snt, w_skt, w_sr, sc);
 }
 
 // ---- GEMV (1..48 rows) -------------------------------------------------------------------------------------------------

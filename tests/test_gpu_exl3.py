@@ -284,6 +284,55 @@ def test_prefill_gemm_matches_the_oracle(env, oracle, bits, m):
         assert (np.abs(got[:m] - lin64) / np.maximum(np.abs(lin64), np.sqrt((lin64 ** 2).mean()))).max() < 1e-2
 
 
+def test_prefill_on_the_stream_k_schedule(env, oracle):
+    """Stream-K: the prefill GEMM walks the tiles' k tiles laid end to end, every program a contiguous run; the pieces of
+    a tile meet through the workspace and the last arriver adds them in piece order. 2400 x 3968 over K = 1024: 10 x 16 =
+    160 tiles of 16 k tiles, the case the library picks the schedule for by itself on 256 CUs; the last row tile ragged,
+    the last column tile half. Option gemm_sk = 1 gives the bits of the forced schedule (2); repeats give the same bits
+    (arrival order does not matter, counters return to zero); the one-piece schedule (0) differs by the order of the
+    f32 sums; both the decoding GEMM and the GEMM over decoded tiles; an add output mode; against the oracle."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    m = 2400
+    t = synth.exl3_tensor(1024, 3968, 4, 77)
+    xd = dev_u16(torch, synth.activations(m, t.k, 8, outliers=True))
+    lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 256)
+    kern.set_option("hat_rows", 65)
+    ws = exl3.Workspace([lin], m)
+
+    def run(sk, hat, dt=exl3.Dtype.F32, pre=float("nan")):
+        kern.set_option("gemm_sk", sk)
+        kern.set_option("hat_rows", 65 if hat else 0)
+        y = torch.full((m + 1, t.n), pre, dtype=torch.float32, device="cuda")
+        lin.forward(xd, exl3.Dtype.Bf16, y, dt, m, ws)
+        torch.cuda.synchronize()
+        out = y.cpu().numpy()
+        assert np.array_equal(out[m].view(np.uint32), np.full(t.n, pre, dtype=np.float32).view(np.uint32))
+        return out[:m]
+
+    try:
+        o = to_oracle(oracle, t)
+        ref = None
+        for hat in (False, True):
+            forced = run(2, hat)
+            for _ in range(5):
+                assert np.array_equal(run(2, hat).view(np.uint32), forced.view(np.uint32)), hat
+            assert np.array_equal(run(1, hat).view(np.uint32), forced.view(np.uint32)), hat
+            pieces = run(0, hat)
+            rms = np.sqrt((pieces.astype(np.float64) ** 2).mean())
+            assert np.abs(forced.astype(np.float64) - pieces).max() < 2e-6 * rms, hat
+            added = run(2, hat, exl3.Dtype.F32Add, 0.25)
+            want = forced.astype(np.float64) + 0.25  # (the add is fused into the last product: one rounding, not two)
+            assert (np.abs(added - want) <= (np.abs(want) + np.abs(forced)) * 2.0 ** -23).all(), hat
+            rows = [0, 1, 17, 255, 256, 1023, 1024, 2047, 2048, 2303, 2304, m - 1]
+            if ref is None:
+                ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k)[rows])
+            assert np.abs(forced[rows].astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4, hat
+    finally:
+        kern.set_option("gemm_sk", 1)
+        kern.set_option("hat_rows", 2048)
+
+
 def test_argument_errors_are_results_not_crashes(env):
     torch, exl3, kern = env
     from ferrite_amd import synth
@@ -510,8 +559,10 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     """Many rows: the trellis is decoded once into fp16 tiles (the GEMM's own LDS images) and the GEMM copies them instead
     of decoding per output tile row. Same fragments and MFMA order, so with whole tiles the same bits in every output
     mode; the two forms walk the tiles in different orders, so with a last round cut along K other tiles are the cut
-    ones and those differ by the order of their f32 sums. The "hat_rows" option moves the row count from which this form
-    runs (0: never). 2304 and 4224 columns: 9 and 17 column tiles, dealt to the XCDs in bands of 8."""
+    ones and those differ by the order of their f32 sums (so do the tiles that the stream-K schedule shares between
+    programs, which is forced here for the pass that compares within a tolerance). The "hat_rows" option moves the row
+    count from which this form runs (0: never). 2304 and 4224 columns: 9 and 17 column tiles, dealt to the XCDs in bands
+    of 8."""
     torch, exl3, kern = env
     from ferrite_amd import synth
     m = 600
@@ -529,6 +580,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
 
     for splits in (None, "1"):
         kern.set_option("gemm_splits", int(splits) if splits else 8)
+        kern.set_option("gemm_sk", 0 if splits else 2)
         for rows in (65, 300, 600):
             for dt, tdt, pre in ((exl3.Dtype.F32, torch.float32, float("nan")), (exl3.Dtype.Bf16, torch.bfloat16, 7.0),
                                  (exl3.Dtype.Bf16Add, torch.bfloat16, 1.5), (exl3.Dtype.F32Add, torch.float32, 0.25)):
@@ -545,6 +597,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
                     assert np.all(np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * rms), (rows, dt)
                 assert (tiles[rows:] == tiles[m]).all()  # rows past `rows` keep the prefill
     kern.set_option("gemm_splits", 8)
+    kern.set_option("gemm_sk", 1)
     # and against the oracle
     kern.set_option("hat_rows", 65)
     y = torch.zeros((m, t.n), dtype=torch.float32, device="cuda")

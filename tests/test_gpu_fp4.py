@@ -149,6 +149,64 @@ def test_fp4_gemm_tiles_cut_or_whole_and_views(env, oracle):
     assert np.array_equal(got, want)
 
 
+def test_gemm_on_the_stream_k_schedule(env, oracle):
+    """Stream-K: the GEMM walks the tiles' k tiles laid end to end, every program a contiguous run, and the pieces of a
+    tile meet through the workspace with the last arriver adding them in piece order. 2400 x 3968 over K = 1024 is
+    10 x 16 = 160 tiles of 16 k tiles (8 for FP8 codes), the case the library picks the schedule for by itself on 256 CUs
+    (fewer tiles than CUs, no cut that fills its rounds): option gemm_sk = 1 gives the bits of the forced schedule (2),
+    repeats give the same bits (arrival order does not matter, counters are back at zero), the one-piece schedule (0)
+    differs by the order of the f32 sums only; NVFP4 and both FP8 forms, the residual epilogue, rows past m untouched,
+    a ragged last row tile and a half last column tile (3968 = 15.5 x 256)."""
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    n, k, m = 3840 + 128, 1024, 2400
+    rng = np.random.default_rng(12)
+    res = dev_u16(torch, bf16_bits(rng.normal(size=(m + 2, n)).astype(np.float32)))
+    for kind in ("nvfp4", "fp8", "fp8_f16"):
+        host = synth.fp8_linear(n, k, 31, input_scale=0.05) if kind != "nvfp4" else synth.fp4_linear(n, k, 31, input_scale=1.0)
+        host.alpha[:] = host.alpha * np.linspace(0.5, 2.0, n).astype(np.float32)
+        lin = host.upload()
+        ws = fp4.Workspace(m, k)
+        xd = dev_u16(torch, fp4_check_activations(m, k, lin.g, 5))
+        kern.set_option("fp8_f16", 1 if kind == "fp8_f16" else 0)
+
+        def run(sk, r=None):
+            kern.set_option("gemm_sk", sk)
+            y = torch.full((m + 2, n), -3.0, dtype=torch.bfloat16, device="cuda")
+            lin.forward(kern, ws, y, n, xd, k, m, res=r)
+            torch.cuda.synchronize()
+            out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+            assert (out[m:] == bf16_bits(np.float32([-3.0]))[0]).all()
+            return out[:m]
+
+        try:
+            forced = run(2)
+            for _ in range(5):
+                assert np.array_equal(run(2), forced), kind
+            assert np.array_equal(run(1), forced), kind  # the library's own choice for this shape
+            pieces = run(0)
+            a, b = bf16_to_f32(forced).astype(np.float64), bf16_to_f32(pieces).astype(np.float64)
+            assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * np.abs(b).max()).all(), kind
+            got = run(2, r=res)
+            assert np.array_equal(got, bf16_bits(bf16_to_f32(forced) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m]))), kind
+        finally:
+            kern.set_option("gemm_sk", 1)
+            kern.set_option("fp8_f16", 0)
+        # against the f64 reference over the quantized operands
+        rows = [0, 1, 17, 255, 256, 1023, 1024, 2047, 2048, 2303, 2304, m - 1]
+        if kind == "nvfp4":
+            codes, sf_tiled = ws.read(m, k)
+            sfa = oracle.untile_scales(sf_tiled, m, k // 16).reshape(m, k // 16)
+            ref = oracle.ref_gemm(oracle.dequant_fp4(codes[rows], sfa[rows], 1.0), oracle.dequant_fp4(host.codes, host.sf, 1.0))
+        else:
+            codes = ws.read_fp8(m, k)
+            ref = oracle.ref_gemm(np.stack([oracle.dequant_fp8_row(codes[r], 1.0) for r in rows]),
+                                  np.stack([oracle.dequant_fp8_row(host.codes[c], 1.0) for c in range(n)]))
+        ref = ref.astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+        scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+        assert (np.abs(a[rows] - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2, kind
+
+
 def test_fp4_gemv_agrees_with_the_gemm(env, oracle):
     """Up to 64 rows run the weight-read-bound GEMV (up to 48 rows a pass, K cut over several programs); option gemv = 0
     sends the same rows through the GEMM. Both sum the same exact products in f32, in different orders; within the GEMV a
