@@ -715,7 +715,12 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     flin_d.quantize(fk, fws_d, x, kd, m)
     ms = timed(lambda: flin_d.gemm(fk, fws_d, y, nd, m))
     res["nvfp4_17408x5120"] = {"gemm_ms": round(ms, 4), "TFLOP/s": round(flops_d / ms / 1e9, 1),
-                               "frac_mfma_peak": round(flops_d / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4)}
+                               "frac_mfma_peak": round(flops_d / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4),
+                               "schedule": "stream-K (160 tiles on %d CUs)" % exl3.cu_count()}
+    # the same launch on the one-piece schedule (tiles cut three ways along K, partials added by a reduce kernel)
+    fk.set_option("gemm_sk", 0)
+    res["nvfp4_17408x5120"]["one_piece_schedule_ms"] = round(timed(lambda: flin_d.gemm(fk, fws_d, y, nd, m)), 4)
+    fk.set_option("gemm_sk", 1)
     del flin_d, fws_d, x, y
     # the two neighbours of that GEMM in the prompt path: the fused gate|up front (SwiGLU + NVFP4 re-quantization in the
     # epilogue, 2 x 17408 output columns) and an FP8 linear of the same shape
