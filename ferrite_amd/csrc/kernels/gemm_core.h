@@ -497,7 +497,8 @@ __device__ __forceinline__ bool gemm_sk_meet(f32x16 (&acc)[4][4], uint32_t p, ui
     uint32_t* cnt = counters + tile;
     // a run's piece of a tile in which the run does not begin is the run's last segment
     auto slot_of = [&](uint32_t q) { return 2 * q + (sk_start(q, base, rem) < t0 ? 1u : 0u); };
-    if (tid == 0) *flag = __hip_atomic_load(cnt, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // (a read-modify-write, which is performed where all XCDs meet: no stale copy of the counter can answer it)
+    if (tid == 0) *flag = __hip_atomic_fetch_add(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     uint32_t seen = *flag;
     __syncthreads();
