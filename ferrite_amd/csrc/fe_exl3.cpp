@@ -16,7 +16,7 @@
 namespace {
 
 constexpr uint32_t kMaxRowsPerPass = 64;       // 4 row groups of 16
-constexpr uint32_t kHatRows = 2048;            // rows from which the prefill decodes once into fp16 tiles (8 output tile rows)
+constexpr uint32_t kHatRows = 2049;            // rows from which the prefill decodes once into fp16 tiles (more than 8 output tile rows)
 constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
 constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
@@ -441,17 +441,20 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
         return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_linear_gemv_rotated", "rotated input of 4 GB or more");
     const uint32_t tiles_m = (rows + 255) / 256, tiles_n = (n / 128 + 1) / 2;
     if (group == 0 || group > tiles_m) group = tiles_m;
-    FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
-                                          ws->counters_len, kern->opt.gemm_splits, kern->opt.gemm_sk);
     fe_devptr_t tr = l->view.trellis, svh = l->view.svh, part = ws->part.p;
     const bool kept = l->hat.bytes != 0;  // decoded once and kept: any row count above the GEMV's runs over it
-    if (kept || (rows >= kern->opt.hat_rows && ws->hat.bytes >= hat_bytes(l))) {
+    const bool over_hat = kept || (rows >= kern->opt.hat_rows && ws->hat.bytes >= hat_bytes(l));
+    // (decoded tiles are a large weight operand: 32 KB a k tile against the trellis's 2 KB a bit)
+    FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
+                                          ws->counters_len, kern->opt.gemm_splits, kern->opt.gemm_sk, !over_hat);
+    if (over_hat) {
         fe_devptr_t hat = kept ? l->hat.p : ws->hat.p;
         if (!kept) FE_TRY(launch_decode(l, s, hat));
         group = 0;  // the raster that deals column tiles to the XCDs: each decoded weight panel goes through one L2
         void *args[] = {&xh, &hat, &svh, &y, &n, &k, &rows, &mode, &group, &sch.args};
         FE_TRY(fe_hip_launch(sch.stream_k ? kern->gemm_hat_sk : kern->gemm_hat, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     } else {
+        if (sch.stream_k) group = 1;  // column tiles fastest: the programs that are in step share a panel of inputs
         void *args[] = {&xh, &tr, &svh, &y, &n, &k, &rows, &mode, &stride_k, &stride_nb, &group, &sch.args};
         FE_TRY(fe_hip_launch((sch.stream_k ? kern->gemm_sk : kern->gemm)[bits_slot(l->bits)], sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     }

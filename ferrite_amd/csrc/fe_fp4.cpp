@@ -23,7 +23,7 @@ struct fe_fp4_kernels {
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4[3] = {nullptr, nullptr, nullptr};
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
-    fe_function_t gemm4_sk = nullptr, gemm8_sk = nullptr, gemm8c_sk = nullptr;  // the same on the stream-K schedule
+    fe_function_t gemm4_sk = nullptr, gemm8_sk = nullptr, gemm8c_sk = nullptr, swiglu4_sk = nullptr;  // the same on the stream-K schedule
     uint32_t cus = 0;
     // Switches of the launch paths: read from the environment once, at load; fe_fp4_kernels_set_option changes them
     // afterwards. No forward call reads the environment.
@@ -75,7 +75,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (!c) c = fe_hip_module_get_function(&k->gemm8c, k->module, "fe_gemm_fp8_codes");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8c, kGemmLds);
     struct { fe_function_t *f; const char *nm; } sks[] = {
-        {&k->gemm4_sk, "fe_gemm_nvfp4_sk"}, {&k->gemm8_sk, "fe_gemm_fp8_sk"}, {&k->gemm8c_sk, "fe_gemm_fp8_codes_sk"}};
+        {&k->gemm4_sk, "fe_gemm_nvfp4_sk"}, {&k->gemm8_sk, "fe_gemm_fp8_sk"}, {&k->gemm8c_sk, "fe_gemm_fp8_codes_sk"},
+        {&k->swiglu4_sk, "fe_gemm_nvfp4_swiglu_sk"}};
     for (auto &e : sks) {
         if (!c) c = fe_hip_module_get_function(e.f, k->module, e.nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(*e.f, kGemmLds);
@@ -342,7 +343,7 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
     // expansion on the 16-bit instruction, k tiles of 64; same products, another order of the f32 sums)
     const bool codes8 = l->fp8 && !kern->fp8_f16;
     FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, codes8 ? k / 128 : k / 64, kern->cus, ws->part.p, ws->part.bytes,
-                                          ws->counters.p, kGemvCounters, kern->gemm_splits, kern->gemm_sk);
+                                          ws->counters.p, kGemvCounters, kern->gemm_splits, kern->gemm_sk, /*small_b=*/!l->fp8);
     // stream-K programs sit at different depths of K: one row tile at a time (column tiles fastest) keeps those that are
     // in step on one panel of activations
     if (sch.stream_k && kern->xcd < 0) group = 1;
@@ -395,10 +396,11 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
     fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
     FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
-                                          kGemvCounters, kern->gemm_splits, 0);  // (this kernel has the one-piece form only)
+                                          kGemvCounters, kern->gemm_splits, kern->gemm_sk, /*small_b=*/false);
+    if (sch.stream_k && kern->xcd < 0) group = 1;
     void *args[] = {&aq,    &w,     &sw,    &alpha, &m,       &n,       &k,    &group, &w_snt, &w_skt,
                     &w_sr,  &s_snt, &s_skt, &s_sr,  &sch.args, &q_codes, &q_sf, &q_aq,  &down_g};
-    FE_TRY(fe_hip_launch(kern->swiglu4, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
+    FE_TRY(fe_hip_launch(sch.stream_k ? kern->swiglu4_sk : kern->swiglu4, sch.programs, 1, 1, 256, 1, 1, kGemmLds, s, args));
     if (sch.stream_k || !sch.split.cut()) return 0;
     const FeGemmSplit &gs = sch.split;
     uint32_t full = gs.full, splits = gs.splits;

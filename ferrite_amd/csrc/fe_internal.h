@@ -127,39 +127,65 @@ struct FeGemmSchedule {
     uint32_t programs = 0;
     bool stream_k = false;
 };
-// mode 0: always one piece a program. mode 2: stream-K wherever the workspace allows (tests). mode 1: stream-K where
-// it is the faster schedule, as measured (MI355X, NVFP4 and EXL3, 20..1088 tiles): all of
-//  * fewer tiles than CUs, and the best cut of the one-piece schedule leaves a partly filled round (160 tiles on 256
-//    CUs: three pieces a tile are 480 programs; with 128, 192 or 224 tiles a cut fills its rounds and stream-K has
-//    nothing to gain);
+// mode 0: always one piece a program. mode 2: runs over all tiles wherever the workspace allows, mode 3: as many whole
+// rounds as leave runs of a good shape (both for tests). mode 1: stream-K where it is the faster schedule, as measured
+// (MI355X, NVFP4, FP8 and EXL3, 20..1088 tiles). The runs must have a good shape:
 //  * at most three pieces a tile (runs of at least half a tile): the piece that arrives last adds the others alone,
-//    which takes about 5 us a piece;
+//    which takes about 5 us a piece (32 tiles of 8 pieces: 74 against 39 us);
 //  * equal runs, and programs 8 apart (the same XCD) in step, i.e. at the same depth of K at the same time: they then
-//    share operand panels in their L2. Without it every program streams its own operands past the L2 and the GEMM runs
-//    10..25 % slower than the one-piece schedule, whose programs all walk K in step (240 tiles: 579 against 479 us).
-// 160 tiles (2048 rows x 5120 columns): 5..14 % faster than the one-piece schedule. With a whole round or more of tiles
-// the one-piece schedule wins (5120 x 17408 at 2048 rows: 2..10 %). Needs two partial slots a program and a zeroed
-// counter a tile.
+//    share a panel of activations in their L2. Without it every program streams its own operands past the L2 and the
+//    GEMM runs 10..25 % slower than the one-piece schedule, whose programs all walk K in step (240 tiles: 579 against
+//    479 us).
+// Fewer tiles than CUs: runs over all tiles, where the best cut of the one-piece schedule leaves a partly filled round
+// (160 tiles on 256 CUs, 2048 rows x 5120 columns: three pieces a tile are 480 programs; 5..14 % faster. With 128, 192
+// or 224 tiles a cut fills its rounds and stream-K loses 1..12 %). More tiles than CUs, not a multiple, small weight
+// operand (small_b: packed weights of a few KB a k tile; NVFP4, FP8, the decoding EXL3 GEMM): as many whole rounds as
+// leave runs of a good shape, then the runs; no cut last round, no reduce launch (NVFP4 5120 x 17408: 544 tiles = one
+// whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at 4096; 17408 x 5120 at
+// 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles as the weight operand (32 KB a k tile) the
+// programs of the runs, which no longer share weight panels, stream too much past the L2: 349 -> 366..378 us, not taken.
+// Needs two partial slots a program and a zeroed counter a tile.
 constexpr uint32_t kFeXcds = 8;
 inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t cus, fe_devptr_t part, size_t part_bytes,
-                                       fe_devptr_t counters, size_t counters_len, uint32_t cap, int mode) {
+                                       fe_devptr_t counters, size_t counters_len, uint32_t cap, int mode, bool small_b) {
     FeGemmSchedule r;
     const uint32_t slots = (uint32_t)(part_bytes / kFeGemmPartBytes);
     r.split = fe_gemm_split(tiles, ktiles, cus, slots, cap);
     r.programs = r.split.programs();
     r.args = {r.split.full, r.split.splits, 0, 0, part, (uint32_t)std::min<size_t>(part_bytes, 0xffffffffu), 0, counters};
-    const uint64_t units = (uint64_t)tiles * ktiles;
-    const uint32_t programs = (uint32_t)std::min<uint64_t>({cus, units, slots / 2});
-    if (!mode || !programs || !counters || tiles > counters_len || units >= (1ull << 31) ||
+    const uint32_t programs = std::min<uint32_t>({cus, tiles * ktiles, slots / 2});
+    if (!mode || !programs || !counters || tiles > counters_len || (uint64_t)tiles * ktiles >= (1ull << 31) ||
         (size_t)programs * 2 * kFeGemmPartBytes > 0xffffffffu)
         return r;
-    const uint32_t base = (uint32_t)(units / programs), rem = (uint32_t)(units % programs);
-    if (mode == 1 && !(tiles < cus && rem == 0 && 2 * base >= ktiles && (kFeXcds * base) % ktiles == 0 &&
-                       (r.split.cut() * r.split.splits) % cus != 0))
+    // whole rounds first (mode 3, and mode 1 where it pays), the runs over the tiles after them
+    uint32_t whole = 0, base = 0, rem = 0;
+    auto runs = [&](uint32_t rounds) {
+        whole = rounds * programs;
+        const uint32_t units = (tiles - whole) * ktiles;
+        base = units / programs, rem = units % programs;
+    };
+    auto good = [&]() { return rem == 0 && 2 * base >= ktiles && (kFeXcds * base) % ktiles == 0; };
+    auto most_whole_rounds = [&]() {
+        for (uint32_t rounds = tiles / programs + 1; rounds-- > 0;) {
+            runs(rounds);
+            if (base > 0 && good()) return true;
+        }
+        return false;
+    };
+    runs(0);
+    if (mode == 1) {
+        if (tiles < cus) {
+            if (!(good() && (r.split.cut() * r.split.splits) % cus != 0)) return r;
+        } else if (!(small_b && tiles % cus != 0 && most_whole_rounds())) {
+            return r;
+        }
+    } else if (mode >= 3 && !most_whole_rounds()) {
         return r;
-    if (base >= ktiles && rem == 0 && base % ktiles == 0) return r;  // whole tiles only: nothing to gain
+    }
+    if (base == 0 || (base >= ktiles && rem == 0 && base % ktiles == 0 && whole == 0)) return r;  // whole tiles only: nothing to gain
     r.stream_k = true;
     r.programs = programs;
+    r.args.full_tiles = whole;
     r.args.sk_base = base, r.args.sk_rem = rem;
     return r;
 }

@@ -552,8 +552,9 @@ __device__ __forceinline__ bool gemm_sk_meet(f32x16 (&acc)[4][4], uint32_t p, ui
 }
 
 // How a GEMM launch is spread over its programs. sk_base == 0: one piece a program (gemm_work: whole tiles, then the
-// cut tiles, whose partials a reduce kernel adds). Otherwise stream-K: grid = the programs, runs of sk_base (+ 1 for the
-// first sk_rem) k tiles; part holds two slots a program, counters one word a tile, zero at rest.
+// cut tiles, whose partials a reduce kernel adds). Otherwise stream-K: grid = the programs; the first full_tiles tiles (a
+// multiple of the grid) are computed whole, round-robin, and the tiles after them are shared as runs of sk_base (+ 1 for
+// the first sk_rem) k tiles; part holds two slots a program, counters one word a tile, zero at rest.
 struct GemmSched {
     uint32_t full_tiles, splits, sk_base, sk_rem;
     float* part;
@@ -578,11 +579,24 @@ __device__ __forceinline__ void gemm_schedule(const GemmSched& sc, uint32_t tile
         else
             finish(wk.tm, wk.tn, acc);
     } else {
+        // the first sc.full_tiles tiles (a multiple of the grid) are taken whole, program p those p, p + grid, ...; the
+        // runs are laid over the tiles after them
+        const uint32_t whole = sc.full_tiles;
+        uint32_t next_whole = p;
         uint32_t u = sk_start(p, sc.sk_base, sc.sk_rem);
         const uint32_t uend = sk_start(p + 1, sc.sk_base, sc.sk_rem);
-        while (u < uend) {
-            const uint32_t tile = u / ktiles, t0 = tile * ktiles, kt0 = u - t0;
-            const uint32_t ktn = ktiles - kt0 < uend - u ? ktiles - kt0 : uend - u;
+        while (next_whole < whole || u < uend) {
+            uint32_t tile, t0 = 0, kt0 = 0, ktn = ktiles;
+            if (next_whole < whole) {
+                tile = next_whole;
+                next_whole += gridDim.x;
+            } else {
+                const uint32_t rel = u / ktiles;
+                t0 = rel * ktiles, kt0 = u - t0;
+                ktn = ktiles - kt0 < uend - u ? ktiles - kt0 : uend - u;
+                tile = whole + rel;
+                u += ktn;
+            }
             uint32_t tm, tn;
             gemm_raster(tile, tiles_m, tiles_n, group, tm, tn);
             __syncthreads();  // the epilogue of the segment before is done with the LDS
@@ -591,7 +605,6 @@ __device__ __forceinline__ void gemm_schedule(const GemmSched& sc, uint32_t tile
             if (ktn != ktiles)
                 fin = gemm_sk_meet(acc, p, tile, t0, ktiles, sc.sk_base, sc.sk_rem, sc.part, sc.part_bytes, sc.counters, lds);
             if (fin) finish(tm, tn, acc);
-            u += ktn;
         }
     }
 }

@@ -448,14 +448,24 @@ extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_reduce(uint16_t*
 // Fused MLP front: act = SwiGLU(x . [gate|up]^T), NVFP4-quantized with global scale qg (1 / input_scale of the down
 // projection) into q_codes [M][inter/2], q_sf (tiled, kb = inter/16) and the fp16 operand q_aq [M][inter]; w, sw, alpha =
 // gate and up interleaved in blocks of 8 rows, N = 2 inter, N % 256 == 0. (kernels/k-fp4/src/lib.rs:747-752)
-extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_swiglu(
-    const _Float16* aq, const uint8_t* w, const uint8_t* sw, const float* alpha, uint32_t m, uint32_t n, uint32_t k,
-    uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt, uint32_t s_sr,
-    GemmSched sc, uint8_t* q_codes, uint8_t* q_sf, _Float16* q_aq, float qg) {  // (one piece a program only)
+#define FP4_SWIGLU_PARAMS                                                                                                \
+    const _Float16 *aq, const uint8_t *w, const uint8_t *sw, const float *alpha, uint32_t m, uint32_t n, uint32_t k,           \
+        uint32_t group_m, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt, uint32_t s_sr,        \
+        GemmSched sc, uint8_t *q_codes, uint8_t *q_sf, _Float16 *q_aq, float qg
+template <bool SK>
+__device__ __forceinline__ void gemm_nvfp4_swiglu_kernel(FP4_SWIGLU_PARAMS) {
     FpOut out = {nullptr, nullptr, 0, q_codes, q_sf, q_aq, qg};
-    fp_gemm_body<true, false>(
+    fp_gemm_body<true, SK>(
         [&](uint32_t tn) { return fp4_producer(w, sw, tn, n / 128, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr); }, out, aq, alpha,
         FP4_OPERAND_SCALE, m, n, k, group_m, sc);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_swiglu(FP4_SWIGLU_PARAMS) {
+    gemm_nvfp4_swiglu_kernel<false>(aq, w, sw, alpha, m, n, k, group_m, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr, sc, q_codes, q_sf,
+                                    q_aq, qg);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_gemm_nvfp4_swiglu_sk(FP4_SWIGLU_PARAMS) {
+    gemm_nvfp4_swiglu_kernel<true>(aq, w, sw, alpha, m, n, k, group_m, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr, sc, q_codes, q_sf,
+                                   q_aq, qg);
 }
 
 extern "C" __global__ __launch_bounds__(256) void fe_gemm_nvfp4_swiglu_reduce(const float* part, const float* alpha, uint32_t m,

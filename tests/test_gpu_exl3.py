@@ -284,17 +284,20 @@ def test_prefill_gemm_matches_the_oracle(env, oracle, bits, m):
         assert (np.abs(got[:m] - lin64) / np.maximum(np.abs(lin64), np.sqrt((lin64 ** 2).mean()))).max() < 1e-2
 
 
-def test_prefill_on_the_stream_k_schedule(env, oracle):
+@pytest.mark.parametrize("m,n,forced", [(2400, 3968, 2), (6600, 4096, 3)])
+def test_prefill_on_the_stream_k_schedule(env, oracle, m, n, forced):
     """Stream-K: the prefill GEMM walks the tiles' k tiles laid end to end, every program a contiguous run; the pieces of
     a tile meet through the workspace and the last arriver adds them in piece order. 2400 x 3968 over K = 1024: 10 x 16 =
-    160 tiles of 16 k tiles, the case the library picks the schedule for by itself on 256 CUs; the last row tile ragged,
-    the last column tile half. Option gemm_sk = 1 gives the bits of the forced schedule (2); repeats give the same bits
-    (arrival order does not matter, counters return to zero); the one-piece schedule (0) differs by the order of the
-    f32 sums; both the decoding GEMM and the GEMM over decoded tiles; an add output mode; against the oracle."""
+    160 tiles of 16 k tiles on 256 CUs (forced: 2, runs over all tiles), the last row tile ragged, the last column tile
+    half; the library picks the schedule for it by itself (option gemm_sk = 1 gives the bits of the forced schedule).
+    6600 x 4096: 416 tiles, one whole round and runs of 10 k tiles over the other 160 (forced: 3): its own choice for the
+    decoding GEMM, not for the GEMM over decoded tiles, whose programs would stream the fp16 weights past the L2 (there
+    gemm_sk = 1 gives the bits of the one-piece schedule). Repeats give the same bits (arrival order does not matter,
+    counters return to zero); the one-piece schedule (0) differs by the order of the f32 sums; an add output mode;
+    against the oracle."""
     torch, exl3, kern = env
     from ferrite_amd import synth
-    m = 2400
-    t = synth.exl3_tensor(1024, 3968, 4, 77)
+    t = synth.exl3_tensor(1024, n, 4, 77)
     xd = dev_u16(torch, synth.activations(m, t.k, 8, outliers=True))
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 256)
     kern.set_option("hat_rows", 65)
@@ -314,23 +317,24 @@ def test_prefill_on_the_stream_k_schedule(env, oracle):
         o = to_oracle(oracle, t)
         ref = None
         for hat in (False, True):
-            forced = run(2, hat)
-            for _ in range(5):
-                assert np.array_equal(run(2, hat).view(np.uint32), forced.view(np.uint32)), hat
-            assert np.array_equal(run(1, hat).view(np.uint32), forced.view(np.uint32)), hat
+            want = run(forced, hat)
+            for _ in range(4):
+                assert np.array_equal(run(forced, hat).view(np.uint32), want.view(np.uint32)), hat
             pieces = run(0, hat)
+            own = pieces if hat and forced == 3 else want
+            assert np.array_equal(run(1, hat).view(np.uint32), own.view(np.uint32)), hat
             rms = np.sqrt((pieces.astype(np.float64) ** 2).mean())
-            assert np.abs(forced.astype(np.float64) - pieces).max() < 2e-6 * rms, hat
-            added = run(2, hat, exl3.Dtype.F32Add, 0.25)
-            want = forced.astype(np.float64) + 0.25  # (the add is fused into the last product: one rounding, not two)
-            assert (np.abs(added - want) <= (np.abs(want) + np.abs(forced)) * 2.0 ** -23).all(), hat
-            rows = [0, 1, 17, 255, 256, 1023, 1024, 2047, 2048, 2303, 2304, m - 1]
+            assert np.abs(want.astype(np.float64) - pieces).max() < 2e-6 * rms, hat
+            added = run(forced, hat, exl3.Dtype.F32Add, 0.25)
+            plus = want.astype(np.float64) + 0.25  # (the add is fused into the last product: one rounding, not two)
+            assert (np.abs(added - plus) <= (np.abs(plus) + np.abs(want)) * 2.0 ** -23).all(), hat
+            rows = sorted({r for r in (0, 1, 17, 255, 256, 1023, 1024, 2047, 2048, 2303, 2304, m // 2, m - 1) if r < m})
             if ref is None:
                 ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k)[rows])
-            assert np.abs(forced[rows].astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4, hat
+            assert np.abs(want[rows].astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4, hat
     finally:
         kern.set_option("gemm_sk", 1)
-        kern.set_option("hat_rows", 2048)
+        kern.set_option("hat_rows", 2049)
 
 
 def test_argument_errors_are_results_not_crashes(env):
@@ -606,7 +610,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     o = to_oracle(oracle, t)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
-    kern.set_option("hat_rows", 2048)
+    kern.set_option("hat_rows", 2049)
 
 
 def test_prefill_over_kept_decoded_weights(env, oracle):

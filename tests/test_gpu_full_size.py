@@ -188,11 +188,13 @@ def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
 
 
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
-@pytest.mark.parametrize("m", [128, 300, 512, 2048])
+@pytest.mark.parametrize("m", [128, 300, 512, 2048, 2304])
 def test_exl3_prefill_at_full_size(env, oracle, shape, m):
     """Prompt rows with 1 % outlier channels x20 through the MFMA GEMM, including the tiles cut along K and the reduce
-    kernel: 2048 rows run over tiles decoded once per call, 128, 300 and 512 rows (the chunks a prompt usually comes in)
-    decode inside the GEMM, at the real strides and with the K cut the launcher picks for one or two rows of output tiles.
+    kernel: 2304 rows run over tiles decoded once per call; 128, 300, 512 (the chunks a prompt usually comes in) and 2048
+    rows decode inside the GEMM, at the real strides and with the schedule the launcher picks: a K cut for one or two
+    rows of output tiles, at 2048 rows the stream-K schedule (a whole round and runs over the rest for 5120 x 17408,
+    runs over all 160 tiles for 17408 x 5120).
     Stage by stage against the GPU's own rotated input (1e-4 of the rms), and end to end against the reference's f64
     linear on the bf16 inputs for the reference's row sample (crates/fe-fp4/src/bin/fp4-check.rs:96)."""
     torch, exl3, kern = env
