@@ -93,7 +93,8 @@ __device__ __forceinline__ GemmWork gemm_work(uint32_t pid, uint32_t tiles_m, ui
 // 8 (e >> 2) + 4 (L >> 5) + (e & 3) for element e of the 16. The producer supplies a register image Raw of its share of
 // a weight k tile, load(kt, raw, half) (global -> the registers of half 0 or 1) and store(raw, Bs, part) for part 0, 1
 // (decode that half of
-// the share -> LDS tile of GM_BN rows, chunks placed with gm_swz), and kStoreValu, about the number of VALU
+// the share -> LDS tile of GM_BN rows, chunks placed with gm_swz), kQuarters (false; true: store_quarter(raw, Bs, q)
+// for q = 0..3 instead of store, see below) and kStoreValu, about the number of VALU
 // instructions of the two parts together.
 //
 // Schedule of one k tile (a wavefront runs alone on its SIMD, so the overlap is arranged inside the instruction stream):
@@ -165,80 +166,164 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[set][i], fb[set][j], acc[i][j], 0, 0, 0);
     };
 
-    typename Producer::Raw braw;
-    load_b(braw, 0, 0);
-    load_b(braw, 0, 1);
-    load_a(0, 0, 8);
+    if constexpr (Producer::kQuarters) {
+        // A producer whose decode is many vector ALU instructions (the trellis: about 240 a k tile and lane) spreads it
+        // over all four slices, a quarter each (store_quarter(raw, Bs, q), q = 0..3), so that no slice has more of them
+        // between two MFMAs than the matrix pipe covers. Quarter 0 of tile kt + 2 is decoded in slice 3 of tile kt, after
+        // the barrier, into the stage that tile kt has just left; quarters 1..3 in slices 0..2 of tile kt + 1. Two
+        // register images: `braw` of the tile whose quarters 1..3 are due, `bnext` of the one after it.
+        constexpr int kValu = Producer::kStoreValu / 4 / 16 + 1;
+        typename Producer::Raw braw, bnext;
+        load_b(braw, 0, 0);
+        load_b(braw, 0, 1);
+        load_a(0, 0, 8);
+        load_b(bnext, 1, 0);
+        load_b(bnext, 1, 1);
 #pragma unroll
-    for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
-    store_a(lds, 0, 8);
-    load_b(braw, 1, 0);
-    load_b(braw, 1, 1);
-    load_a(1, 0, 8);
-    __syncthreads();
-    read_frags(0, lds, 0);
-
-    // One k tile: writes tile kt + 1 into the other LDS stage (weights from braw, half in each of the first two slices,
-    // activations from areg, a quarter in the second and the rest in the third) and reloads the registers with tile kt + 2 in the slice after they are
-    // written out, so that every slice carries a similar share of the memory instructions. The
-    // sched_group_barrier sequences ask for one MFMA, then a few of the other instructions, and so on, so that memory
-    // instructions are issued while the matrix pipe works instead of in bursts that hold back the next MFMA.
-    for (uint32_t kt = 0; kt < ktiles; kt++) {
-        const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
-        unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
-        constexpr int kValu = Producer::kStoreValu / 2 / 16 + 1;  // vector ALU instructions between two MFMAs
-        // slice 0
-        read_frags(1, cur, 1);
-        prod.store(braw, nxt + GM_A_BYTES, 0);
-        mfmas(0);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // slice 1
-        read_frags(0, cur, 2);
-        prod.store(braw, nxt + GM_A_BYTES, 1);
-        store_a(nxt, 0, 2);  // a quarter of the activations' LDS writes here: slice 2 is the one bound by the LDS
-        load_b(braw, kt + 2, 0);
-        load_b(braw, kt + 2, 1);
-        mfmas(1);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // slice 2
-        read_frags(1, cur, 3);
-        store_a(nxt, 2, 8);
-        mfmas(0);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+        for (int q = 0; q < 4; q++) prod.store_quarter(braw, lds + GM_A_BYTES, q);
+        store_a(lds, 0, 8);
+        load_a(1, 0, 8);
+        prod.store_quarter(bnext, lds + GM_STAGE_BYTES + GM_A_BYTES, 0);
+        braw = bnext;
         __syncthreads();
-        // slice 3, with the first fragments of tile kt + 1
-        read_frags(0, nxt, 0);
-        load_a(kt + 2, 0, 8);
-        mfmas(1);
+        read_frags(0, lds, 0);
+        for (uint32_t kt = 0; kt < ktiles; kt++) {
+            const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
+            unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
+            // slice 0
+            read_frags(1, cur, 1);
+            prod.store_quarter(braw, nxt + GM_A_BYTES, 1);
+            mfmas(0);
 #pragma unroll
-        for (int i = 0; i < 16; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slice 1
+            read_frags(0, cur, 2);
+            prod.store_quarter(braw, nxt + GM_A_BYTES, 2);
+            store_a(nxt, 0, 2);
+            load_b(bnext, kt + 2, 0);
+            load_b(bnext, kt + 2, 1);
+            mfmas(1);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slice 2
+            read_frags(1, cur, 3);
+            prod.store_quarter(braw, nxt + GM_A_BYTES, 3);
+            store_a(nxt, 2, 8);
+            mfmas(0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            // slice 3, with the first fragments of tile kt + 1 and the first quarter of tile kt + 2
+            read_frags(0, nxt, 0);
+            load_a(kt + 2, 0, 8);
+            prod.store_quarter(bnext, lds + (kt & 1) * GM_STAGE_BYTES + GM_A_BYTES, 0);
+            mfmas(1);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            braw = bnext;
         }
-        __builtin_amdgcn_sched_barrier(0);
+    } else {
+        typename Producer::Raw braw;
+        load_b(braw, 0, 0);
+        load_b(braw, 0, 1);
+        load_a(0, 0, 8);
+#pragma unroll
+        for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
+        store_a(lds, 0, 8);
+        load_b(braw, 1, 0);
+        load_b(braw, 1, 1);
+        load_a(1, 0, 8);
+        __syncthreads();
+        read_frags(0, lds, 0);
+
+        // One k tile: writes tile kt + 1 into the other LDS stage (weights from braw, half in each of the first two slices,
+        // activations from areg, a quarter in the second and the rest in the third) and reloads the registers with tile kt + 2 in the slice after they are
+        // written out, so that every slice carries a similar share of the memory instructions. The
+        // sched_group_barrier sequences ask for one MFMA, then a few of the other instructions, and so on, so that memory
+        // instructions are issued while the matrix pipe works instead of in bursts that hold back the next MFMA.
+        for (uint32_t kt = 0; kt < ktiles; kt++) {
+            const unsigned char* cur = lds + (kt & 1) * GM_STAGE_BYTES;
+            unsigned char* nxt = lds + ((kt + 1) & 1) * GM_STAGE_BYTES;
+            constexpr int kValu = Producer::kStoreValu / 2 / 16 + 1;  // vector ALU instructions between two MFMAs
+            // slice 0
+            read_frags(1, cur, 1);
+            prod.store(braw, nxt + GM_A_BYTES, 0);
+            mfmas(0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slice 1
+            read_frags(0, cur, 2);
+            prod.store(braw, nxt + GM_A_BYTES, 1);
+            store_a(nxt, 0, 2);  // a quarter of the activations' LDS writes here: slice 2 is the one bound by the LDS
+            load_b(braw, kt + 2, 0);
+            load_b(braw, kt + 2, 1);
+            mfmas(1);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, kValu, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // slice 2
+            read_frags(1, cur, 3);
+            store_a(nxt, 2, 8);
+            mfmas(0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            // slice 3, with the first fragments of tile kt + 1
+            read_frags(0, nxt, 0);
+            load_a(kt + 2, 0, 8);
+            mfmas(1);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     __syncthreads();  // the LDS tiles are free for the epilogue
 }

@@ -27,6 +27,7 @@ struct Bf16Producer {
         u32x4 c[2][4];
     };
     static constexpr int kStoreValu = 0;
+    static constexpr bool kQuarters = false;
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
 #pragma unroll
         for (int b = 0; b < 2; b++) {

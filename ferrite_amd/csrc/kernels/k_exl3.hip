@@ -317,6 +317,25 @@ __device__ __forceinline__ void decode_lane(const LaneWords<BITS>& lw, f16x8 (&o
 #undef FE_PAIR
 }
 
+// Row half H of the same: op[kh] = decode_lane's op[H][kh], with only the windows and extracts those 16 values need.
+template <int BITS>
+__device__ __forceinline__ void decode_lane_half(const LaneWords<BITS>& lw, int h, f16x8 (&op)[2]) {
+    const LaneWindows<BITS> win = lane_windows<BITS>(lw);
+#define FE_PAIR(H, KH, C) mul1_finish2(lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H)>(lw, win), lane_x<BITS, 8 * (C) + 2 * (KH) + 4 * (H) + 1>(lw, win))
+#define FE_OP(H, KH)                                                                             \
+    {                                                                                            \
+        u32x4 t = {FE_PAIR(H, KH, 0), FE_PAIR(H, KH, 1), FE_PAIR(H, KH, 2), FE_PAIR(H, KH, 3)};  \
+        op[KH] = __builtin_bit_cast(f16x8, t);                                                   \
+    }
+    if (h == 0) {
+        FE_OP(0, 0) FE_OP(0, 1)
+    } else {
+        FE_OP(1, 0) FE_OP(1, 1)
+    }
+#undef FE_OP
+#undef FE_PAIR
+}
+
 // Store 4 consecutive outputs. mode: 0 bf16, 1 f32, 2 bf16 y += v (f32 add, one rounding), 3 f32 y += v.
 // (kernels/k-exl3/src/gemv.rs:122-145)
 __device__ __forceinline__ void store4(void* y, uint32_t mode, size_t i, float (&v)[4]) {
@@ -786,7 +805,8 @@ struct Exl3Producer {
     struct Raw {
         LaneWords<BITS> w[2];
     };
-    static constexpr int kStoreValu = 240;  // about the VALU instructions of store()
+    static constexpr int kStoreValu = 240;  // about the VALU instructions of the four quarters together
+    static constexpr bool kQuarters = true;  // the main loop spreads the decode over its four slices
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
 #pragma unroll
         for (int b = 0; b < 2; b++) {
@@ -795,18 +815,18 @@ struct Exl3Producer {
             r.w[b] = load_lane_words<BITS>(p + run_off, p + prev_off);
         }
     }
-    // part 0: the first column block, part 1: the second
-    __device__ __forceinline__ void store(const Raw& r, unsigned char* Bs, int part) const {
+    // quarter q: row half q & 1 (rows n = brow + 8 (q & 1) of the lane's tile) of column block q >> 1
+    __device__ __forceinline__ void store_quarter(const Raw& r, unsigned char* Bs, int q) const {
 #pragma unroll
-        for (int b = 0; b < 2; b++) {
-            if (b != part) continue;
-            f16x8 op[2][2];
-            decode_lane<BITS>(r.w[b], op);
+        for (int b = 0; b < 2; b++)
 #pragma unroll
-            for (int h = 0; h < 2; h++)
+            for (int h = 0; h < 2; h++) {
+                if (2 * b + h != q) continue;
+                f16x8 op[2];
+                decode_lane_half<BITS>(r.w[b], h, op);
 #pragma unroll
-                for (int kh = 0; kh < 2; kh++) *(f16x8*)(Bs + gm_swz(128 * b + brow + 8 * h, 2 * ks + kh)) = op[h][kh];
-        }
+                for (int kh = 0; kh < 2; kh++) *(f16x8*)(Bs + gm_swz(128 * b + brow + 8 * h, 2 * ks + kh)) = op[kh];
+            }
     }
 };
 
@@ -936,6 +956,7 @@ struct HatProducer {
         u32x4 c[2][4];
     };
     static constexpr int kStoreValu = 0;
+    static constexpr bool kQuarters = false;
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
 #pragma unroll
         for (int b = 0; b < 2; b++) {

@@ -180,6 +180,7 @@ struct Fp4Producer {
         uint32_t s2[2];
     };
     static constexpr int kStoreValu = 96;  // about the VALU instructions of store()
+    static constexpr bool kQuarters = false;
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
         r.c[half] = *(const u32x4*)(w + (size_t)kt * w_skt + 16 * half);
         r.s2[half] = *(const uint16_t*)(sw + (size_t)kt * s_skt + 2 * half);
@@ -257,6 +258,7 @@ struct Fp8Producer {
         u32x4 c[4];
     };
     static constexpr int kStoreValu = 40;
+    static constexpr bool kQuarters = false;
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
         const uint8_t* p = w + (size_t)kt * w_skt + 32 * half;
         r.c[2 * half] = *(const u32x4*)p;
@@ -514,6 +516,7 @@ struct Fp8CodeProducer {
         u32x4 c[2][4];
     };
     static constexpr int kStoreValu = 0;
+    static constexpr bool kQuarters = false;
     // thread t: 16-byte chunk t & 7 of rows (t >> 3) + 32 j of each 128-row half; chunks 0..3 come from 64-wide weight
     // tile 2 kt, chunks 4..7 from 2 kt + 1
     __device__ __forceinline__ void load(uint32_t kt, Raw& r, int half) const {
