@@ -41,6 +41,8 @@ SYMBOLS = {
     "fe_hip_last_error": (C.c_char_p, []),
     "fe_hip_malloc": (I, [C.POINTER(U64), SZ]),
     "fe_hip_free": (I, [U64]),
+    "fe_hip_canary_on": (I, []),
+    "fe_hip_canary_tails": (I, [P, SZ, C.POINTER(SZ)]),
     "fe_hip_memset_d8": (I, [U64, C.c_uint8, SZ, P]),
     "fe_hip_memset_d32": (I, [U64, U32, SZ, P]),
     "fe_hip_memcpy_htod": (I, [U64, P, SZ]),

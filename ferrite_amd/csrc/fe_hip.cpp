@@ -13,6 +13,7 @@ extern "C" hipError_t hipExtModuleLaunchKernel(hipFunction_t f, uint32_t globalW
 #include <cstdio>
 #include <cstring>
 #include <fstream>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -70,16 +71,83 @@ int fe_hip_synchronize(void) {
     return 0;
 }
 
+// Debug aids of the allocator (crates/fe-cuda/src/lib.rs:213-228, 299-343), both read from the environment once:
+// FE_CANARY=1 gives every allocation a 64 KB tail filled with 0xA5 that fe_hip_canary_tails checks (an overflow into a
+// neighbouring allocation raises no fault); FE_ZERO_ALLOC=0 leaves new memory as the driver hands it out instead of
+// zeroing it (the default, as in the reference: a kernel that reads memory it never wrote then at least reads the same
+// thing every run).
+namespace {
+constexpr size_t kCanaryPad = 64 << 10;
+std::mutex g_canary_lock;
+std::vector<std::pair<fe_devptr_t, size_t>> g_canary_live;
+bool env_flag(const char *name, bool fallback) {
+    const char *e = getenv(name);
+    return e && *e ? atoi(e) != 0 : fallback;
+}
+bool canary_on() {
+    static const bool on = env_flag("FE_CANARY", false);
+    return on;
+}
+bool zero_alloc() {
+    static const bool on = env_flag("FE_ZERO_ALLOC", true);
+    return on;
+}
+}  // namespace
+
 int fe_hip_malloc(fe_devptr_t *out, size_t bytes) {
     void *p = nullptr;
-    HIPCHK(hipMalloc(&p, bytes ? bytes : 1));
+    const size_t n = bytes ? bytes : 1;
+    HIPCHK(hipMalloc(&p, n + (canary_on() ? kCanaryPad : 0)));
+    if (zero_alloc()) HIPCHK(hipMemsetD8Async((hipDeviceptr_t)p, 0, n, nullptr));
+    if (canary_on()) {
+        HIPCHK(hipMemsetD8Async((hipDeviceptr_t)((char *)p + bytes), 0xA5, kCanaryPad, nullptr));
+        std::lock_guard<std::mutex> g(g_canary_lock);
+        g_canary_live.emplace_back((fe_devptr_t)p, bytes);
+    }
+    if (zero_alloc() || canary_on()) HIPCHK(hipStreamSynchronize(nullptr));
     *out = (fe_devptr_t)p;
     return 0;
 }
 
 int fe_hip_free(fe_devptr_t p) {
     if (!p) return 0;
+    if (canary_on()) {
+        std::lock_guard<std::mutex> g(g_canary_lock);
+        for (size_t i = 0; i < g_canary_live.size(); i++)
+            if (g_canary_live[i].first == p) {
+                g_canary_live.erase(g_canary_live.begin() + (long)i);
+                break;
+            }
+    }
     HIPCHK(hipFree((void *)p));
+    return 0;
+}
+
+int fe_hip_canary_on(void) { return canary_on() ? 1 : 0; }
+
+int fe_hip_canary_tails(fe_canary_tail *out, size_t cap, size_t *count) {
+    if (!count) return fe_set_error(hipErrorInvalidValue, "fe_hip_canary_tails", "null count");
+    *count = 0;
+    if (!canary_on()) return 0;
+    std::vector<std::pair<fe_devptr_t, size_t>> live;
+    {
+        std::lock_guard<std::mutex> g(g_canary_lock);
+        live = g_canary_live;
+    }
+    HIPCHK(hipDeviceSynchronize());
+    std::vector<unsigned char> buf(kCanaryPad);
+    for (const auto &e : live) {
+        HIPCHK(hipMemcpyDtoH(buf.data(), (hipDeviceptr_t)(e.first + e.second), kCanaryPad));
+        size_t bad = 0, first = 0;
+        for (size_t i = 0; i < kCanaryPad; i++)
+            if (buf[i] != 0xA5) {
+                if (!bad) first = i;
+                bad++;
+            }
+        if (!bad) continue;
+        if (out && *count < cap) out[*count] = {e.first, e.second, first, bad};
+        ++*count;
+    }
     return 0;
 }
 

@@ -39,6 +39,17 @@ const char *fe_hip_last_error(void);
 /* DeviceBuffer::alloc / zeroed / drop, memset (crates/fe-cuda/src/lib.rs:201-297) */
 int fe_hip_malloc(fe_devptr_t *out, size_t bytes);
 int fe_hip_free(fe_devptr_t p);
+/* Debug aids of the allocator (crates/fe-cuda/src/lib.rs:213-228, 299-343). FE_ZERO_ALLOC=0 in the environment turns
+ * off the zeroing of every new allocation (on by default, as in the reference). FE_CANARY=1 gives every allocation a
+ * 64 KB tail filled with 0xA5; fe_hip_canary_tails reports, for up to cap of the live allocations whose tail has been
+ * written, the base, the size, the offset of the first damaged tail byte and the number of damaged bytes (count: how
+ * many there are in all), canary::tails of the reference. Both variables are read once, at the first allocation. */
+typedef struct fe_canary_tail {
+    fe_devptr_t base;
+    size_t bytes, first, damaged;
+} fe_canary_tail;
+int fe_hip_canary_on(void);
+int fe_hip_canary_tails(fe_canary_tail *out, size_t cap, size_t *count);
 int fe_hip_memset_d8(fe_devptr_t p, uint8_t v, size_t n, fe_stream_t s);
 int fe_hip_memset_d32(fe_devptr_t p, uint32_t v, size_t n, fe_stream_t s);
 /* Synchronous copies: the device is synchronized before and after, because pageable host memory is not ordered
