@@ -16,7 +16,7 @@
 namespace {
 
 constexpr uint32_t kMaxRowsPerPass = 64;       // 4 row groups of 16
-constexpr uint32_t kHatRows = 2049;            // rows from which the prefill decodes once into fp16 tiles (more than 8 output tile rows)
+constexpr uint32_t kHatRows = 3072;            // rows from which the prefill decodes once into fp16 tiles (12 output tile rows)
 constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
 constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
@@ -369,7 +369,7 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     int cus = 0, c = 0;
     if (max_rows > kMaxRowsPerPass) c = fe_hip_cu_count(&cus);
     // arrival counters: a word a column block of the linears of one launch (GEMV); a word an output tile (stream-K GEMM)
-    ws->counters_len = std::max<size_t>({top(nbs), (size_t)4 * cus, 1});
+    ws->counters_len = std::max<size_t>({top(nbs), (size_t)32 * cus, 1});
     // (rotated inputs: one linear's at max_rows, or those of the linears of one launch at up to 64 rows each)
     if (!c) c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * gemv_rows) * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);

@@ -334,7 +334,7 @@ def test_prefill_on_the_stream_k_schedule(env, oracle, m, n, forced):
             assert np.abs(want[rows].astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4, hat
     finally:
         kern.set_option("gemm_sk", 1)
-        kern.set_option("hat_rows", 2049)
+        kern.set_option("hat_rows", 3072)
 
 
 def test_argument_errors_are_results_not_crashes(env):
@@ -610,7 +610,7 @@ def test_prefill_over_decoded_tiles_has_the_bits_of_the_decoding_gemm(env, oracl
     o = to_oracle(oracle, t)
     ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, t.k))
     assert np.abs(y.cpu().numpy().astype(np.float64) - ref).max() / np.sqrt((ref ** 2).mean()) < 1e-4
-    kern.set_option("hat_rows", 2049)
+    kern.set_option("hat_rows", 3072)
 
 
 def test_prefill_over_kept_decoded_weights(env, oracle):

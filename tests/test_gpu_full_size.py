@@ -188,10 +188,10 @@ def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
 
 
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
-@pytest.mark.parametrize("m", [128, 300, 512, 2048, 2304])
+@pytest.mark.parametrize("m", [128, 300, 512, 2048, 3072])
 def test_exl3_prefill_at_full_size(env, oracle, shape, m):
     """Prompt rows with 1 % outlier channels x20 through the MFMA GEMM, including the tiles cut along K and the reduce
-    kernel: 2304 rows run over tiles decoded once per call; 128, 300, 512 (the chunks a prompt usually comes in) and 2048
+    kernel: 3072 rows run over tiles decoded once per call; 128, 300, 512 (the chunks a prompt usually comes in) and 2048
     rows decode inside the GEMM, at the real strides and with the schedule the launcher picks: a K cut for one or two
     rows of output tiles, at 2048 rows the stream-K schedule (a whole round and runs over the rest for 5120 x 17408,
     runs over all 160 tiles for 17408 x 5120).
