@@ -98,6 +98,7 @@ SYMBOLS = {
     "fe_fp4_kernels_load": (I, [PP]),
     "fe_fp4_kernels_destroy": (I, [P]),
     "fe_fp4_kernels_set_option": (I, [P, C.c_char_p, C.c_int32]),
+    "fe_gemm_schedule_query": (I, [U32, U32, U32, C.c_int32, C.c_int32] + [C.POINTER(U32)] * 6),
     "fe_fp4_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, P, F]),
     "fe_fp4_linear_from_view": (I, [PP, C.c_char_p, U32, U32, U64, U64, U64, F]),
     "fe_fp8_linear_upload": (I, [PP, C.c_char_p, U32, U32, P, P, F]),

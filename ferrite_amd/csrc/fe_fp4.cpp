@@ -123,6 +123,18 @@ int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value
     return 0;
 }
 
+int fe_gemm_schedule_query(uint32_t tiles, uint32_t ktiles, uint32_t cus, int32_t mode, int32_t small_b, uint32_t *stream_k,
+                           uint32_t *programs, uint32_t *whole, uint32_t *splits, uint32_t *run, uint32_t *run_rem) {
+    if (!tiles || !ktiles || !cus || !stream_k || !programs || !whole || !splits || !run || !run_rem)
+        return fe_set_error(FE_ERR_ARG, "fe_gemm_schedule_query", "null or zero argument");
+    // a stand-in workspace: nonzero addresses that are never dereferenced here
+    const FeGemmSchedule s = fe_gemm_schedule(tiles, ktiles, cus, 1, (size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes, 1,
+                                              (size_t)tiles, 8, mode, small_b != 0);
+    *stream_k = s.stream_k ? 1 : 0, *programs = s.programs, *whole = s.args.full_tiles;
+    *splits = s.stream_k ? 1 : s.split.splits, *run = s.args.sk_base, *run_rem = s.args.sk_rem;
+    return 0;
+}
+
 static int check_shape(const char *name, uint32_t n, uint32_t k) {
     if (!n || !k || n % kTile || k % 128) {
         char msg[160];

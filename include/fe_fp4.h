@@ -30,6 +30,14 @@ int fe_fp4_kernels_destroy(fe_fp4_kernels *k);
  * GEMM never / where it is the faster one / wherever the workspace allows). forward() reads no environment variable. No
  * counterpart in the reference (its FE_FP4_GROUP is read at load too, crates/fe-fp4/src/lib.rs:31-32, 68). */
 int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value);
+/* How a GEMM launch of `tiles` 256 x 256 output tiles, `ktiles` k tiles each, would be spread over `cus` CUs under
+ * gemm_sk = mode (the schedule the EXL3, NVFP4 and FP8 GEMMs share; small_b: packed weights of a few KB a k tile), with a
+ * workspace of two partial slots a CU and enough counters: stream_k 0 = one piece a program (whole = tiles computed
+ * whole, splits = pieces of each remaining tile, added by a reduce launch), 1 = stream-K (whole = tiles computed whole in
+ * rounds, then runs of run (+ 1 for the first run_rem programs) k tiles over the rest). Pure host arithmetic, no GPU
+ * call. No counterpart in the reference; for tests and tuners. */
+int fe_gemm_schedule_query(uint32_t tiles, uint32_t ktiles, uint32_t cus, int32_t mode, int32_t small_b, uint32_t *stream_k,
+                           uint32_t *programs, uint32_t *whole, uint32_t *splits, uint32_t *run, uint32_t *run_rem);
 
 /* HostLinear::upload (lib.rs:425-440) of an NVFP4 linear already fused on the host: codes [n][k/2], scales row-major
  * [n][k/16] (e4m3), alpha[n] = max(input_scale) * weight_scale_2 of the column's part, g = 1 / max(input_scale). */

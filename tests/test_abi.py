@@ -177,3 +177,43 @@ def test_compute_calls_fail_loudly_without_a_gpu():
     from ferrite_amd import _lib
     with pytest.raises(_lib.FeError):
         _lib.check(_lib.lib().fe_hip_init(0))
+
+
+def gemm_schedule(tiles, ktiles, cus=256, mode=1, small_b=True):
+    from ferrite_amd import _lib
+    out = [C.c_uint32(0) for _ in range(6)]
+    _lib.check(_lib.lib().fe_gemm_schedule_query(tiles, ktiles, cus, mode, int(small_b), *[C.byref(o) for o in out]))
+    return dict(zip(("stream_k", "programs", "whole", "splits", "run", "run_rem"), (o.value for o in out)))
+
+
+def test_gemm_schedule_choice():
+    """Host arithmetic of the schedule the GEMMs share (no GPU call): stream-K only where its runs have the shape that was
+    measured faster, the one-piece schedule with its K cut everywhere else; every schedule covers each k tile once."""
+    # 2048 rows x 5120 columns: 160 tiles on 256 CUs, no cut fills its rounds -> runs of 5/8 of a tile over all tiles
+    s = gemm_schedule(160, 272)
+    assert s == {"stream_k": 1, "programs": 256, "whole": 0, "splits": 1, "run": 170, "run_rem": 0}
+    assert gemm_schedule(160, 80)["run"] == 50 and gemm_schedule(160, 80, small_b=False)["stream_k"] == 1
+    # 2048 x 17408: 544 tiles -> one whole round, runs of 90 k tiles over the other 288; not with a large weight operand
+    s = gemm_schedule(544, 80)
+    assert s == {"stream_k": 1, "programs": 256, "whole": 256, "splits": 1, "run": 90, "run_rem": 0}
+    s = gemm_schedule(544, 80, small_b=False)
+    assert (s["stream_k"], s["programs"], s["whole"], s["splits"]) == (0, 512 + 32 * 7, 512, 7)
+    # 4096 x 17408: three whole rounds + runs of 100; 4096 x 5120 over K = 17408: 320 tiles as runs of 340
+    assert gemm_schedule(1088, 80)["whole"] == 768 and gemm_schedule(1088, 80)["run"] == 100
+    assert gemm_schedule(320, 272)["whole"] == 0 and gemm_schedule(320, 272)["run"] == 340
+    # tile counts that a K cut balances, or whose runs would not be in step, or with many pieces a tile: one piece a program
+    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (512, 80)):
+        assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
+    assert gemm_schedule(160, 272, mode=0)["stream_k"] == 0
+    # forced: runs over all tiles (2) / as many whole rounds as leave good runs (3)
+    s = gemm_schedule(544, 80, mode=2)
+    assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 170, 0)
+    assert gemm_schedule(544, 80, mode=3, small_b=False)["whole"] == 256
+    s = gemm_schedule(27, 16, mode=2)  # 432 k tiles on 256 programs: 176 runs of 2, 80 of 1
+    assert (s["stream_k"], s["run"], s["run_rem"]) == (1, 1, 176)
+    # every k tile exactly once
+    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 3)):
+        s = gemm_schedule(tiles, ktiles, mode=mode)
+        assert s["stream_k"] == 1
+        assert s["whole"] % s["programs"] == 0
+        assert s["whole"] * ktiles + s["programs"] * s["run"] + s["run_rem"] == tiles * ktiles
