@@ -136,14 +136,18 @@ struct FeGemmSchedule {
 //    share a panel of activations in their L2. Without it every program streams its own operands past the L2 and the
 //    GEMM runs 10..25 % slower than the one-piece schedule, whose programs all walk K in step (240 tiles: 579 against
 //    479 us).
-// Fewer tiles than CUs: runs over all tiles, where the best cut of the one-piece schedule leaves a partly filled round
-// (160 tiles on 256 CUs, 2048 rows x 5120 columns: three pieces a tile are 480 programs; 5..14 % faster. With 128, 192
-// or 224 tiles a cut fills its rounds and stream-K loses 1..12 %). More tiles than CUs, not a multiple, small weight
-// operand (small_b: packed weights of a few KB a k tile; NVFP4, FP8, the decoding EXL3 GEMM): as many whole rounds as
-// leave runs of a good shape, then the runs; no cut last round, no reduce launch (NVFP4 5120 x 17408: 544 tiles = one
-// whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at 4096; 17408 x 5120 at
-// 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles as the weight operand (32 KB a k tile) the
-// programs of the runs, which no longer share weight panels, stream too much past the L2: 349 -> 366..378 us, not taken.
+// Fewer tiles than CUs: runs over all tiles, (a) where the runs have the good shape and the best cut of the one-piece
+// schedule leaves a partly filled round (160 tiles on 256 CUs, 2048 rows x 5120 columns: three pieces a tile are 480
+// programs; 5..14 % faster. With 128 tiles a cut fills its rounds, 192 or 224 tiles run whole on as many CUs, which then
+// clock higher under the power limit: stream-K loses 1..12 %), or (b), small
+// weight operand only (small_b: packed weights of a few KB a k tile; NVFP4, the decoding EXL3 GEMM), where the one-piece
+// schedule loses 12 % or more to its rounds even though the runs are not in step (129..162 tiles: 9..27 % faster; with
+// 120 or 240 tiles it loses 7 % and stream-K 9..20 %). More tiles than CUs, not a multiple, small weight operand: as
+// many whole rounds as leave runs of the good shape, then the runs; no cut last round, no reduce launch (NVFP4 5120 x
+// 17408: 544 tiles = one whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at
+// 4096; 17408 x 5120 at 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles or FP8 codes as the
+// weight operand (32 KB a k tile) the programs of the runs, which no longer share weight panels, stream too much past
+// the L2 (349 -> 366..378 us, 165 -> 182): not taken.
 // Needs two partial slots a program and a zeroed counter a tile.
 constexpr uint32_t kFeXcds = 8;
 inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t cus, fe_devptr_t part, size_t part_bytes,
@@ -175,7 +179,12 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
     runs(0);
     if (mode == 1) {
         if (tiles < cus) {
-            if (!(good() && (r.split.cut() * r.split.splits) % cus != 0)) return r;
+            // what the one-piece schedule loses to its partly filled rounds, as a fraction of the balanced time
+            const uint32_t sp = r.split.splits;
+            const float one_piece = (float)((tiles * sp + cus - 1) / cus) / (float)sp, balanced = (float)tiles / (float)cus;
+            const float gain = one_piece / balanced - 1.0f;
+            const bool pieces_ok = 2 * base >= ktiles;
+            if (!(pieces_ok && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f)))) return r;
         } else if (!(small_b && tiles % cus != 0 && most_whole_rounds())) {
             return r;
         }

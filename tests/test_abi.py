@@ -201,7 +201,13 @@ def test_gemm_schedule_choice():
     # 4096 x 17408: three whole rounds + runs of 100; 4096 x 5120 over K = 17408: 320 tiles as runs of 340
     assert gemm_schedule(1088, 80)["whole"] == 768 and gemm_schedule(1088, 80)["run"] == 100
     assert gemm_schedule(320, 272)["whole"] == 0 and gemm_schedule(320, 272)["run"] == 340
-    # tile counts that a K cut balances, or whose runs would not be in step, or with many pieces a tile: one piece a program
+    # 129..160 tiles, where the one-piece schedule's three pieces a tile leave its second round half empty: runs over all
+    # tiles even though they are not in step, for a small weight operand only
+    s = gemm_schedule(136, 80)
+    assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 42, 128)
+    assert gemm_schedule(136, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(148, 64)["run"] == 37
+    # tile counts that a K cut balances, or that run whole in one round, or whose runs would not be in step, or with many
+    # pieces a tile: one piece a program
     for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (512, 80)):
         assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
     assert gemm_schedule(160, 272, mode=0)["stream_k"] == 0
