@@ -142,7 +142,9 @@ struct FeGemmSchedule {
 // clock higher under the power limit: stream-K loses 1..12 %), or (b), small
 // weight operand only (small_b: packed weights of a few KB a k tile; NVFP4, the decoding EXL3 GEMM), where the one-piece
 // schedule loses 12 % or more to its rounds even though the runs are not in step (129..162 tiles: 9..27 % faster; with
-// 120 or 240 tiles it loses 7 % and stream-K 9..20 %). More tiles than CUs, not a multiple, small weight operand: as
+// 120 or 240 tiles it loses 7 % and stream-K 9..20 %). More tiles than CUs, small weight operand: the same two tests on
+// the tiles of the last, partly filled round, with the whole rounds in front of the runs (1536 rows x 17408 columns, 408
+// tiles = 256 whole + runs over 152: NVFP4 246 -> 226 us, the decoding EXL3 GEMM 303 -> 296); and otherwise, if not a multiple of the CUs, as
 // many whole rounds as leave runs of the good shape, then the runs; no cut last round, no reduce launch (NVFP4 5120 x
 // 17408: 544 tiles = one whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at
 // 4096; 17408 x 5120 at 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles or FP8 codes as the
@@ -178,16 +180,18 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
     };
     runs(0);
     if (mode == 1) {
-        if (tiles < cus) {
+        // the tiles of the last, partly filled round (all tiles when there are fewer than CUs): are runs over them worth it?
+        const uint32_t last = tiles % cus;
+        bool take = false;
+        if (last && (tiles < cus || small_b)) {
+            runs(tiles / cus);
             // what the one-piece schedule loses to its partly filled rounds, as a fraction of the balanced time
             const uint32_t sp = r.split.splits;
-            const float one_piece = (float)((tiles * sp + cus - 1) / cus) / (float)sp, balanced = (float)tiles / (float)cus;
+            const float one_piece = (float)((last * sp + cus - 1) / cus) / (float)sp, balanced = (float)last / (float)cus;
             const float gain = one_piece / balanced - 1.0f;
-            const bool pieces_ok = 2 * base >= ktiles;
-            if (!(pieces_ok && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f)))) return r;
-        } else if (!(small_b && tiles % cus != 0 && most_whole_rounds())) {
-            return r;
+            take = programs == cus && 2 * base >= ktiles && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f));
         }
+        if (!take && !(small_b && tiles > cus && last && most_whole_rounds())) return r;
     } else if (mode >= 3 && !most_whole_rounds()) {
         return r;
     }

@@ -206,6 +206,10 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(136, 80)
     assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 42, 128)
     assert gemm_schedule(136, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(148, 64)["run"] == 37
+    # the same for the last round of a larger launch: 1536 x 17408 is 408 tiles = one whole round + runs over the other 152
+    s = gemm_schedule(408, 80)
+    assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 47, 128)
+    assert gemm_schedule(408, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(680, 80)["stream_k"] == 0
     # tile counts that a K cut balances, or that run whole in one round, or whose runs would not be in step, or with many
     # pieces a tile: one piece a program
     for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (512, 80)):
@@ -218,7 +222,7 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(27, 16, mode=2)  # 432 k tiles on 256 programs: 176 runs of 2, 80 of 1
     assert (s["stream_k"], s["run"], s["run_rem"]) == (1, 1, 176)
     # every k tile exactly once
-    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 3)):
+    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 3), (408, 80, 1), (136, 80, 1)):
         s = gemm_schedule(tiles, ktiles, mode=mode)
         assert s["stream_k"] == 1
         assert s["whole"] % s["programs"] == 0
