@@ -149,7 +149,10 @@ struct FeGemmSchedule {
 // 17408: 544 tiles = one whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at
 // 4096; 17408 x 5120 at 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles or FP8 codes as the
 // weight operand (32 KB a k tile) the programs of the runs, which no longer share weight panels, stream too much past
-// the L2 (349 -> 366..378 us, 165 -> 182): not taken.
+// the L2 (349 -> 366..378 us, 165 -> 182): not taken. Whole rounds only, two or more, small weight operand: the stream-K
+// kernel with the last round as runs of one tile each (NVFP4 512 tiles 270 -> 256 us, 1024 tiles 542 -> 506, 1340..1360
+// TFLOP/s; the decoding EXL3 GEMM +0..2 %; a one-piece kernel that walks its pieces from one workgroup a CU gained
+// nothing, so it is not the start of new workgroups that costs).
 // Needs two partial slots a program and a zeroed counter a tile.
 constexpr uint32_t kFeXcds = 8;
 inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t cus, fe_devptr_t part, size_t part_bytes,
@@ -191,6 +194,8 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
             const float gain = one_piece / balanced - 1.0f;
             take = programs == cus && 2 * base >= ktiles && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f));
         }
+        // (whole rounds only, two or more: the last one as runs of one tile each, i.e. the same work in one workgroup a CU)
+        if (!take && small_b && !last && tiles >= 2 * cus && programs == cus) runs(tiles / cus - 1), take = true;
         if (!take && !(small_b && tiles > cus && last && most_whole_rounds())) return r;
     } else if (mode >= 3 && !most_whole_rounds()) {
         return r;

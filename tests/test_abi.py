@@ -212,9 +212,13 @@ def test_gemm_schedule_choice():
     assert gemm_schedule(408, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(680, 80)["stream_k"] == 0
     # tile counts that a K cut balances, or that run whole in one round, or whose runs would not be in step, or with many
     # pieces a tile: one piece a program
-    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (512, 80)):
+    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (256, 80)):
         assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
     assert gemm_schedule(160, 272, mode=0)["stream_k"] == 0
+    # whole rounds only, two or more: the same tiles from one workgroup a CU (the last round as runs of one tile)
+    s = gemm_schedule(512, 80)
+    assert (s["stream_k"], s["programs"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 256, 80, 0)
+    assert gemm_schedule(512, 80, small_b=False)["stream_k"] == 0
     # forced: runs over all tiles (2) / as many whole rounds as leave good runs (3)
     s = gemm_schedule(544, 80, mode=2)
     assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 170, 0)
