@@ -19,6 +19,10 @@ def test_forward_calls_replay_from_a_graph():
     from ferrite_amd import _lib, exl3, fp4, synth
     lib, check = _lib.lib(), _lib.check
     kern, fk = exl3.Kernels.load(), fp4.Kernels.load()
+    # the 300-row calls on the stream-K schedule: tiles shared between programs meet through the workspace, whose arrival
+    # counters the kernels re-arm themselves
+    kern.set_option("gemm_sk", 2)
+    fk.set_option("gemm_sk", 2)
     t = synth.exl3_tensor(1024, 384, 4, 5)
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 64)  # column blocks shared by several programs
     uneven = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(7, 4, 4, 0))  # 7 uneven runs
