@@ -62,7 +62,8 @@ __device__ __forceinline__ void gemm_raster(uint32_t pid, uint32_t tiles_m, uint
     tn = r / gsize;
 }
 
-// What a program computes. Programs 0 .. full_tiles - 1 take one output tile each over all of K. The remaining tiles
+// What a program computes on the one-piece schedule (the stream-K schedule is further down). Programs 0 .. full_tiles - 1
+// take one output tile each over all of K. The remaining tiles
 // (a last round that would leave most CUs idle) are cut `splits` ways along K: program full_tiles + i takes k tiles
 // [kt0, kt0 + ktn) of tile full_tiles + i / splits and leaves its 256 x 256 f32 partial in slot i of the workspace; a
 // reduce kernel adds the slots of a tile in split order and finishes it, so results do not depend on timing.
