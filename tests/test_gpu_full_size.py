@@ -208,11 +208,13 @@ def test_exl3_prefill_at_full_size(env, oracle, shape, m):
     assert end_to_end(oracle, layer, xd, rows, got[rows]) < 2e-3
 
 
-@pytest.mark.parametrize("m", [1, 16, 2048])
-def test_nvfp4_at_full_size(env, oracle, m):
+@pytest.mark.parametrize("m,shape", [(1, "gate_up"), (16, "gate_up"), (2048, "gate_up"), (2048, "down")])
+def test_nvfp4_at_full_size(env, oracle, m, shape):
+    """The NVFP4 linear at the layer's shapes: the GEMV at 1 and 16 rows; at 2048 rows the GEMM on the stream-K schedule
+    (5120 x 17408: one whole round and runs over the rest; 17408 x 5120: runs over all 160 tiles, 272 k tiles each)."""
     torch, exl3, kern = env
     from ferrite_amd import fp4, synth
-    k, n = SHAPES["gate_up"]
+    k, n = SHAPES[shape]
     fk = fp4.Kernels.load()
     host = synth.fp4_linear(n, k, 20251, input_scale=1.0)
     lin = host.upload()
