@@ -237,3 +237,33 @@ def test_nvfp4_at_full_size(env, oracle, m, shape):
     scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
     assert (np.abs(got - ref) / scale).max() < 8e-3  # fp4-check.rs:134-144
     assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
+
+
+@pytest.mark.parametrize("shape", ["gate_up", "down"])
+def test_fp8_at_full_size(env, oracle, shape):
+    """The FP8 linear on the 8-bit matrix instruction at 2048 rows and the layer's shapes (one piece a program with a K cut
+    for 5120 x 17408, stream-K over all 160 tiles for 17408 x 5120): quantizer bit for bit on sampled rows, the GEMM
+    against an f64 product over the same codes on the reference's row sample (crates/fe-fp4/src/bin/fp4-check.rs:96)."""
+    torch, exl3, kern = env
+    from ferrite_amd import fp4, synth
+    k, n = SHAPES[shape]
+    m = 2048
+    fk = fp4.Kernels.load()
+    host = synth.fp8_linear(n, k, 20252, input_scale=0.05, weight_scale=0.003)
+    lin = host.upload()
+    ws = fp4.Workspace(m, k)
+    xb = synth.activations(m, k, 6)
+    y = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    lin.forward(fk, ws, y, n, dev_u16(torch, xb), k, m)
+    torch.cuda.synchronize()
+    codes = ws.read_fp8(m, k)
+    rows = sorted({0, 1, 17, 127, 128, m // 2, m - 1})
+    for r in rows[:3]:
+        assert np.array_equal(codes[r], oracle.quant_fp8_row(xb[r], lin.g))
+    a = np.stack([oracle.dequant_fp8_row(codes[r], 1.0) for r in rows])
+    w = np.stack([oracle.dequant_fp8_row(host.codes[c], 1.0) for c in range(n)])
+    ref = oracle.ref_gemm(a, w).astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+    got = y[rows].float().cpu().numpy().astype(np.float64)
+    scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
+    assert (np.abs(got - ref) / scale).max() < 8e-3
+    assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
