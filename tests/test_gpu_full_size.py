@@ -267,3 +267,45 @@ def test_fp8_at_full_size(env, oracle, shape):
     scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
     assert (np.abs(got - ref) / scale).max() < 8e-3
     assert (np.abs(got - ref) / np.maximum(np.abs(ref), 1e-2 * scale)).max() < 1e-2
+
+
+def test_swiglu_front_at_full_size(env, oracle):
+    """The fused gate|up front at the layer's size (2048 rows, 2 x 17408 columns over K = 5120): SwiGLU and the NVFP4
+    re-quantization in the GEMM's epilogue against the same steps done on the host from the unfused bf16 output of the
+    same linear, on sampled rows. silu runs on the hardware exponential and reciprocal, so a bf16 rounding of it may
+    fall on the other side of a tie: such flips are counted, and dequantized the two agree to one step of an element."""
+    torch, exl3, kern = env
+    from ferrite_amd import fp4, synth
+    k, inter = SHAPES["gate_up"]
+    m = 2048
+    fk = fp4.Kernels.load()
+    g, u = synth.fp4_linear(inter, k, 1, name="gate"), synth.fp4_linear(inter, k, 2, name="up")
+    fused = fp4.HostLinear.fuse([("gate", g.codes, g.sf, 1.0, 1.0), ("up", u.codes, u.sf, 1.0, 1.0)])
+    fused.alpha[:] = fused.alpha * np.float32(0.01)  # outputs of order 1, where silu bends
+    sw = fused.into_swiglu().upload()
+    del g, u, fused
+    ws, act = fp4.Workspace(m, k), fp4.Workspace(m, inter)
+    xd = dev_u16(torch, synth.activations(m, k, 9))
+    yi = torch.zeros((m, 2 * inter), dtype=torch.bfloat16, device="cuda")
+    sw.forward(fk, ws, yi, 2 * inter, xd, k, m)
+    down_g = 0.5
+    sw.forward_swiglu(fk, ws, act, xd, k, m, down_g)
+    torch.cuda.synchronize()
+    rows = sorted({0, 1, 17, 127, 128, 255, 256, m // 2, m - 1})
+    bits = yi[rows].view(torch.int16).cpu().numpy().view(np.uint16)
+    y = (bits.astype(np.uint32) << 16).view(np.float32).reshape(len(rows), inter // 8, 2, 8)
+    gate, up = y[:, :, 0, :].reshape(len(rows), inter).astype(np.float64), y[:, :, 1, :].reshape(len(rows), inter)
+
+    def bf16_round(x):
+        b = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+        return (((b + 0x7FFF + ((b >> 16) & 1)) >> 16).astype(np.uint32) << 16).view(np.float32)
+
+    want_act = bf16_round(bf16_round((gate / (1.0 + np.exp(-gate))).astype(np.float32)) * up)
+    want_bits = (want_act.view(np.uint32) >> 16).astype(np.uint16)
+    want_codes, want_sf = oracle.quant_fp4(want_bits, down_g)
+    codes, sf_tiled = act.read(m, inter)
+    sfa = oracle.untile_scales(sf_tiled, m, inter // 16).reshape(m, inter // 16)
+    bad_sf, bad_codes = (sfa[rows] != want_sf).mean(), (codes[rows] != want_codes).mean()
+    assert bad_sf < 2e-3 and bad_codes < 5e-3, (bad_sf, bad_codes)
+    a_got, a_want = oracle.dequant_fp4(codes[rows], sfa[rows], 1.0), oracle.dequant_fp4(want_codes, want_sf, 1.0)
+    assert np.abs(a_got - a_want).max() <= 0.26 * np.abs(a_want).max()
