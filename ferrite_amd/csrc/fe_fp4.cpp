@@ -408,7 +408,8 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
     fe_devptr_t q_codes = act->codes.p, q_sf = act->sf.p, q_aq = act->aq.p;
     uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
     FeGemmSchedule sch = fe_gemm_schedule(tiles_m * tiles_n, k / 64, kern->cus, ws->part.p, ws->part.bytes, ws->counters.p,
-                                          kGemvCounters, kern->gemm_splits, kern->gemm_sk, /*small_b=*/false);
+                                          kGemvCounters, kern->gemm_splits, kern->gemm_sk >= 2 ? kern->gemm_sk : 0, true);
+    // (stream-K only when forced: this kernel's stream-K form was slower wherever measured, 688 -> 714 us on 5120 x 34816)
     if (sch.stream_k && kern->xcd < 0) group = 1;
     void *args[] = {&aq,    &w,     &sw,    &alpha, &m,       &n,       &k,    &group, &w_snt, &w_skt,
                     &w_sr,  &s_snt, &s_skt, &s_sr,  &sch.args, &q_codes, &q_sf, &q_aq,  &down_g};

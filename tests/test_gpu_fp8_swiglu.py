@@ -138,8 +138,9 @@ def test_swiglu_front(env, oracle, inter, k, m):
 
 
 def test_swiglu_front_on_the_stream_k_schedule(env, oracle):
-    """The fused gate|up front on the stream-K schedule (2400 rows x 2 x 2048 columns over K = 1024: 160 tiles on 256 CUs,
-    the library's own choice): repeats give the same bytes; against the one-piece schedule the f32 sums differ in their
+    """The fused gate|up front on the stream-K schedule, forced (2400 rows x 2 x 2048 columns over K = 1024: 160 tiles on
+    256 CUs; by itself the library keeps this kernel on the one-piece schedule, which measured faster): repeats give the
+    same bytes; against the one-piece schedule the f32 sums differ in their
     order, so a few values land on the other side of a rounding step: such flips are counted, and dequantized the two
     activations agree to one step of an element."""
     torch, fp4, kern = env
@@ -164,9 +165,9 @@ def test_swiglu_front_on_the_stream_k_schedule(env, oracle):
         for _ in range(3):
             c, s_ = run(2)
             assert np.array_equal(c, c2) and np.array_equal(s_, s2)
-        c1, s1 = run(1)
-        assert np.array_equal(c1, c2) and np.array_equal(s1, s2)
         c0, s0 = run(0)
+        c1, s1 = run(1)  # the library's own choice for this kernel is the one-piece schedule
+        assert np.array_equal(c1, c0) and np.array_equal(s1, s0)
     finally:
         kern.set_option("gemm_sk", 1)
     assert (s0 != s2).mean() < 2e-3 and (c0 != c2).mean() < 5e-3, ((s0 != s2).mean(), (c0 != c2).mean())
