@@ -128,31 +128,24 @@ struct FeGemmSchedule {
     bool stream_k = false;
 };
 // mode 0: always one piece a program. mode 2: runs over all tiles wherever the workspace allows, mode 3: as many whole
-// rounds as leave runs of a good shape (both for tests). mode 1: stream-K where it is the faster schedule, as measured
-// (MI355X, NVFP4, FP8 and EXL3, 20..1088 tiles). The runs must have a good shape:
-//  * at most three pieces a tile (runs of at least half a tile): the piece that arrives last adds the others alone,
-//    which takes about 5 us a piece (32 tiles of 8 pieces: 74 against 39 us);
-//  * equal runs, and programs 8 apart (the same XCD) in step, i.e. at the same depth of K at the same time: they then
-//    share a panel of activations in their L2. Without it every program streams its own operands past the L2 and the
-//    GEMM runs 10..25 % slower than the one-piece schedule, whose programs all walk K in step (240 tiles: 579 against
-//    479 us).
-// Fewer tiles than CUs: runs over all tiles, (a) where the runs have the good shape and the best cut of the one-piece
-// schedule leaves a partly filled round (160 tiles on 256 CUs, 2048 rows x 5120 columns: three pieces a tile are 480
-// programs; 5..14 % faster. With 128 tiles a cut fills its rounds, 192 or 224 tiles run whole on as many CUs, which then
-// clock higher under the power limit: stream-K loses 1..12 %), or (b), small
-// weight operand only (small_b: packed weights of a few KB a k tile; NVFP4, the decoding EXL3 GEMM), where the one-piece
-// schedule loses 12 % or more to its rounds even though the runs are not in step (129..162 tiles: 9..27 % faster; with
-// 120 or 240 tiles it loses 7 % and stream-K 9..20 %). More tiles than CUs, small weight operand: the same two tests on
-// the tiles of the last, partly filled round, with the whole rounds in front of the runs (1536 rows x 17408 columns, 408
-// tiles = 256 whole + runs over 152: NVFP4 246 -> 226 us, the decoding EXL3 GEMM 303 -> 296); and otherwise, if not a multiple of the CUs, as
-// many whole rounds as leave runs of the good shape, then the runs; no cut last round, no reduce launch (NVFP4 5120 x
-// 17408: 544 tiles = one whole round + runs of 90 k tiles over the other 288: 308 -> 297 us at 2048 rows, 603 -> 575 at
-// 4096; 17408 x 5120 at 4096 rows, 320 tiles as runs of 340: 620 -> 558). With decoded fp16 tiles or FP8 codes as the
-// weight operand (32 KB a k tile) the programs of the runs, which no longer share weight panels, stream too much past
-// the L2 (349 -> 366..378 us, 165 -> 182): not taken. Whole rounds only, two or more, small weight operand: the stream-K
-// kernel with the last round as runs of one tile each (NVFP4 512 tiles 270 -> 256 us, 1024 tiles 542 -> 506, 1340..1360
-// TFLOP/s; the decoding EXL3 GEMM +0..2 %; a one-piece kernel that walks its pieces from one workgroup a CU gained
-// nothing, so it is not the start of new workgroups that costs).
+// rounds as leave runs that are in step (both for tests). mode 1: stream-K where it is the faster schedule, as measured
+// (MI355X, NVFP4, FP8 and EXL3, 20..1088 tiles). It pays where the one-piece schedule cannot fill its last round: the
+// tiles of that round (all tiles when there are fewer than CUs) then run as runs over all CUs, behind the whole rounds.
+// Taken when the one-piece schedule cuts those tiles (tiles that run whole in one partly filled round are left alone:
+// 192 or 224 tiles on as many CUs clock higher under the power limit, stream-K loses 1..12 % there), a tile has at most
+// three pieces (runs of at least half a tile: the piece that arrives last adds the others alone, about 5 us a piece; 32
+// tiles of 8 pieces: 74 against 39 us), and either
+//  (a) the cut leaves a partly filled round and the runs are equal and in step, programs 8 apart (the same XCD) at the same
+//      depth of K at the same time, so that they share panels in their L2 (160 tiles on 256 CUs, 2048 rows x 5120
+//      columns: NVFP4 300 -> 284 us, FP8 166 -> 154, EXL3 over kept tiles 358 -> 352, decoding 393 -> 363), or
+//  (b) small weight operand only (small_b: packed weights of a few KB a k tile; NVFP4, the decoding EXL3 GEMM): the cut
+//      loses 12 % or more to its rounds, whether or not the runs are in step (129..160 tiles: three pieces a tile, a
+//      second round half empty; NVFP4 +14..27 %, EXL3 +11..15 %; 1536 rows x 17408 columns = 256 whole + 152: 241 -> 227
+//      us). Where it loses 7 % (120 or 240 tiles) stream-K loses 9..20 %: programs that are not in step stream their
+//      operands past the L2.
+// With a whole number of rounds, or whole rounds and runs that are in step over more than the last round (544 tiles as
+// 256 + runs of 90 k tiles), stream-K and the one-piece schedule are within 1 % of each other: one piece a program.
+// With decoded fp16 tiles or FP8 codes as the weight operand (32 KB a k tile) runs behind whole rounds lose 4..9 %.
 // Needs two partial slots a program and a zeroed counter a tile.
 constexpr uint32_t kFeXcds = 8;
 inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t cus, fe_devptr_t part, size_t part_bytes,
@@ -194,9 +187,7 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
             const float gain = one_piece / balanced - 1.0f;
             take = programs == cus && 2 * base >= ktiles && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f));
         }
-        // (whole rounds only, two or more: the last one as runs of one tile each, i.e. the same work in one workgroup a CU)
-        if (!take && small_b && !last && tiles >= 2 * cus && programs == cus) runs(tiles / cus - 1), take = true;
-        if (!take && !(small_b && tiles > cus && last && most_whole_rounds())) return r;
+        if (!take) return r;
     } else if (mode >= 3 && !most_whole_rounds()) {
         return r;
     }

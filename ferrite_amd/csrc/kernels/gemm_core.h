@@ -175,15 +175,21 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         // register images: `braw` of the tile whose quarters 1..3 are due, `bnext` of the one after it.
         constexpr int kValu = Producer::kStoreValu / 4 / 16 + 1;
         typename Producer::Raw braw, bnext;
+        // (the scheduling barriers keep the loads of tile 1 in the order of the loop's own: weights, then activations.
+        // The waits the compiler places in the loop are the stricter of those this order and the loop's need; with the
+        // loads of the prologue interleaved, every k tile began by waiting for activation loads it had just issued.)
         load_b(braw, 0, 0);
         load_b(braw, 0, 1);
         load_a(0, 0, 8);
         load_b(bnext, 1, 0);
         load_b(bnext, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < 4; q++) prod.store_quarter(braw, lds + GM_A_BYTES, q);
         store_a(lds, 0, 8);
+        __builtin_amdgcn_sched_barrier(0);
         load_a(1, 0, 8);
+        __builtin_amdgcn_sched_barrier(0);
         prod.store_quarter(bnext, lds + GM_STAGE_BYTES + GM_A_BYTES, 0);
         braw = bnext;
         __syncthreads();
@@ -251,15 +257,20 @@ __device__ __forceinline__ void gemm_mainloop(const _Float16* __restrict__ a, ui
         }
     } else {
         typename Producer::Raw braw;
+        // (scheduling barriers: the loads of tile 1 in the loop's own order, weights then activations, see above)
         load_b(braw, 0, 0);
         load_b(braw, 0, 1);
         load_a(0, 0, 8);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
         store_a(lds, 0, 8);
+        __builtin_amdgcn_sched_barrier(0);
         load_b(braw, 1, 0);
         load_b(braw, 1, 1);
+        __builtin_amdgcn_sched_barrier(0);
         load_a(1, 0, 8);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
         read_frags(0, lds, 0);
 
@@ -405,15 +416,20 @@ __device__ __forceinline__ void gemm_mainloop_f8(const uint8_t* __restrict__ a, 
     };
 
     typename Producer::Raw braw;
+    // (scheduling barriers: the loads of tile 1 in the loop's own order, weights then activations, as in gemm_mainloop)
     load_b(braw, 0, 0);
     load_b(braw, 0, 1);
     load_a(0, 0, 8);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int p = 0; p < 2; p++) prod.store(braw, lds + GM_A_BYTES, p);
     store_a(lds, 0, 8);
+    __builtin_amdgcn_sched_barrier(0);
     load_b(braw, 1, 0);
     load_b(braw, 1, 1);
+    __builtin_amdgcn_sched_barrier(0);
     load_a(1, 0, 8);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();
     read_a(0, lds, 0, 2);
     read_b(0, lds, 0, 4);

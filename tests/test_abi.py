@@ -193,14 +193,15 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(160, 272)
     assert s == {"stream_k": 1, "programs": 256, "whole": 0, "splits": 1, "run": 170, "run_rem": 0}
     assert gemm_schedule(160, 80)["run"] == 50 and gemm_schedule(160, 80, small_b=False)["stream_k"] == 1
-    # 2048 x 17408: 544 tiles -> one whole round, runs of 90 k tiles over the other 288; not with a large weight operand
+    # 2048 x 17408: 544 tiles = two whole rounds and 32 tiles, which would be 8 pieces each as runs: one piece a program,
+    # the last 32 cut 7 ways; the same for whole rounds only
     s = gemm_schedule(544, 80)
-    assert s == {"stream_k": 1, "programs": 256, "whole": 256, "splits": 1, "run": 90, "run_rem": 0}
-    s = gemm_schedule(544, 80, small_b=False)
     assert (s["stream_k"], s["programs"], s["whole"], s["splits"]) == (0, 512 + 32 * 7, 512, 7)
-    # 4096 x 17408: three whole rounds + runs of 100; 4096 x 5120 over K = 17408: 320 tiles as runs of 340
-    assert gemm_schedule(1088, 80)["whole"] == 768 and gemm_schedule(1088, 80)["run"] == 100
-    assert gemm_schedule(320, 272)["whole"] == 0 and gemm_schedule(320, 272)["run"] == 340
+    assert gemm_schedule(1088, 80)["stream_k"] == 0 and gemm_schedule(320, 272)["stream_k"] == 0
+    assert gemm_schedule(512, 80)["stream_k"] == 0
+    # whole rounds in front of a last round of 160 tiles
+    s = gemm_schedule(416, 16)
+    assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 10, 0)
     # 129..160 tiles, where the one-piece schedule's three pieces a tile leave its second round half empty: runs over all
     # tiles even though they are not in step, for a small weight operand only
     s = gemm_schedule(136, 80)
@@ -212,13 +213,9 @@ def test_gemm_schedule_choice():
     assert gemm_schedule(408, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(680, 80)["stream_k"] == 0
     # tile counts that a K cut balances, or that run whole in one round, or whose runs would not be in step, or with many
     # pieces a tile: one piece a program
-    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (256, 80)):
+    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (256, 80), (512, 80)):
         assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
     assert gemm_schedule(160, 272, mode=0)["stream_k"] == 0
-    # whole rounds only, two or more: the same tiles from one workgroup a CU (the last round as runs of one tile)
-    s = gemm_schedule(512, 80)
-    assert (s["stream_k"], s["programs"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 256, 80, 0)
-    assert gemm_schedule(512, 80, small_b=False)["stream_k"] == 0
     # forced: runs over all tiles (2) / as many whole rounds as leave good runs (3)
     s = gemm_schedule(544, 80, mode=2)
     assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 170, 0)
@@ -226,7 +223,7 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(27, 16, mode=2)  # 432 k tiles on 256 programs: 176 runs of 2, 80 of 1
     assert (s["stream_k"], s["run"], s["run_rem"]) == (1, 1, 176)
     # every k tile exactly once
-    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 3), (408, 80, 1), (136, 80, 1)):
+    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 3), (27, 16, 2), (1088, 80, 3), (416, 16, 1), (408, 80, 1), (136, 80, 1)):
         s = gemm_schedule(tiles, ktiles, mode=mode)
         assert s["stream_k"] == 1
         assert s["whole"] % s["programs"] == 0
