@@ -193,12 +193,15 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(160, 272)
     assert s == {"stream_k": 1, "programs": 256, "whole": 0, "splits": 1, "run": 170, "run_rem": 0}
     assert gemm_schedule(160, 80)["run"] == 50 and gemm_schedule(160, 80, small_b=False)["stream_k"] == 1
-    # 2048 x 17408: 544 tiles = two whole rounds and 32 tiles, which would be 8 pieces each as runs: one piece a program,
-    # the last 32 cut 7 ways; the same for whole rounds only
+    # 2048 x 17408: 544 tiles = two whole rounds and 32 tiles, which would be 8 pieces each as runs: one whole round and runs
+    # of 90 k tiles over the other 288 (in step), for a small weight operand; else one piece a program, the last 32 cut 7
+    # ways. 4096 x 17408: three whole rounds + runs of 100. Whole rounds only, or no whole round in front: one piece
     s = gemm_schedule(544, 80)
+    assert s == {"stream_k": 1, "programs": 256, "whole": 256, "splits": 1, "run": 90, "run_rem": 0}
+    s = gemm_schedule(544, 80, small_b=False)
     assert (s["stream_k"], s["programs"], s["whole"], s["splits"]) == (0, 512 + 32 * 7, 512, 7)
-    assert gemm_schedule(1088, 80)["stream_k"] == 0 and gemm_schedule(320, 272)["stream_k"] == 0
-    assert gemm_schedule(512, 80)["stream_k"] == 0
+    assert gemm_schedule(1088, 80)["whole"] == 768 and gemm_schedule(1088, 80)["run"] == 100
+    assert gemm_schedule(320, 272)["stream_k"] == 0 and gemm_schedule(512, 80)["stream_k"] == 0
     # whole rounds in front of a last round of 160 tiles
     s = gemm_schedule(416, 16)
     assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 10, 0)
@@ -223,7 +226,7 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(27, 16, mode=2)  # 432 k tiles on 256 programs: 176 runs of 2, 80 of 1
     assert (s["stream_k"], s["run"], s["run_rem"]) == (1, 1, 176)
     # every k tile exactly once
-    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 3), (27, 16, 2), (1088, 80, 3), (416, 16, 1), (408, 80, 1), (136, 80, 1)):
+    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 1), (408, 80, 1), (136, 80, 1)):
         s = gemm_schedule(tiles, ktiles, mode=mode)
         assert s["stream_k"] == 1
         assert s["whole"] % s["programs"] == 0
