@@ -26,8 +26,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out);
 int fe_fp4_kernels_destroy(fe_fp4_kernels *k);
 /* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
  * "group_m" (FE_FP4_GROUP), "gemv" 0/1 (FE_FP4_NO_GEMV), "gemv_sk" (FE_FP4_GEMV_SK; 0 = automatic), "xcd" -1/0/1
- * (FE_FP4_XCD), "fp8_f16" 0/1 (FE_FP8_F16), "gemm_splits" (FE_GEMM_SPLITS), "gemm_sk" 0/1/2 (FE_GEMM_SK: the stream-K schedule of the
- * GEMM never / where it is the faster one / wherever the workspace allows). forward() reads no environment variable. No
+ * (FE_FP4_XCD), "fp8_f16" 0/1 (FE_FP8_F16), "gemm_splits" (FE_GEMM_SPLITS), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the
+ * GEMM never / where it is the faster one / over all tiles / whole rounds then runs, the last two for tests). forward() reads no environment variable. No
  * counterpart in the reference (its FE_FP4_GROUP is read at load too, crates/fe-fp4/src/lib.rs:31-32, 68). */
 int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value);
 /* How a GEMM launch of `tiles` 256 x 256 output tiles, `ktiles` k tiles each, would be spread over `cus` CUs under
