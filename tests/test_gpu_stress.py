@@ -1,5 +1,5 @@
-"""Stress of the EXL3 decode path, bounded so that it runs in seconds: random shapes, bit widths, plans, layouts and row
-counts against the oracle (each case stops at its first mismatch and names itself), and thousands of random
+"""Stress of the EXL3 decode path and of the prefill GEMMs' schedules, bounded so that it runs in seconds: random shapes, bit
+widths, plans, layouts and row counts against the oracle (each case stops at its first mismatch and names itself), and thousands of random
 (linear, rows) calls on one shared workspace without a synchronization in between, every one compared bit for bit with
 the first result of its kind (the role of crates/fe-exl3/src/bin/exl3-stress.rs:62-98, which runs 256k such calls)."""
 import numpy as np
@@ -106,3 +106,72 @@ def test_random_calls_on_a_shared_workspace_repeat_their_bits():
             if not torch.equal(y.view(torch.int32), want[(li, m)].view(torch.int32)):
                 bad += 1
         assert bad == 0, f"batch {bi}: {bad} of {calls} calls differ from their first result"
+
+
+def test_random_prefill_shapes_on_both_schedules(oracle):
+    """The prefill GEMMs (EXL3 decoding in the GEMM and over decoded tiles, NVFP4) on random shapes of 65..1500 rows under
+    the one-piece schedule and both forced stream-K forms: every schedule against the oracle (EXL3) or within the order
+    of the f32 sums of the one-piece result (NVFP4, which the other tests pin to its reference), and a repeat of every
+    stream-K launch bit for bit (pieces of a tile arrive in whatever order; tiles of up to eight and more pieces occur
+    here). Each case names itself."""
+    import torch
+    from ferrite_amd import exl3, fp4, synth
+    kern, fk = exl3.Kernels.load(), fp4.Kernels.load()
+    rng = np.random.default_rng(77)
+    try:
+        for case in range(20):
+            k = int(rng.integers(2, 13)) * 128
+            n = int(rng.integers(1, 17)) * 128
+            m = int(rng.integers(65, 1500))
+            bits = int(rng.choice([3, 4, 5]))
+            what = f"case {case}: m {m} k {k} n {n} bits {bits}"
+            t = synth.exl3_tensor(k, n, bits, 3000 + case)
+            lin = exl3.Linear.new(kern, exl3.DeviceExl3(t, bool(rng.integers(0, 2))), 64)
+            kern.set_option("hat_rows", 65)
+            ws = exl3.Workspace([lin], m)
+            x = dev_u16(torch, synth.activations(m, k, case, outliers=True))
+            o = oracle.Exl3(t.k, t.n, t.bits, t.trellis, t.suh, t.svh)
+            rows = sorted({0, 1, m // 3, m // 2, m - 2, m - 1})
+            ref = None
+            for hat in (0, 65):
+                kern.set_option("hat_rows", hat)
+                for sk in (0, 2, 3):
+                    kern.set_option("gemm_sk", sk)
+                    outs = []
+                    for rep in range(2 if sk else 1):
+                        y = torch.full((m + 1, n), float("nan"), dtype=torch.float32, device="cuda")
+                        lin.forward(x, exl3.Dtype.Bf16, y, exl3.Dtype.F32, m, ws)
+                        torch.cuda.synchronize()
+                        outs.append(y.cpu().numpy())
+                    if ref is None:
+                        ref = oracle.gemv_ref(o, oracle.w_hat_f16(o), ws.xh(m, k)[rows])
+                    err = np.abs(outs[0][rows] - ref).max() / max(np.sqrt((ref ** 2).mean()), 1e-30)
+                    assert err < 1e-4, (what, hat, sk, err)
+                    assert np.isnan(outs[0][m]).all(), (what, hat, sk)
+                    if sk:
+                        assert np.array_equal(outs[0][:m].view(np.uint32), outs[1][:m].view(np.uint32)), (what, hat, sk)
+            kern.set_option("gemm_sk", 1)
+            kern.set_option("hat_rows", 3072)
+            host = synth.fp4_linear(n, k, 4000 + case, input_scale=1.0)
+            flin = host.upload()
+            fws = fp4.Workspace(m, k)
+            got = {}
+            for sk in (0, 2, 3):
+                fk.set_option("gemm_sk", sk)
+                for rep in range(2 if sk else 1):
+                    yb = torch.full((m + 1, n), -3.0, dtype=torch.bfloat16, device="cuda")
+                    flin.forward(fk, fws, yb, n, x, k, m)
+                    torch.cuda.synchronize()
+                    out = yb.float().cpu().numpy()
+                    assert (out[m] == -3.0).all(), (what, sk)
+                    if rep:
+                        assert np.array_equal(out[:m], got[sk]), (what, sk)
+                    got[sk] = out[:m]
+                if sk:
+                    a, b = got[sk].astype(np.float64), got[0].astype(np.float64)
+                    assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-4 * np.abs(b).max()).all(), (what, sk)
+            fk.set_option("gemm_sk", 1)
+    finally:
+        kern.set_option("gemm_sk", 1)
+        kern.set_option("hat_rows", 3072)
+        fk.set_option("gemm_sk", 1)
