@@ -600,8 +600,9 @@ struct Fp4GemvStage {
 // 128-row weight tile and one of sk runs of k tiles, its four wavefronts alternate k tiles. Each wavefront expands its
 // codes in registers straight into the A operand of v_mfma_f32_16x16x32_f16 (rows = weight rows, columns = activation
 // rows; one expansion serves all XR groups of activation rows); the wavefronts' sums meet in LDS. With sk > 1 the
-// splits leave f32 partials in z[split][m][n]; the last to arrive (counters[tile]) adds them in split order, finishes
-// the tile and re-arms the counter, so the result does not depend on timing. A row's sums do not depend on XR. Weight
+// splits leave f32 partials in z (per weight tile and split, 8 KB per group of 16 activation rows, in the order the
+// lanes hold them); the last to arrive (counters[tile]) adds them in split order, finishes the tile and re-arms the
+// counter, so the result does not depend on timing. A row's sums do not depend on XR. Weight
 // addressing as in fe_gemm_nvfp4.
 template <int XR>
 __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw,
@@ -611,7 +612,15 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
                                                 uint32_t s_skt, uint32_t s_sr) {
     __shared__ f32x4 red[4][FP4_GEMV_RG][64];
     __shared__ uint32_t last_flag;
+    // Both forms of every positive e4m3 scale (fp4_scale: ten vector instructions per 16 weights when computed), looked
+    // up instead: the loop is bound by vector instruction issue and the LDS pipe is idle in it.
+    __shared__ u32x2 scale_lut[128];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
+    if (tid < 128) {
+        Fp4Scale s = fp4_scale(tid);
+        scale_lut[tid] = (u32x2){__float_as_uint(s.pow2), __builtin_bit_cast(uint32_t, s.t)};
+    }
+    const uint32_t scale_rot = (8 * g + 29) & 31;  // rotating right by this leaves the lane's scale byte times 8 in bits 3..10
     const uint32_t nts = n / 128, nt = blockIdx.x % nts, split = blockIdx.x / nts;
     const uint32_t ktiles = k / 64, kt_begin = split * ktiles / sk, kt_end = (split + 1) * ktiles / sk;
     const uint8_t* wp = w + (size_t)nt * w_snt + (size_t)r * w_sr + 8 * g;
@@ -642,7 +651,11 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
     auto compute = [&](const Fp4GemvStage<XR>& st) {
 #pragma unroll
         for (int rg = 0; rg < FP4_GEMV_RG; rg++) {
-            Fp4Scale s = fp4_scale((st.sc[rg] >> (8 * g)) & 0xff);
+            const uint32_t at = __builtin_amdgcn_alignbit(st.sc[rg], st.sc[rg], scale_rot) & 0x3f8;
+            const u32x2 e = *(const u32x2*)((const char*)scale_lut + at);
+            const uint32_t tt = e[1];  // (a bit cast straight from the vector's element reads the vector's first bytes)
+            Fp4Scale s;
+            s.pow2 = __uint_as_float(e[0]), s.t = __builtin_bit_cast(f16x2, tt);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 u32x4 a = fp4x8_to_f16(st.cw[rg][j], s);
@@ -652,33 +665,26 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
             }
         }
     };
-    // Two k tiles in flight per wavefront. With one group of activation rows, loads past the end re-read the last k tile
-    // of the run (never used), which keeps the loop free of branches around memory instructions; with more groups a
-    // stage is up to 22 loads and skipping the unused ones is worth the branch (5120 x 5120 at 48 rows: 23 against 28 us).
-    Fp4GemvStage<XR> s0, s1;
-    const uint32_t last = kt_end - 1;
-    auto refill = [&](Fp4GemvStage<XR>& st, uint32_t t) {
-        if constexpr (XR == 1)
-            load(st, t < last ? t : last);
-        else if (t < kt_end)
-            load(st, t);
-    };
+    // NS k tiles in flight per wavefront (a ring of stages indexed by constants; three, four and six were measured and
+    // are no faster). Loads past the end of the run are skipped (a wavefront-uniform branch).
+    constexpr int NS = 2;
+    Fp4GemvStage<XR> st[NS];
     uint32_t kt = kt_begin + wave;
-    load(s0, kt < last ? kt : last);
-    refill(s1, kt + 4);
+#pragma unroll
+    for (int i = 0; i < NS; i++)
+        if (kt + 4 * i < kt_end) load(st[i], kt + 4 * i);
+    __syncthreads();  // scale_lut
     // (the scheduling barriers keep each refill where it is written: the compiler otherwise sinks the loads to just
     // before their use, a whole stage later)
-    for (; kt + 4 < kt_end; kt += 8) {
-        compute(s0);
-        __builtin_amdgcn_sched_barrier(0);
-        refill(s0, kt + 8);
-        __builtin_amdgcn_sched_barrier(0);
-        compute(s1);
-        __builtin_amdgcn_sched_barrier(0);
-        refill(s1, kt + 12);
-        __builtin_amdgcn_sched_barrier(0);
+    for (; kt < kt_end; kt += 4 * NS) {
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            if (kt + 4 * i < kt_end) compute(st[i]);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kt + 4 * (i + NS) < kt_end) load(st[i], kt + 4 * (i + NS));
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
-    if (kt < kt_end) compute(s0);
     // The four wavefronts' sums meet in LDS, one group of activation rows at a time; wavefront v finishes weight row
     // groups 2 v and 2 v + 1. Lane (r, g) then holds, for weight row group rg, output row 16 xr + r, columns
     // n0 + 16 rg + 4 g .. + 3.
@@ -712,13 +718,16 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
         return;
     }
     // Partials cross to another program, possibly on another XCD with its own L2: agent-scope accesses, ordered by the
-    // barriers around the arrival counter.
+    // barriers around the arrival counter. A program's partial lies in z as its lanes hold it (a wavefront's store is 1 KB
+    // in one piece), and the finisher's lanes hold the same elements: zp(split, xr, h) is this lane's f32x4.
+    auto zp = [&](uint32_t sp, int xr, int h) {
+        return z + ((((size_t)nt * sk + sp) * XR + xr) * 8 + 2 * wave + h) * 256 + 4 * lane;
+    };
 #pragma unroll
     for (int xr = 0; xr < XR; xr++) {
-        const uint32_t row = 16 * xr + r;
-        if (row < m) {
+        if (16 * xr + r < m) {
 #pragma unroll
-            for (int h = 0; h < 2; h++) store_agent_f32x4(z + ((size_t)split * m + row) * n + col + 16 * h, sum[xr][h]);
+            for (int h = 0; h < 2; h++) store_agent_f32x4(zp(split, xr, h), sum[xr][h]);
         }
     }
     agent_stores_wait();  // this lane's stores are acknowledged at agent scope
@@ -730,7 +739,8 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
     __syncthreads();
     if (!last_flag) return;
     if (tid == 0) __hip_atomic_store(&counters[nt], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // the loads of 8 splits are in flight together (an agent-scope load takes a trip to memory); sums in split order
+    // the loads of up to 8 splits are in flight together (an agent-scope load takes a trip to memory); sums in split order
+    const __amdgpu_buffer_rsrc_t zrs = __builtin_amdgcn_make_buffer_rsrc((void*)z, 0, nts * sk * XR * 8192u, 0x00020000);
 #pragma unroll
     for (int xr = 0; xr < XR; xr++) {
         const uint32_t row = 16 * xr + r;
@@ -740,9 +750,13 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
             f32x4 t[16];
 #pragma unroll
             for (int b = 0; b < 8; b++) {
-                const uint32_t sp = s0 + b < sk ? s0 + b : sk - 1;
+                if (s0 + b < sk) {
 #pragma unroll
-                for (int h = 0; h < 2; h++) t[2 * b + h] = load_agent_f32x4(z + ((size_t)sp * m + row) * n + col + 16 * h);
+                    for (int h = 0; h < 2; h++)
+                        t[2 * b + h] = load_agent_f32x4(zrs, (uint32_t)((const char*)zp(s0 + b, xr, h) - (const char*)z), 0);
+                } else {
+                    t[2 * b] = t[2 * b + 1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+                }
             }
             agent_loads_wait(t);
 #pragma unroll
