@@ -97,6 +97,22 @@ __device__ __forceinline__ Fp4Scale fp4_scale(uint32_t b) {  // b: e4m3 code, si
     s.t = (f16x2){t, t};
     return s;
 }
+// Both forms of all 128 positive e4m3 codes as a 1 KB table in LDS (fp4_scale is about ten vector instructions per 16
+// weights; a lookup is two and an LDS read). Filled by the first 128 threads; a barrier must follow before the first lookup.
+__device__ __forceinline__ void fp4_scale_lut_fill(u32x2* lut) {
+    if (threadIdx.x < 128) {
+        Fp4Scale s = fp4_scale(threadIdx.x);
+        lut[threadIdx.x] = (u32x2){__float_as_uint(s.pow2), __builtin_bit_cast(uint32_t, s.t)};
+    }
+}
+// at = 8 x the scale's code (the table's byte offset)
+__device__ __forceinline__ Fp4Scale fp4_scale_lut(const u32x2* lut, uint32_t at) {
+    const u32x2 e = *(const u32x2*)((const char*)lut + at);
+    const uint32_t t = e[1];  // (a bit cast straight from the vector's element reads the vector's first bytes)
+    Fp4Scale s;
+    s.pow2 = __uint_as_float(e[0]), s.t = __builtin_bit_cast(f16x2, t);
+    return s;
+}
 // 8 codes of one u32 -> 8 fp16 (code * 2^E * t), elements in order
 __device__ __forceinline__ u32x4 fp4x8_to_f16(uint32_t w, Fp4Scale s) {
     u32x4 o;
@@ -190,6 +206,8 @@ struct Fp4Producer {
 #pragma unroll
         for (int d = 0; d < 8; d++) {
             if (d / 4 != part) continue;
+            // (computed: looked up in an LDS table as the GEMV does, the reads queue behind the fragment reads of the
+            // k tile in flight and the GEMM is 5 % slower)
             Fp4Scale sc = fp4_scale((r.s2[d >> 2] >> (8 * ((d >> 1) & 1))) & 0xff);
             *(u32x4*)(Bs + gm_swz(row, d)) = fp4x8_to_f16(r.c[d >> 2][d & 3], sc);
         }
@@ -612,14 +630,9 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
                                                 uint32_t s_skt, uint32_t s_sr) {
     __shared__ f32x4 red[4][FP4_GEMV_RG][64];
     __shared__ uint32_t last_flag;
-    // Both forms of every positive e4m3 scale (fp4_scale: ten vector instructions per 16 weights when computed), looked
-    // up instead: the loop is bound by vector instruction issue and the LDS pipe is idle in it.
-    __shared__ u32x2 scale_lut[128];
+    __shared__ u32x2 scale_lut[128];  // the loop is bound by vector instruction issue and the LDS pipe is idle in it
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 15, g = lane >> 4;
-    if (tid < 128) {
-        Fp4Scale s = fp4_scale(tid);
-        scale_lut[tid] = (u32x2){__float_as_uint(s.pow2), __builtin_bit_cast(uint32_t, s.t)};
-    }
+    fp4_scale_lut_fill(scale_lut);
     const uint32_t scale_rot = (8 * g + 29) & 31;  // rotating right by this leaves the lane's scale byte times 8 in bits 3..10
     const uint32_t nts = n / 128, nt = blockIdx.x % nts, split = blockIdx.x / nts;
     const uint32_t ktiles = k / 64, kt_begin = split * ktiles / sk, kt_end = (split + 1) * ktiles / sk;
@@ -652,10 +665,7 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
 #pragma unroll
         for (int rg = 0; rg < FP4_GEMV_RG; rg++) {
             const uint32_t at = __builtin_amdgcn_alignbit(st.sc[rg], st.sc[rg], scale_rot) & 0x3f8;
-            const u32x2 e = *(const u32x2*)((const char*)scale_lut + at);
-            const uint32_t tt = e[1];  // (a bit cast straight from the vector's element reads the vector's first bytes)
-            Fp4Scale s;
-            s.pow2 = __uint_as_float(e[0]), s.t = __builtin_bit_cast(f16x2, tt);
+            const Fp4Scale s = fp4_scale_lut(scale_lut, at);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 u32x4 a = fp4x8_to_f16(st.cw[rg][j], s);
