@@ -208,9 +208,11 @@ def test_exl3_prefill_at_full_size(env, oracle, shape, m):
     assert end_to_end(oracle, layer, xd, rows, got[rows]) < 2e-3
 
 
-@pytest.mark.parametrize("m,shape", [(1, "gate_up"), (16, "gate_up"), (2048, "gate_up"), (2048, "down")])
+@pytest.mark.parametrize("m,shape", [(1, "gate_up"), (16, "gate_up"), (1, "down"), (40, "down"), (64, "gate_up"),
+                                     (2048, "gate_up"), (2048, "down")])
 def test_nvfp4_at_full_size(env, oracle, m, shape):
-    """The NVFP4 linear at the layer's shapes: the GEMV at 1 and 16 rows; at 2048 rows the GEMM on the stream-K schedule
+    """The NVFP4 linear at the layer's shapes: the GEMV at 1, 16, 40 rows (three groups of 16 in a pass, K cut 12 ways on
+    17408 x 5120) and 64 rows (two passes); at 2048 rows the GEMM on the stream-K schedule
     (5120 x 17408: one whole round and runs over the rest; 17408 x 5120: stream-K over all 160 tiles, 272 k tiles each)."""
     torch, exl3, kern = env
     from ferrite_amd import fp4, synth
@@ -232,7 +234,7 @@ def test_nvfp4_at_full_size(env, oracle, m, shape):
         assert np.array_equal(codes[r:r + 1], wc) and np.array_equal(sfa[r:r + 1], wsf)
     a = torch.from_numpy(oracle.dequant_fp4(codes, sfa, 1.0)).cuda()
     w = torch.from_numpy(oracle.dequant_fp4(host.codes, host.sf, 1.0)).cuda()
-    ref = ((a.double() if m <= 16 else a) @ (w.double().T if m <= 16 else w.T)).double().cpu().numpy() * host.alpha.astype(np.float64)
+    ref = ((a.double() if m <= 64 else a) @ (w.double().T if m <= 64 else w.T)).double().cpu().numpy() * host.alpha.astype(np.float64)
     got = y.float().cpu().numpy().astype(np.float64)
     scale = np.abs(ref).max(axis=1, keepdims=True).clip(1e-20)
     assert (np.abs(got - ref) / scale).max() < 8e-3  # fp4-check.rs:134-144
