@@ -190,7 +190,20 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
         }
         // (c) small weight operand, a cut last round of too many pieces a tile: one whole round fewer, so that the runs are
         // longer, if they are then in step (544 tiles = 256 whole + runs of 90 k tiles over 288: no reduce launch, 1 % faster)
-        if (!take && !(small_b && last && tiles > cus && most_whole_rounds(1))) return r;
+        if (!take && small_b && last && tiles > cus) take = most_whole_rounds(1);
+        // (d) small weight operand, one whole round and a last round of few tiles (an eighth of the CUs or fewer), which (c)
+        // cannot turn into runs in step: runs over all tiles, if they are equal, at least a tile long (two pieces a tile)
+        // and keep the programs of an XCD at no more than two depths of K at a time. 272 tiles of 80 k tiles (1024 rows x
+        // 17408 columns; the one-piece schedule cuts the 16 tiles 7 ways and adds a reduce launch), runs of 85: EXL3
+        // 199.5 -> 190.8 us, NVFP4 155.0 -> 154.3; 288 tiles, runs of 90: EXL3 211 -> 201, NVFP4 165 -> 162. Behind a
+        // second whole round (528 tiles as 256 + runs of 85) nothing is gained: not taken.
+        if (!take && small_b && last && tiles > cus && tiles < 2 * cus && 8 * last <= cus && r.split.splits > 1 &&
+            programs == cus) {
+            runs(0);
+            const uint32_t step = (kFeXcds * base) % ktiles;
+            take = rem == 0 && base >= ktiles && base >= 64 && (step == 0 || 2 * step == ktiles);
+        }
+        if (!take) return r;
     } else if (mode >= 3 && !most_whole_rounds(0)) {
         return r;
     }

@@ -214,9 +214,16 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(408, 80)
     assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 256, 47, 128)
     assert gemm_schedule(408, 80, small_b=False)["stream_k"] == 0 and gemm_schedule(680, 80)["stream_k"] == 0
+    # one whole round and a last round of an eighth of the CUs or fewer, too short for runs behind the whole round: equal
+    # runs of at least a tile over all tiles, the programs of an XCD at no more than two depths of K (small weight operand)
+    s = gemm_schedule(272, 80)
+    assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, 85, 0)
+    assert gemm_schedule(288, 80)["run"] == 90 and gemm_schedule(272, 80, small_b=False)["stream_k"] == 0
+    for tiles, ktiles in ((280, 80), (528, 80), (272, 16), (296, 80)):  # unequal runs; a second whole round; short runs; 40 tiles
+        assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
     # tile counts that a K cut balances, or that run whole in one round, or whose runs would not be in step, or with many
     # pieces a tile: one piece a program
-    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (272, 80), (256, 80), (512, 80)):
+    for tiles, ktiles in ((128, 80), (192, 80), (224, 80), (240, 272), (120, 272), (32, 80), (8, 80), (256, 80), (512, 80)):
         assert gemm_schedule(tiles, ktiles)["stream_k"] == 0, (tiles, ktiles)
     assert gemm_schedule(160, 272, mode=0)["stream_k"] == 0
     # forced: runs over all tiles (2) / as many whole rounds as leave good runs (3)
@@ -226,7 +233,8 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(27, 16, mode=2)  # 432 k tiles on 256 programs: 176 runs of 2, 80 of 1
     assert (s["stream_k"], s["run"], s["run_rem"]) == (1, 1, 176)
     # every k tile exactly once
-    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 1), (408, 80, 1), (136, 80, 1)):
+    for tiles, ktiles, mode in ((160, 272, 1), (544, 80, 1), (27, 16, 2), (1088, 80, 1), (416, 16, 1), (408, 80, 1), (136, 80, 1),
+                                (272, 80, 1)):
         s = gemm_schedule(tiles, ktiles, mode=mode)
         assert s["stream_k"] == 1
         assert s["whole"] % s["programs"] == 0
