@@ -144,8 +144,9 @@ struct FeGemmSchedule {
 //      us). Where it loses 7 % (120 or 240 tiles) stream-K loses 9..20 %: programs that are not in step stream their
 //      operands past the L2.
 // With a whole number of rounds stream-K and the one-piece schedule are within 1 % of each other: one piece a program.
-// Whole rounds and runs that are in step over more than the last round (544 tiles as 256 + runs of 90 k tiles) spare the
-// reduce launch and are 0..1.5 % faster: taken for a small weight operand, (c) below.
+// Whole rounds and runs that are in step over more than the last round (576 tiles as 256 + runs of 100 k tiles) spare the
+// reduce launch and are 1..3 % faster: taken for a small weight operand, (c) below; (d) and (e) below are two more cases
+// of a small weight operand, runs over all tiles behind no whole round.
 // With decoded fp16 tiles or FP8 codes as the weight operand (32 KB a k tile) runs behind whole rounds lose 4..9 %.
 // Needs two partial slots a program and a zeroed counter a tile.
 constexpr uint32_t kFeXcds = 8;
@@ -180,7 +181,19 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
         // the tiles of the last, partly filled round (all tiles when there are fewer than CUs): are runs over them worth it?
         const uint32_t last = tiles % cus;
         bool take = false;
-        if (last && (tiles < cus || small_b)) {
+        // (e) small weight operand, short K (up to 128 k tiles), between one and 2 1/8 rounds with a cut last round of at
+        // most 5/8 of the CUs: equal runs over all tiles, in step, instead of whole rounds with runs behind them or a cut
+        // (every tile then has two pieces, but the programs reach their tile ends at different times; behind a whole round
+        // all of them meet at once). 5120-wide K, NVFP4 / decoding EXL3, us: 320 tiles 184.5 -> 181 / 235.5 -> 230; 384:
+        // 213 -> 204.5 / 265.5 -> 263; 416: 238 -> 232 / 302 -> 292.5; 544: 286 -> 284.7 / 364 -> 356.5. With a fuller last
+        // round (448 tiles: 248 -> 250 / 315 -> 320), from 2 1/4 rounds on (576, 640, 1088 tiles) and with 272 k tiles a tile
+        // (320 tiles: 675 -> 728) it loses 1..8 %: not taken.
+        if (small_b && last && 8 * last <= 5 * cus && tiles > cus && 8 * tiles <= 17 * cus && ktiles <= 128 &&
+            r.split.splits > 1 && programs == cus) {
+            runs(0);
+            take = good() && base >= 64;
+        }
+        if (!take && last && (tiles < cus || small_b)) {
             runs(tiles / cus);
             // what the one-piece schedule loses to its partly filled rounds, as a fraction of the balanced time
             const uint32_t sp = r.split.splits;
@@ -189,8 +202,10 @@ inline FeGemmSchedule fe_gemm_schedule(uint32_t tiles, uint32_t ktiles, uint32_t
             take = programs == cus && 2 * base >= ktiles && sp > 1 && ((good() && gain > 0.0f) || (small_b && gain >= 0.12f));
         }
         // (c) small weight operand, a cut last round of too many pieces a tile: one whole round fewer, so that the runs are
-        // longer, if they are then in step (544 tiles = 256 whole + runs of 90 k tiles over 288: no reduce launch, 1 % faster)
-        if (!take && small_b && last && tiles > cus) take = most_whole_rounds(1);
+        // longer, if they are then in step (576 tiles = 256 whole + runs of 100 k tiles over 320: no reduce launch, NVFP4
+        // 312 -> 309 us, EXL3 404 -> 392). A last round that runs whole (480 tiles: 224 on as many CUs) is left alone: runs
+        // of 70 behind a whole round are 2..4.5 % slower there.
+        if (!take && small_b && last && tiles > cus && r.split.splits > 1) take = most_whole_rounds(1);
         // (d) small weight operand, one whole round and a last round of few tiles (an eighth of the CUs or fewer), which (c)
         // cannot turn into runs in step: runs over all tiles, if they are equal, at least a tile long (two pieces a tile)
         // and keep the programs of an XCD at no more than two depths of K at a time. 272 tiles of 80 k tiles (1024 rows x

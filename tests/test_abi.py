@@ -193,11 +193,20 @@ def test_gemm_schedule_choice():
     s = gemm_schedule(160, 272)
     assert s == {"stream_k": 1, "programs": 256, "whole": 0, "splits": 1, "run": 170, "run_rem": 0}
     assert gemm_schedule(160, 80)["run"] == 50 and gemm_schedule(160, 80, small_b=False)["stream_k"] == 1
-    # 2048 x 17408: 544 tiles = two whole rounds and 32 tiles, which would be 8 pieces each as runs: one whole round and runs
-    # of 90 k tiles over the other 288 (in step), for a small weight operand; else one piece a program, the last 32 cut 7
-    # ways. 4096 x 17408: three whole rounds + runs of 100. Whole rounds only, or no whole round in front: one piece
+    # 2048 x 17408: 544 tiles = two whole rounds and 32 tiles, which would be 8 pieces each as runs behind them: short K and
+    # at most 2 1/8 rounds -> equal runs of 170 k tiles over all tiles (in step), for a small weight operand; else one piece
+    # a program, the last 32 cut 7 ways. 2304 x 16384 (576 tiles, 2 1/4 rounds): one whole round and runs of 100 over the
+    # other 320. 4096 x 17408: three whole rounds + runs of 100. Whole rounds only, or long K with no whole round in front:
+    # one piece
     s = gemm_schedule(544, 80)
-    assert s == {"stream_k": 1, "programs": 256, "whole": 256, "splits": 1, "run": 90, "run_rem": 0}
+    assert s == {"stream_k": 1, "programs": 256, "whole": 0, "splits": 1, "run": 170, "run_rem": 0}
+    s = gemm_schedule(576, 80)
+    assert s == {"stream_k": 1, "programs": 256, "whole": 256, "splits": 1, "run": 100, "run_rem": 0}
+    for tiles, run in ((320, 100), (384, 120), (416, 130)):  # between one and two rounds, a last round of up to 5/8 of the CUs
+        s = gemm_schedule(tiles, 80)
+        assert (s["stream_k"], s["whole"], s["run"], s["run_rem"]) == (1, 0, run, 0)
+    for tiles in (448, 480):  # a fuller last round that runs whole: left alone
+        assert gemm_schedule(tiles, 80)["stream_k"] == 0
     s = gemm_schedule(544, 80, small_b=False)
     assert (s["stream_k"], s["programs"], s["whole"], s["splits"]) == (0, 512 + 32 * 7, 512, 7)
     assert gemm_schedule(1088, 80)["whole"] == 768 and gemm_schedule(1088, 80)["run"] == 100

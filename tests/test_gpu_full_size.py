@@ -194,7 +194,7 @@ def test_exl3_prefill_at_full_size(env, oracle, shape, m):
     kernel: 3072 rows run over tiles decoded once per call; 128, 300, 512 (the chunks a prompt usually comes in) and 2048
     rows decode inside the GEMM, at the real strides and with the schedule the launcher picks: a K cut for one or two
     rows of output tiles (512 rows x 17408 columns, 136 tiles: stream-K), at 1024 rows x 17408 columns equal runs of 85 k
-    tiles over all 272 tiles, at 2048 rows a whole round and runs over the rest for 5120 x 17408, stream-K over all 160
+    tiles over all 272 tiles, at 2048 rows runs of 170 over all 544 tiles for 5120 x 17408, stream-K over all 160
     tiles for 17408 x 5120.
     Stage by stage against the GPU's own rotated input (1e-4 of the rms), and end to end against the reference's f64
     linear on the bf16 inputs for the reference's row sample (crates/fe-fp4/src/bin/fp4-check.rs:96)."""
@@ -215,7 +215,7 @@ def test_nvfp4_at_full_size(env, oracle, m, shape):
     """The NVFP4 linear at the layer's shapes: the GEMV at 1, 16, 40 rows (three groups of 16 in a pass, K cut 12 ways on
     17408 x 5120) and 64 rows (two passes); at 1024 rows on 5120 x 17408 the GEMM as equal runs of 85 k tiles over all 272 tiles; at 2048
     rows the GEMM on the stream-K schedule
-    (5120 x 17408: one whole round and runs over the rest; 17408 x 5120: stream-K over all 160 tiles, 272 k tiles each)."""
+    (5120 x 17408: runs of 170 k tiles over all 544 tiles; 17408 x 5120: stream-K over all 160 tiles, 272 k tiles each)."""
     torch, exl3, kern = env
     from ferrite_amd import fp4, synth
     k, n = SHAPES[shape]
