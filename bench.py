@@ -71,15 +71,25 @@ class Events:
         self.check(self.lib.fe_hip_event_elapsed_ms(C.byref(out), a, b))
         return out.value
 
-    def loop_us(self, stream, fn, reps):
-        """Microseconds per call of fn() over `reps` back-to-back calls between one pair of recorded events."""
+    ramp_ms = 0.0  # untimed calls in front of every timed loop, until the GPU holds its clocks (set from --ramp-ms)
+
+    def loop_us(self, stream, fn, reps, ramp_ms=None):
+        """Microseconds per call of fn() over `reps` back-to-back calls between one pair of recorded events, after
+        `ramp_ms` (default: self.ramp_ms) of the same calls untimed: host work in front of the loop leaves the GPU at idle
+        clocks, and the first 30 ms of launches read 7-13 % slow."""
+        def burst(n):
+            a, b = self.new(), self.new()
+            self.record(a, stream)
+            for _ in range(n):
+                fn()
+            self.record(b, stream)
+            return self.ms(a, b) * 1e3 / n
         fn()
-        a, b = self.new(), self.new()
-        self.record(a, stream)
-        for _ in range(reps):
-            fn()
-        self.record(b, stream)
-        return self.ms(a, b) * 1e3 / reps
+        ramp_ms = self.ramp_ms if ramp_ms is None else ramp_ms
+        if ramp_ms > 0:
+            us = burst(8)
+            burst(int(ramp_ms * 1e3 / max(us, 1.0)) + 1)
+        return burst(reps)
 
 
 def bf16_to_f64(np, bits):
@@ -164,6 +174,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--ramp-ms", type=float, default=60.0,
+                    help="untimed steps in front of the W + K steps of `value`, until the GPU holds its clocks (0: none)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--no-configs", action="store_true", help="leave out the per-configuration CPU figures and parity")
@@ -190,6 +202,7 @@ def main():
     kern = exl3.Kernels.load()
     lib = _lib.lib()
     ev = Events(lib, _lib.check)
+    ev.ramp_ms = args.ramp_ms
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     blocks = exl3.default_blocks(exl3.cu_count())
 
@@ -257,14 +270,26 @@ def main():
                 rc |= f_record(pair[1], stream)
         _lib.check(rc)
 
-    for _ in range(args.warmup):
+    def timed_steps():  # W untimed steps, then exactly K steps between two synchronizations
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    # The GPU comes out of the host work before this point (the CPU baseline, the uploads) at its idle clocks and takes
+    # about 30 ms of continuous launches to reach the clocks it then holds: the same K steps read 2230 GB/s right after
+    # idle, 2400 after 8 ms, 2500 after 16 ms and 2560 from 32 ms on (no further change up to 250 ms). A decode loop runs
+    # in that steady state, so `value` is taken there: `after_idle` is the reading right after the host work, then the
+    # steps run untimed for --ramp-ms, then W + K steps again.
+    dt_idle = timed_steps()
+    ramp_steps = int(args.ramp_ms * 1e-3 / (dt_idle / args.steps)) + 1 if args.ramp_ms > 0 else 0
+    for _ in range(ramp_steps):
         step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    dt = timed_steps() if ramp_steps else dt_idle
     ms_per_step = dt * 1e3 / args.steps
     value = total_bytes / (dt / args.steps) / 1e9
     # the same K steps once more with an event pair on every launch, for the roofline kernel's own duration and the
@@ -348,9 +373,13 @@ def main():
                          "back_to_back_cold_us": round(single_us, 3), "bytes_per_launch": single_bytes}},
         "cpu_baseline": cpu,
         "per_launch": per,
+        "after_idle": {"value": round(total_bytes / (dt_idle / args.steps) / 1e9, 2), "unit": "GB/s",
+                       "ms_per_step": round(dt_idle * 1e3 / args.steps, 5),
+                       "what": f"the same {args.warmup} + {args.steps} steps right after the host work, before the {ramp_steps} "
+                               f"untimed steps ({args.ramp_ms:g} ms) that bring the GPU to the clocks it holds in a decode loop"},
     }
 
-    out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup)
+    out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup, ramp_steps)
     if not args.no_configs and not args.no_cpu:
         out["configs"] = configs(torch, np, exl3, fp4, synth, kern, ev, stream, tensors, by, ws)
     if not args.no_sweep:
@@ -520,13 +549,18 @@ def graph_us(lib, check, ev, fn, inner, reps=5):
     for _ in range(inner):
         fn(s)
     check(lib.fe_hip_graph_end(s, C.byref(g)))
-    check(lib.fe_hip_graph_launch(g, s))
-    a, b = ev.new(), ev.new()
-    ev.record(a, s)
-    for _ in range(reps):
-        check(lib.fe_hip_graph_launch(g, s))
-    ev.record(b, s)
-    us = ev.ms(a, b) * 1e3 / (reps * inner)
+
+    def burst(n):
+        a, b = ev.new(), ev.new()
+        ev.record(a, s)
+        for _ in range(n):
+            check(lib.fe_hip_graph_launch(g, s))
+        ev.record(b, s)
+        return ev.ms(a, b) * 1e3 / (n * inner)
+    us = burst(1)
+    if ev.ramp_ms > 0:  # (the capture is host work: back to steady clocks first)
+        burst(int(ev.ramp_ms * 1e3 / max(us * inner, 1.0)) + 1)
+    us = burst(reps)
     check(lib.fe_hip_graph_destroy(g))
     check(lib.fe_hip_stream_destroy(s))
     return us
@@ -594,7 +628,7 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
     return res
 
 
-def graph_replay(lib, check, ev, launches, stream, total_bytes, steps, warmup):
+def graph_replay(lib, check, ev, launches, stream, total_bytes, steps, warmup, ramp_steps):
     """The same step captured once into a HIP graph on a stream of its own and replayed: what the step costs when the
     host does not launch its kernels one by one. Reported beside `value`, which stays the eagerly launched step."""
     s = C.c_void_p()
@@ -605,7 +639,7 @@ def graph_replay(lib, check, ev, launches, stream, total_bytes, steps, warmup):
             check(fn(*[s if v is stream else v for v in a]))  # the prepared calls, on the capturing stream
     g = C.c_void_p()
     check(lib.fe_hip_graph_end(s, C.byref(g)))
-    for _ in range(max(warmup, 2)):
+    for _ in range(max(warmup, 2) + ramp_steps):  # (the capture is host work: back to steady clocks first, as for `value`)
         check(lib.fe_hip_graph_launch(g, s))
     a, b = ev.new(), ev.new()
     ev.record(a, s)
@@ -627,13 +661,13 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
     # continuous work on). A prompt is a long run of such launches, so every figure is taken after 0.15 s of the same
     # launches, over 0.15 s more; `after_idle_ms` is the first ten launches after the preceding host work, for comparison.
     def timed(fn, reps=10, steady=True):
-        first = ev.loop_us(stream, fn, reps) / 1e3
+        first = ev.loop_us(stream, fn, reps, ramp_ms=0) / 1e3
         if not steady:
             return first
         n_warm = max(30, int(150.0 / first))
-        ev.loop_us(stream, fn, n_warm)
+        ev.loop_us(stream, fn, n_warm, ramp_ms=0)
         timed.after_idle = first
-        return ev.loop_us(stream, fn, n_warm) / 1e3
+        return ev.loop_us(stream, fn, n_warm, ramp_ms=0) / 1e3
 
     # EXL3
     t = synth.exl3_tensor(k, n, 4, SEED, "gate")
