@@ -181,6 +181,8 @@ def main():
     ap.add_argument("--no-configs", action="store_true", help="leave out the per-configuration CPU figures and parity")
     ap.add_argument("--bracket-events", action="store_true",
                     help="time the roofline kernel with events recorded before and after its launch instead of events attached to its dispatch")
+    ap.add_argument("--step-only", action="store_true",
+                    help="only the timed passes of the step (for a kernel trace in which every GEMV dispatch is one of the step's six launches)")
     ap.add_argument("--no-sweep", action="store_true", help="leave out the M = 1, 4, 8, 16 sweep (for a kernel trace of the step alone)")
     ap.add_argument("--traffic-pass", action="store_true",
                     help="for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE: a streaming read and an elementwise update of "
@@ -313,6 +315,15 @@ def main():
     for li, la in enumerate(launches):  # every launch of the timed region, by its own events
         us = sum(ev.ms(*events[i][li]) for i in range(args.steps)) / args.steps * 1e3
         per[la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
+
+    if args.step_only:
+        print(json.dumps({"metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048", "value": round(value, 2),
+                          "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+                          "ms_per_step": round(ms_per_step, 5), "ramp_steps": ramp_steps,
+                          "roofline": {"kernel": dom_kernel, "avg_launch_us": round(dom_avg_ms * 1e3, 3),
+                                       "achieved": round(achieved, 2), "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                          "per_launch": per}))
+        return
 
     # The dominant launch and the single linear the target names, each alone and back to back between one pair of
     # events, cycling over weight copies past the caches: the kernel's duration plus the gap between two launches.
