@@ -11,14 +11,17 @@ struct FeTunedPlan {
 
 // clang-format off
 static const FeTunedPlan kFeTunedPlans[] = {
-    // MI355X, 256 CUs: us at 1 row / 16 rows of the best candidates (graph-replayed, weights cycled past the caches)
-    {5120, 17408, 3, 256, 4, 2},  // occ 4 wk 2: 17.3 / 24.0; occ 3 wk 8: 18.0 / 23.2; occ 4 wk 8: 18.0 / 23.2
-    {17408, 5120, 3, 256, 3, 8},  // occ 3..5 wk 8 (680 programs, 17 a column block): 18.9 / 26.3; occ 3 wk 2: 19.1 / 26.0
-    {5120, 17408, 4, 256, 4, 2},  // occ 4 wk 2: 17.7 / 24.6; occ 4 wk 8: 18.3 / 23.6; occ 3 wk 8: 18.4 / 23.6
-    {17408, 5120, 4, 256, 3, 8},  // occ 3..5 wk 8: 19.1 / 26.7; occ 3 wk 2: 19.5 / 26.7
-    {5120, 17408, 5, 256, 3, 8},  // occ 3 wk 8: 20.1 / 25.8; occ 4 wk 8: 20.3 / 25.9; occ 4 wk 2: 20.1 / 27.4
-    {17408, 5120, 5, 256, 3, 8},  // occ 3..5 wk 8: 21.1 / 29.0; occ 3 wk 2: 21.3 / 28.7
-    {5120, 5120, 4, 256, 4, 4},   // occ 2..5 wk 4 (400 programs): 10.7 / 14.6
-    {5120, 1024, 4, 256, 4, 4},   // occ 2..5 wk 4 (80 programs): 8.1 / 11.9
+    // MI355X, 256 CUs: us at 1 row / 16 rows of the best candidates (graph-replayed after 40 ms of the same replays, weights
+    // cycled past the caches)
+    {5120, 17408, 3, 256, 4, 2},  // occ 4 wk 2: 17.6 / 24.2; occ 3..5 wk 8: 18.2 / 23.5
+    {17408, 5120, 3, 256, 3, 8},  // occ 3..5 wk 8 (680 programs, 17 a column block): 19.1 / 26.4; occ 3 wk 2: 19.4 / 26.3
+    // (gate + up in one launch: occ 4 wk 2 30.7 us at 1 row, 33.5 at 4, 36.0 at 8, 42.3 at 16; occ 3..5 wk 8 32.5 / 35.5 /
+    // 35.8 / 39.9: the plan is the one of few rows, and one plan for all row counts keeps a row's bits)
+    {5120, 17408, 4, 256, 4, 2},  // occ 4 wk 2: 18.5 / 24.9; occ 3..5 wk 8: 18.5 / 23.9
+    {17408, 5120, 4, 256, 3, 8},  // occ 3 wk 8: 19.3 / 26.8; occ 4, 5 wk 8: 19.6 / 26.8; occ 3 wk 2: 19.8 / 26.7
+    {5120, 17408, 5, 256, 3, 8},  // occ 3 wk 8: 20.5 / 26.3; occ 5 wk 8: 20.6 / 26.3; occ 4 wk 2: 20.9 / 27.7
+    {17408, 5120, 5, 256, 2, 2},  // occ 2 wk 2: 21.1 / 27.6; occ 3..5 wk 8: 21.4 / 29.4
+    {5120, 5120, 4, 256, 4, 4},   // occ 2..5 wk 4 (400 programs): 10.8 / 14.8
+    {5120, 1024, 4, 256, 4, 4},   // occ 2..5 wk 4 (80 programs): 8.2 / 12.1
 };
 // clang-format on
