@@ -358,7 +358,10 @@ def main():
     ceiling = {}
     for bits in BITS:
         grid, iters = 4 * exl3.cu_count(), 256
-        ms = kern.probe_decode(bits, grid, iters, 5)
+        if args.ramp_ms > 0:  # (the probes run at steady clocks like the kernel they bound)
+            ms = kern.probe_decode(bits, grid, iters, 5)
+            kern.probe_decode(bits, grid, iters, int(args.ramp_ms / max(ms, 1e-3)) + 1)
+        ms = kern.probe_decode(bits, grid, iters, 20)
         ceiling[f"b{bits}"] = round(grid * 256 * 32 * iters * bits / 8 / (ms * 1e-3) / 1e9, 1)
 
     out = {
