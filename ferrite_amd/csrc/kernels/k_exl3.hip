@@ -484,7 +484,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
     constexpr uint32_t tw = 8 * BITS;
-    constexpr int DEPTH = 4;  // load steps in flight per lane (8 measured slower: 22.9 against 20.7 us)
+    constexpr int DEPTH = 4;  // load steps in flight per lane (5 and 6 measured 2..5 % slower, 8 10 %: 22.9 against 20.7 us)
     constexpr int GROUP = 8;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t r = lane & 15, g = lane >> 4, q = r & 7, tau = r >> 3;
