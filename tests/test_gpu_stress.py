@@ -1,4 +1,4 @@
-"""Stress of the EXL3 decode path and of the prefill GEMMs' schedules, bounded so that it runs in seconds: random shapes, bit
+"""Stress of the EXL3 decode path, of the prefill GEMMs' schedules and of the NVFP4 GEMV, bounded so that it runs in seconds: random shapes, bit
 widths, plans, layouts and row counts against the oracle (each case stops at its first mismatch and names itself), and thousands of random
 (linear, rows) calls on one shared workspace without a synchronization in between, every one compared bit for bit with
 the first result of its kind (the role of crates/fe-exl3/src/bin/exl3-stress.rs:62-98, which runs 256k such calls)."""
@@ -175,3 +175,40 @@ def test_random_prefill_shapes_on_both_schedules(oracle):
         kern.set_option("gemm_sk", 1)
         kern.set_option("hat_rows", 3072)
         fk.set_option("gemm_sk", 1)
+
+
+def test_random_nvfp4_gemv_shapes_rows_and_splits():
+    """The NVFP4 GEMV on random shapes, 1..64 rows (one to three groups of 16 rows, and two passes) and forced K splits of
+    1..16 (the partials of a split meet through the workspace): every case against the GEMM over the same rows (the same
+    exact products, summed in another order), the row after the batch untouched, a repeat bit for bit. Each case names
+    itself."""
+    import torch
+    from ferrite_amd import fp4, synth
+    fk = fp4.Kernels.load()
+    rng = np.random.default_rng(3)
+    try:
+        for case in range(60):
+            n, k = int(rng.integers(1, 17)) * 128, int(rng.integers(2, 33)) * 128
+            m, sk = int(rng.integers(1, 65)), int(rng.choice([0, 1, 2, 3, 5, 8, 16]))
+            what = f"case {case}: n {n} k {k} rows {m} split {sk}"
+            lin = synth.fp4_linear(n, k, 100 + case, input_scale=1.0).upload()
+            ws = fp4.Workspace(m, k)
+            x = dev_u16(torch, synth.activations(m, k, case))
+
+            def run():
+                y = torch.full((m + 1, n), -3.0, dtype=torch.bfloat16, device="cuda")
+                lin.forward(fk, ws, y, n, x, k, m)
+                torch.cuda.synchronize()
+                return y.float().cpu().numpy()
+
+            fk.set_option("gemv_sk", sk)
+            a, again = run(), run()
+            fk.set_option("gemv", 0)
+            b = run()
+            fk.set_option("gemv", 1)
+            assert np.array_equal(a, again) and (a[m] == -3.0).all(), what
+            a, b = a[:m].astype(np.float64), b[:m].astype(np.float64)
+            assert (np.abs(a - b) <= np.abs(b) / 100.0 + 1e-3 * np.abs(b).max()).all(), what
+    finally:
+        fk.set_option("gemv", 1)
+        fk.set_option("gemv_sk", 0)
