@@ -1,7 +1,8 @@
-"""Stress of the EXL3 decode path, of the prefill GEMMs' schedules and of the NVFP4 GEMV, bounded so that it runs in seconds: random shapes, bit
-widths, plans, layouts and row counts against the oracle (each case stops at its first mismatch and names itself), and thousands of random
-(linear, rows) calls on one shared workspace without a synchronization in between, every one compared bit for bit with
-the first result of its kind (the role of crates/fe-exl3/src/bin/exl3-stress.rs:62-98, which runs 256k such calls)."""
+"""Stress of the EXL3 decode path, of the prefill GEMMs' schedules and of the NVFP4 GEMV, bounded so that it runs in
+seconds: random shapes, bit widths, plans, layouts and row counts against the oracle (each case stops at its first
+mismatch and names itself), and thousands of random (linear, rows) calls on one shared workspace without a
+synchronization in between, every one compared bit for bit with the first result of its kind (the role of
+crates/fe-exl3/src/bin/exl3-stress.rs:62-98, which runs 256k such calls)."""
 import numpy as np
 import pytest
 
