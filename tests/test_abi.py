@@ -248,3 +248,24 @@ def test_gemm_schedule_choice():
         assert s["stream_k"] == 1
         assert s["whole"] % s["programs"] == 0
         assert s["whole"] * ktiles + s["programs"] * s["run"] + s["run_rem"] == tiles * ktiles
+
+
+def test_gemm_schedule_covers_every_k_tile_once():
+    """Whatever the policy picks (every tile count up to five rounds, several K lengths, both kinds of weight operand, all
+    modes): a stream-K schedule's whole rounds and runs add up to tiles x k tiles, whole rounds are a multiple of the
+    grid, and a one-piece schedule's cut tiles fit one launch."""
+    for ktiles in (16, 40, 64, 80, 128, 272):
+        for tiles in list(range(1, 1300, 7)) + [160, 256, 272, 288, 320, 384, 416, 448, 480, 512, 528, 544, 576, 640, 1088]:
+            for small_b in (True, False):
+                for mode in (0, 1, 2, 3):
+                    s = gemm_schedule(tiles, ktiles, mode=mode, small_b=small_b)
+                    what = (tiles, ktiles, small_b, mode, s)
+                    if s["stream_k"]:
+                        assert mode != 0 and s["programs"] <= 256 and s["whole"] % s["programs"] == 0 and s["whole"] <= tiles, what
+                        assert s["whole"] * ktiles + s["programs"] * s["run"] + s["run_rem"] == tiles * ktiles, what
+                        assert s["run_rem"] < s["programs"] and s["run"] + (1 if s["run_rem"] else 0) > 0, what
+                    else:
+                        assert s["whole"] <= tiles and s["splits"] >= 1, what
+                        assert s["programs"] == s["whole"] + (tiles - s["whole"]) * s["splits"], what
+                        assert s["splits"] == 1 or s["splits"] * 4 <= ktiles, what
+
