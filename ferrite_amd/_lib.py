@@ -88,6 +88,9 @@ SYMBOLS = {
     "fe_exl3_linear_forward_swiglu": (I, [P, P, P, U64, U64, U32, U64, I, U32, P]),
     "fe_exl3_linear_forward_group": (I, [PP, SZ, P, P, U64, I, C.POINTER(U64), I, U32, P]),
     "fe_exl3_linear_forward_group_launches": (I, [PP, SZ, U32, P]),
+    "fe_exl3_mlp_forward": (I, [P, P, P, P, P, U64, I, U64, U64, U64, I, U32, P]),
+    "fe_exl3_mlp_forward_launches": (I, [P, P, P, U32, I, P]),
+    "fe_exl3_workspace_chain_status": (I, [P, C.POINTER(U32)]),
     "fe_exl3_linear_rotate_input": (I, [P, P, P, U64, I, U32, P]),
     "fe_exl3_linear_gemv_rotated": (I, [P, P, U64, U64, I, U32, P]),
     "fe_exl3_reconstruct_hat_f16": (I, [P, P, C.POINTER(View), U64]),

@@ -22,6 +22,7 @@ constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
 constexpr uint32_t kCuLds = 160 * 1024;        // LDS of a CU
+constexpr size_t kChainStride = 64;            // FE_CHAIN_STRIDE: u32 words between two ready words of the one-launch MLP
 
 bool env_is(const char *name, const char *v) {
     const char *e = getenv(name);
@@ -50,6 +51,9 @@ struct fe_exl3_options {
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
     uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
+    uint32_t mlp_chain = 1;        // the decode MLP (gate, up, down) as one launch where it applies (FE_EXL3_NO_CHAIN=1: off)
+    uint32_t chain_perm = 1;       // the down stage's workgroups in the order in which their inputs get ready (FE_EXL3_CHAIN_PERM)
+    uint32_t chain_spin = 1u << 16;  // polls a program of the down stage waits for the front stage's outputs (FE_EXL3_CHAIN_SPIN)
 };
 
 struct fe_exl3_kernels {
@@ -58,6 +62,7 @@ struct fe_exl3_kernels {
     fe_function_t rot_in = nullptr, rot_in_group = nullptr, probe_v4 = nullptr;
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemvb[6][4] = {};                               // the decode GEMV, [bits slot][row groups - 1]
+    fe_function_t mlp[6] = {};                                    // the decode MLP in one launch, [bits slot]
     uint32_t cus = 0;
     fe_function_t gemm[6] = {}, gemm_sk[6] = {};  // decode inside the GEMM: one piece a program / stream-K
     fe_function_t gemm_reduce = nullptr;
@@ -81,7 +86,8 @@ struct fe_exl3_workspace {
     uint32_t max_rows = 0, max_k = 0;
     FeBuf xh, z, counters, part;  // part: partial tiles of the prefill GEMM (rows > 64 only)
     FeBuf hat;                    // decoded fp16 weights of one linear (workspaces of hat_rows rows or more)
-    size_t z_len = 0, counters_len = 0;
+    FeBuf chain;                  // state of the one-launch MLP: sequence, error, finished blocks, ready words (u32)
+    size_t z_len = 0, counters_len = 0, chain_len = 0;
 };
 
 int fe_load_module(fe_module_t *out, const char *env, const unsigned char *begin, const unsigned char *end) {
@@ -135,6 +141,9 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
             get(&k->gemvb[i][rg - 1], nm);
             if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemvb[i][rg - 1], 84 * 1024);
         }
+        snprintf(nm, sizeof nm, "exl3_mlp_b%d", kBits[i]);
+        get(&k->mlp[i], nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->mlp[i], 84 * 1024);
         snprintf(nm, sizeof nm, "exl3_gemm_b%d", kBits[i]);
         get(&k->gemm[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm[i], kGemmLds);
@@ -159,6 +168,9 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     o.gemm_group_m = env_u32("FE_EXL3_GROUP", o.gemm_group_m);
     o.gemm_splits = env_u32("FE_GEMM_SPLITS", o.gemm_splits);
     o.gemm_sk = env_u32("FE_GEMM_SK", o.gemm_sk);
+    o.mlp_chain = env_u32("FE_EXL3_NO_CHAIN", 0) ? 0 : 1;
+    o.chain_spin = env_u32("FE_EXL3_CHAIN_SPIN", o.chain_spin);
+    o.chain_perm = env_u32("FE_EXL3_CHAIN_PERM", o.chain_perm);
     if (!c) {
         int cus = 0;
         c = fe_hip_cu_count(&cus);
@@ -192,6 +204,9 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     else if (nm == "gemm_group_m") o.gemm_group_m = value;
     else if (nm == "gemm_splits") o.gemm_splits = value;
     else if (nm == "gemm_sk") o.gemm_sk = value;
+    else if (nm == "mlp_chain") o.mlp_chain = value;
+    else if (nm == "chain_spin") o.chain_spin = value;
+    else if (nm == "chain_perm") o.chain_perm = value;
     else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
     return 0;
 }
@@ -374,6 +389,11 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     if (!c) c = ws->xh.alloc((size_t)std::max(max_rows, kGroupMax * gemv_rows) * max_k * 2);
     if (!c) c = ws->z.alloc(ws->z_len * 4);
     if (!c) c = ws->counters.zeroed(ws->counters_len * 4);
+    // one-launch MLP: 4 state words and a ready word per column block of two front members
+    size_t max_nb = 1;
+    for (size_t nb : nbs) max_nb = std::max(max_nb, nb);
+    ws->chain_len = kChainStride * (1 + 2 * max_nb);
+    if (!c) c = ws->chain.zeroed(ws->chain_len * 4);
     if (!c && cus > 0) c = ws->part.alloc((size_t)cus * kFeGemmSlotsPerCu * kFeGemmPartBytes);
     // zeroed once: the unused half of the last tile of an odd count of column blocks is read (and its sums discarded)
     if (!c && max_rows >= hat_rows && max_hat) c = ws->hat.zeroed(max_hat);
@@ -712,6 +732,137 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
         FE_TRY(fe_hip_launch(kern->rot_in_group, (k + 511) / 512, rows, (uint32_t)count, 128, 1, 1, 0, s, rargs));
     }
     return launch_job(ls, count, s, xhs, ys, y_dtype, rows, ws, in, fn);
+}
+
+}  // extern "C"
+
+// mirrors MlpChain of k_exl3.hip
+struct MlpChainArgs {
+    GemvJobArgs front;
+    GemvJobArgs::Member down;
+    fe_devptr_t state;
+    uint32_t front_wgs, interleave;
+    uint32_t k1, chunk1, inv_spb1, fuse1;
+    uint32_t k2, chunk2, inv_spb2, fuse2;
+    uint32_t perm_blocks, perm_per, spin_limit, pad;
+};
+static_assert(sizeof(MlpChainArgs) == 24 + kGroupMax * 88 + 88 + 8 + 14 * 4, "MlpChain layout");
+
+static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, fe_devptr_t xh, fe_devptr_t y, fe_devptr_t z,
+                        fe_devptr_t counters) {
+    m.trellis = l->view.trellis, m.svh = l->view.svh, m.suh = l->view.suh, m.xh = xh, m.y = y, m.z = z, m.counters = counters;
+    m.n = l->n, m.programs = l->programs;
+    view_strides(l->view, &m.stride_k, &m.stride_nb);
+    const uint32_t units = (l->k / 128) * (l->n / 128);
+    m.base = units / l->programs, m.rem = units % l->programs;
+    m.inv_base = 0xffffffffu / m.base, m.inv_base1 = 0xffffffffu / (m.base + 1);
+}
+
+static uint32_t units_per_program(const fe_exl3_linear *l) {
+    const uint32_t units = (l->k / 128) * (l->n / 128);
+    return (units + l->programs - 1) / l->programs;
+}
+
+// Whether the decode MLP gate, up -> SwiGLU -> down runs as one launch: trellis linears of one width, gate and up of one
+// shape whose outputs are down's input, every stage rotating its own input at this row count, a run of the down stage
+// within the 32 units a wavefront watches, and a workspace with room for the three side by side.
+static bool mlp_chain_fits(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe_exl3_linear *d, uint32_t rows,
+                           const fe_exl3_workspace *ws, int y_dtype) {
+    if (!g || !u || !d || !ws || !g->kern->opt.mlp_chain) return false;
+    if (g->kern != u->kern || g->kern != d->kern || g->bits != u->bits || g->bits != d->bits) return false;
+    if (g->k != u->k || g->n != u->n || d->k != g->n) return false;
+    if (rows < 1 || rows > 16 || rows > ws->max_rows || y_dtype < 0 || y_dtype > 3) return false;
+    if (!fused_rotation_fits(g, rows) || !fused_rotation_fits(u, rows) || !fused_rotation_fits(d, rows)) return false;
+    if (units_per_program(d) > 32) return false;
+    if (std::max(g->k, d->k) > ws->max_k || (size_t)2 * rows * g->k * 2 > ws->xh.bytes) return false;
+    if (job_z(g, rows) + job_z(u, rows) + job_z(d, rows) > ws->z_len) return false;
+    if ((size_t)(2 * (g->n / 128) + d->n / 128) > ws->counters_len || kChainStride * (1 + 2 * (size_t)(g->n / 128)) > ws->chain_len) return false;
+    return true;
+}
+
+static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe_exl3_linear *d, fe_stream_t s, fe_devptr_t x,
+                      int x_dtype, fe_devptr_t yg, fe_devptr_t yu, fe_devptr_t y, int y_dtype, uint32_t rows,
+                      const fe_exl3_workspace *ws) {
+    const fe_exl3_kernels *kern = g->kern;
+    MlpChainArgs a{};
+    const fe_exl3_linear *front[2] = {g, u};
+    const fe_devptr_t ys[2] = {yg, yu};
+    const uint32_t occ = std::max({g->plan.occ, u->plan.occ, d->plan.occ});
+    const uint32_t places = std::max(1u, (occ ? occ : 4) * std::max(kern->cus, 1u));
+    // (as launch_job: consecutive programs of the front stage share a workgroup when they are more than the CUs hold)
+    a.fuse1 = kern->opt.fuse && rows <= 4 ? std::min(4u, std::max(1u, (g->programs + u->programs + places - 1) / places)) : 1;
+    a.fuse2 = 1;
+    size_t z_at = 0, cnt_at = 0;
+    uint32_t wgs = 0;
+    a.front.count = 2;
+    for (int i = 0; i < 2; i++) {
+        const fe_exl3_linear *l = front[i];
+        fill_member(a.front.m[i], l, ws->xh.p + (size_t)i * rows * l->k * 2, ys[i], ws->z.p + z_at * 4, ws->counters.p + cnt_at * 4);
+        a.front.first[i] = wgs;
+        wgs += (l->programs + a.fuse1 - 1) / a.fuse1;
+        z_at += job_z(l, rows), cnt_at += l->n / 128;
+    }
+    for (size_t i = 2; i <= kGroupMax; i++) a.front.first[i] = wgs;
+    a.front_wgs = wgs;
+    a.interleave = g->programs == u->programs ? 1 : 0;
+    fill_member(a.down, d, ws->xh.p, y, ws->z.p + z_at * 4, ws->counters.p + cnt_at * 4);
+    a.state = ws->chain.p;
+    a.k1 = g->k, a.k2 = d->k;
+    a.inv_spb1 = 0xffffffffu / (a.k1 / 64), a.inv_spb2 = 0xffffffffu / (a.k2 / 64);
+    const uint32_t red = rows * kRedPitch * 4;
+    auto chunk_of = [&](uint32_t run_steps) {
+        const uint32_t c = std::max(4u, ((kJobLdsBudget - red) / rows - 16) / 128 / 4 * 4);
+        return std::min(c, (run_steps + 3) / 4 * 4);
+    };
+    a.chunk1 = chunk_of(2 * a.fuse1 * std::max(units_per_program(g), units_per_program(u)));
+    a.chunk2 = chunk_of(2 * a.fuse2 * units_per_program(d));
+    uint32_t lds = red + rows * (std::max(a.chunk1, a.chunk2) * 128 + 16);
+    if (occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
+    // the down stage's programs in the order in which their inputs get ready: all column blocks of the first channels first
+    const uint32_t nbd = d->n / 128;
+    if (kern->opt.chain_perm && d->programs % nbd == 0 && d->programs / nbd > 1) a.perm_blocks = nbd, a.perm_per = d->programs / nbd;
+    a.spin_limit = kern->opt.chain_spin;
+    const uint32_t grid = a.front_wgs + (d->programs + a.fuse2 - 1) / a.fuse2;
+    uint32_t x_mode = (uint32_t)x_dtype & 1, ldx = g->k, mode = (uint32_t)y_dtype;
+    void *args[] = {&a, &x, &x_mode, &ldx, &rows, &mode};
+    return fe_hip_launch(kern->mlp[bits_slot(g->bits)], grid, 1, 1, 256, 1, 1, lds, s, args);
+}
+
+extern "C" {
+
+int fe_exl3_mlp_forward_launches(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down, uint32_t rows,
+                                 int y_dtype, const fe_exl3_workspace *ws) {
+    return mlp_chain_fits(gate, up, down, rows, ws, y_dtype) ? 1 : 0;
+}
+
+int fe_exl3_mlp_forward(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down,
+                        const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype, fe_devptr_t yg, fe_devptr_t yu,
+                        fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws) {
+    const char *fn = "fe_exl3_mlp_forward";
+    if (!gate || !up || !down || !kern || !ws || !x || !yg || !yu || !y) return fe_set_error(FE_ERR_ARG, fn, "null argument");
+    if (x_dtype != FE_DTYPE_BF16 && x_dtype != FE_DTYPE_F32) return fe_set_error(FE_ERR_ARG, fn, "x is bf16 or f32");
+    if (gate->n != up->n || down->k != gate->n) return fe_set_error(FE_ERR_SHAPE, fn, "gate and up must produce down's input");
+    if (yg % 8 || yu % 8) return fe_set_error(FE_ERR_ARG, fn, "gate / up outputs: 8-byte aligned");
+    if (mlp_chain_fits(gate, up, down, rows, ws, y_dtype))
+        return launch_mlp(gate, up, down, s, x, x_dtype, yg, yu, y, y_dtype, rows, ws);
+    const fe_exl3_linear *front[2] = {gate, up};
+    const fe_devptr_t ys[2] = {yg, yu};
+    FE_TRY(fe_exl3_linear_forward_group(front, 2, kern, s, x, x_dtype, ys, FE_DTYPE_BF16, rows, ws));
+    return fe_exl3_linear_forward_swiglu(down, kern, s, yg, yu, gate->n, y, y_dtype, rows, ws);
+}
+
+int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error) {
+    if (!ws || !error) return fe_set_error(FE_ERR_ARG, "fe_exl3_workspace_chain_status", "null argument");
+    uint32_t st[4] = {};
+    FE_TRY(fe_hip_synchronize());
+    FE_TRY(fe_hip_memcpy_dtoh(st, ws->chain.p, sizeof st));
+    *error = st[1];
+    if (st[1] || st[2]) {  // a wait ran out: the ready words and the count of that launch are void
+        FE_TRY(fe_hip_memset_d8(ws->chain.p, 0, ws->chain_len * 4, nullptr));
+        FE_TRY(fe_hip_memset_d8(ws->counters.p, 0, ws->counters_len * 4, nullptr));
+        FE_TRY(fe_hip_synchronize());
+    }
+    return 0;
 }
 
 int fe_exl3_reconstruct_hat_f16(const fe_exl3_kernels *kern, fe_stream_t s, const fe_exl3_view *w, fe_devptr_t out) {

@@ -175,6 +175,16 @@ __device__ __forceinline__ RotRaw rot_load(const RotSrc& src, const uint16_t* su
     r.s = *(const u32x2*)(suh + c);
     return r;
 }
+// The same for mode 2 when gate and up were written by other programs of this launch, possibly on another XCD: the
+// loads are agent-scope buffer loads (gs, us: resources over the two arrays), which miss this XCD's L2.
+__device__ __forceinline__ RotRaw rot_load_agent(__amdgpu_buffer_rsrc_t gs, __amdgpu_buffer_rsrc_t us, const uint16_t* suh,
+                                                 uint32_t xat, uint32_t c) {
+    RotRaw r;
+    r.xb = __builtin_amdgcn_raw_buffer_load_b64(gs, 2 * xat, 0, 16);
+    r.ub = __builtin_amdgcn_raw_buffer_load_b64(us, 2 * xat, 0, 16);
+    r.s = *(const u32x2*)(suh + c);
+    return r;
+}
 __device__ __forceinline__ u32x2 rot_finish(const RotRaw& r, uint32_t mode, uint32_t l32) {
     float v[4];
     if (mode == 1) {
@@ -478,11 +488,65 @@ __device__ __forceinline__ LaneWords<BITS> load_lane_words_buf(__amdgpu_buffer_r
     return r;
 }
 
-template <int BITS, int RG>
+
+// Timeline of the decode GEMV (a build with -DFE_GEMV_STAMPS, never the shipped one): wavefront w of workgroup g leaves
+// the 100 MHz wall clock at up to twelve points of its life at stamps[(4 g + w) * 12 + slot], u64, where stamps lies
+// 128 KB into the rotated-input area of the launch's first member (single-row launches on a workspace of 64 rows).
+#ifdef FE_GEMV_STAMPS
+#define FE_STAMP(slot)                                                                                  \
+    do {                                                                                                \
+        if (stamp_at && (threadIdx.x & 63) == 0) stamp_at[slot] = __builtin_amdgcn_s_memrealtime();     \
+    } while (0)
+#else
+#define FE_STAMP(slot) \
+    do {               \
+    } while (0)
+#endif
+
+// The decode MLP in one launch (exl3_mlp_b*): the front stage's programs (gate and up, CHAIN = 1) write their outputs
+// through to memory and publish every finished column block; the programs of the down stage (CHAIN = 2), which follow
+// them in the grid, request their first weights, wait for the blocks their channels need and rotate SwiGLU(gate, up)
+// straight from the front stage's outputs. Workgroups are dispatched in grid order, so a waiting program only ever waits
+// for programs that are already resident or done; the wait is bounded all the same (spin_limit polls, then the error
+// word is set and the program goes on with what it finds, so every launch ends). state: [0] sequence number of the
+// last completed launch, [1] error word, [2] finished column blocks of the down stage,
+// [(1 + i * nbf + b) * FE_CHAIN_STRIDE] the ready word of front member i's block b = the sequence number of the launch
+// that finished it. The down stage's last finisher advances [0]; nothing is cleared between launches, so a captured
+// launch replays. Polls are trips to memory: with the ready words packed into a few cache lines the watchers crowd
+// one memory channel and slow the front stage's own hand-offs down (56.5 us for the 27B-shaped MLP at 4 bits against
+// 46.5 us with a word per 256 bytes and 50.9 us for the two launches), and polling more often than every half
+// microsecond costs more than it finds out.
+#ifndef FE_CHAIN_STRIDE
+#define FE_CHAIN_STRIDE 64  // u32 words from one ready word to the next
+#endif
+#ifndef FE_CHAIN_SLEEP
+#define FE_CHAIN_SLEEP 16  // s_sleep units (64 cycles each) between two polls of a waiting program
+#endif
+struct ChainCtx {
+    uint32_t* state;
+    uint32_t* ready;  // front stage: this member's ready words; down stage: those of front members 0 (gate) and 1 (up)
+    uint32_t nbf;     // column blocks of a front member = 128-channel blocks of the down stage's input
+    uint32_t nb_down, spin_limit;
+};
+__device__ __forceinline__ uint32_t load_agent_u32(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int BITS, int RG, int CHAIN = 0>
 __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, uint32_t np, uint32_t k, uint32_t m, uint32_t y_mode,
-                                           uint32_t chunk, uint32_t inv_spb, const RotSrc src) {
+                                           uint32_t chunk, uint32_t inv_spb, const RotSrc src, uint16_t* stamp_base,
+                                           const ChainCtx ch = ChainCtx{}) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ uint32_t last_flag;
+    uint32_t chain_target = 0;  // this launch's sequence number
+    if constexpr (CHAIN != 0) chain_target = load_agent_u32(ch.state) + 1;
+#ifdef FE_GEMV_STAMPS
+    unsigned long long* stamp_at =
+        stamp_base && m == 1 ? (unsigned long long*)(stamp_base + 65536) + (size_t)(blockIdx.x * 4 + (threadIdx.x >> 6)) * 12 : nullptr;
+    FE_STAMP(0);
+#else
+    (void)stamp_base;
+#endif
     constexpr uint32_t tw = 8 * BITS;
     constexpr int DEPTH = 4;  // load steps in flight per lane (5 and 6 measured 2..5 % slower, 8 10 %: 22.9 against 20.7 us)
     constexpr int GROUP = 8;  // steps of straight-line code per loop iteration (a multiple of DEPTH)
@@ -547,11 +611,21 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         return a;
     };
     RotRaw rot_raw = {};
-    if (rotating) {
+    // (resources over gate and up for the down stage's agent-scope loads; unused otherwise)
+    const __amdgpu_buffer_rsrc_t chain_gs = __builtin_amdgcn_make_buffer_rsrc((void*)src.x, 0, m * src.ld * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t chain_us = __builtin_amdgcn_make_buffer_rsrc((void*)src.x2, 0, m * src.ld * 2, 0x00020000);
+    auto load_pair = [&](const RotAt& a) {
+        if constexpr (CHAIN == 2)
+            return rot_load_agent(chain_gs, chain_us, mb.suh, (uint32_t)a.xat, a.c);
+        else
+            return rot_load(src, mb.suh, a.xat, a.c);
+    };
+    const uint32_t rot_mode = CHAIN == 2 ? 2u : src.mode;
+    if (rotating && CHAIN != 2) {
         const uint32_t nblk = (S < chunk ? S : chunk) / 2;
         if (hw < nblk) {
             RotAt a = rot_at(0, 0, hw);
-            rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+            rot_raw = load_pair(a);
         }
     }
     // the output scales of this lane's four columns of the block the run stands in (for the program that finishes it)
@@ -570,6 +644,34 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
     LaneWords<BITS> ring[DEPTH];  // indexed by constants only, so it stays in registers
 #pragma unroll
     for (int j = 0; j < DEPTH; j++) issue(ring[j]);
+    FE_STAMP(1);
+    if constexpr (CHAIN == 2) {
+        // Unit j of the run reads channels block (st_run0 / 2 + j) % upb of the input: lanes 0..31 of the workgroup's first
+        // wavefront watch gate's ready words of the run's units, lanes 32..63 up's (the host keeps a run within 32 units);
+        // the other wavefronts wait at the barrier, which costs no issue slots. A poll is a trip to memory; between polls
+        // the wavefront sleeps, so that the watchers do not crowd the memory channel that holds the words.
+        uint32_t chain_spins = 0;
+        if (wave == 0) {
+            const uint32_t units = S / 2, j = lane & 31;
+            uint32_t kb = st_run0 / 2 + j;
+            kb -= kb >= upb ? upb : 0;
+            kb = kb >= upb ? kb % upb : kb;
+            const uint32_t* rw = ch.ready + ((lane >> 5) * ch.nbf + kb) * FE_CHAIN_STRIDE;
+            bool pending = true;
+            for (uint32_t spins = 0; spins < ch.spin_limit; spins++, chain_spins++) {
+                const uint32_t v = j < units ? load_agent_u32(rw) : chain_target;
+                pending = __builtin_amdgcn_ballot_w64(v != chain_target) != 0;
+                if (!pending) break;
+                __builtin_amdgcn_s_sleep(FE_CHAIN_SLEEP);
+            }
+            if (pending && lane == 0) __hip_atomic_fetch_or(ch.state + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        __syncthreads();
+        FE_STAMP(9);
+#ifdef FE_GEMV_STAMPS
+        if (stamp_at && lane == 0) stamp_at[10] = chain_spins;
+#endif
+    }
 
     auto one = [&](LaneWords<BITS>& slot, uint32_t t) {  // t: load step within the staged chunk
         f16x8 op[2][2];
@@ -598,7 +700,34 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         v[1] = v[1] * FE_HAD_SCALE * f16_bits_to_f32(sv[0] >> 16);
         v[2] = v[2] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] & 0xffff);
         v[3] = v[3] * FE_HAD_SCALE * f16_bits_to_f32(sv[1] >> 16);
-        store4(mb.y, y_mode, (size_t)row * n + col0 + 4 * l32, v);
+        if constexpr (CHAIN == 1)  // bf16, written through: the down stage's programs read it in this launch
+            store_agent_u32x2((uint16_t*)mb.y + (size_t)row * n + col0 + 4 * l32,
+                              (u32x2){pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3])});
+        else
+            store4(mb.y, y_mode, (size_t)row * n + col0 + 4 * l32, v);
+    };
+    // A column block is finished (all of the workgroup's threads come here). Front stage: once every lane's stores are
+    // acknowledged, its ready word takes this launch's number. Down stage: the block is counted, and the last one
+    // completes the launch.
+    auto block_done = [&](uint32_t fnb) {
+        if constexpr (CHAIN == 1) {
+            agent_stores_wait();
+            __syncthreads();
+            if (tid == 0) __hip_atomic_store(ch.ready + fnb * FE_CHAIN_STRIDE, chain_target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#ifdef FE_GEMV_STAMPS
+            if (tid == 0 && stamp_at)
+                ((unsigned long long*)(stamp_base + 65536))[8192 * 12 + (ch.ready - (ch.state + FE_CHAIN_STRIDE)) / FE_CHAIN_STRIDE + fnb] = __builtin_amdgcn_s_memrealtime();
+#endif
+        } else if constexpr (CHAIN == 2) {
+            if (tid == 0) {
+                const uint32_t old = __hip_atomic_fetch_add(ch.state + 2, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (old + 1 == ch.nb_down) {
+                    __hip_atomic_store(ch.state + 2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __hip_atomic_store(ch.state, chain_target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+        }
+        (void)fnb;
     };
 
     // The segment of column block fnb that ends here: its sums meet in LDS, and then either are the block's sums (the
@@ -618,6 +747,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
         }
         __syncthreads();
+        FE_STAMP(4);
         const uint32_t col0 = fnb * 128;
         // programs of the block's first and last unit
         const uint32_t cut = rem * (base + 1), ua = fnb * upb, ub = ua + upb - 1;
@@ -629,6 +759,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
                 float v[4] = {t[0], t[1], t[2], t[3]};
                 finish(v, col0, row);
             }
+            block_done(fnb);
             return;
         }
         // Hand-off of the segment's sums to another program, possibly on another XCD with its own L2:
@@ -642,12 +773,14 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         for (uint32_t row = hw; row < m; row += 8)
             store_agent_f32x4(zseg + row * 128 + 4 * l32, *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32));
         agent_stores_wait();
+        FE_STAMP(5);
         __syncthreads();
         if (tid == 0) {
             uint32_t old = __hip_atomic_fetch_add(&mb.counters[fnb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             last_flag = (old == last_prog - first_prog);
         }
         __syncthreads();
+        FE_STAMP(6);
         if (last_flag) {
             // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB segments each, 8 or 12 agent-scope
             // loads in flight (each takes a trip to memory: the trips overlap); every row's segments are added in program
@@ -692,6 +825,8 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             else
                 rows_of(std::integral_constant<int, 2>{});
             if (tid == 0) __hip_atomic_store(&mb.counters[fnb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            block_done(fnb);
+            FE_STAMP(7);
         }
     };
 
@@ -705,17 +840,17 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             const bool any = b < nblk;
             if (any) {
                 a = rot_at(c0, row, b);
-                if (c0) rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+                if (c0 || CHAIN == 2) rot_raw = load_pair(a);
             }
             while (any && row < m) {
-                u32x2 o = rot_finish(rot_raw, src.mode, l32);
+                u32x2 o = rot_finish(rot_raw, rot_mode, l32);
                 *(u32x2*)(xs + a.off) = o;
                 if (a.keep && mb.xh) *(u32x2*)(mb.xh + a.at) = o;
                 b += 8;
                 if (b >= nblk) b = hw, row++;
                 if (row < m) {
                     a = rot_at(c0, row, b);
-                    rot_raw = rot_load(src, mb.suh, a.xat, a.c);
+                    rot_raw = load_pair(a);
                 }
             }
         } else {  // rotated inputs of the chunk's load steps -> xs [row][cs * 64 fp16], NB 16-byte pieces in flight a thread
@@ -740,6 +875,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             }
         }
         __syncthreads();
+        FE_STAMP(2);
         // the chunk's load steps, segment by segment (a segment ends with its column block, with the chunk ...
         uint32_t i = 0;
         while (i < cs) {
@@ -760,6 +896,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
                     if (s0 + j < seg) one(ring[j], i + s0 + j);
             }
             ring_turn<BITS, DEPTH>(ring, seg % DEPTH);
+            FE_STAMP(3);
             i += seg, st += seg;
             const bool block_end = st == spb, run_end = c0 + i == lend;
             if (block_end || run_end) {
@@ -772,6 +909,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             }
         }
     }
+    FE_STAMP(8);
 }
 
 // (second launch bound: wavefronts per SIMD the registers must allow. Four programs a CU for up to 16 rows.)
@@ -783,9 +921,54 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         while (i + 1 < job.count && blockIdx.x >= job.first[i + 1]) i++;                                              \
         const uint32_t p0 = (blockIdx.x - job.first[i]) * fuse, left = job.m[i].programs - p0;                        \
         gemvb_body<BITS, RG>(job.m[i], p0, left < fuse ? left : fuse, k, m, y_mode, chunk, inv_spb,                   \
-                             RotSrc{x, x2, x_mode, ldx});                                                             \
+                             RotSrc{x, x2, x_mode, ldx}, job.m[0].xh);                                                \
     }
 #define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
+
+// The decode MLP in one launch, 1..16 rows: grid = the front stage's workgroups (gate and up, alternating when their
+// counts are equal, so that block b of both is finished at about the same time), then the down stage's. With perm_blocks
+// set, down workgroup w runs program (w % perm_blocks) * perm_per + w / perm_blocks: the programs of all column blocks for
+// the first channels come first, in the order in which the front stage finishes them.
+struct MlpChain {
+    GemvJob front;
+    GemvMember down;
+    uint32_t* state;
+    uint32_t front_wgs, interleave;
+    uint32_t k1, chunk1, inv_spb1, fuse1;
+    uint32_t k2, chunk2, inv_spb2, fuse2;
+    uint32_t perm_blocks, perm_per, spin_limit, pad;
+};
+#define MLP_KERNEL(BITS)                                                                                              \
+    extern "C" __global__ __launch_bounds__(256, 4) void exl3_mlp_b##BITS(MlpChain c, const void* x, uint32_t x_mode,  \
+                                                                          uint32_t ldx, uint32_t m, uint32_t y_mode) { \
+        const uint32_t w = blockIdx.x, nbf = c.front.m[0].n / 128, nbd = c.down.n / 128;                              \
+        if (w < c.front_wgs) {                                                                                        \
+            uint32_t i = 0, lw = w;                                                                                   \
+            if (c.interleave) {                                                                                       \
+                i = w & 1, lw = w >> 1;                                                                               \
+            } else {                                                                                                  \
+                while (i + 1 < c.front.count && w >= c.front.first[i + 1]) i++;                                       \
+                lw = w - c.front.first[i];                                                                            \
+            }                                                                                                         \
+            const uint32_t p0 = lw * c.fuse1, left = c.front.m[i].programs - p0;                                      \
+            gemvb_body<BITS, 1, 1>(c.front.m[i], p0, left < c.fuse1 ? left : c.fuse1, c.k1, m, 0, c.chunk1, c.inv_spb1, \
+                                   RotSrc{x, nullptr, x_mode, ldx}, c.front.m[0].xh,                                  \
+                                   ChainCtx{c.state, c.state + (1 + i * nbf) * FE_CHAIN_STRIDE, nbf, nbd, c.spin_limit}); \
+        } else {                                                                                                      \
+            uint32_t lw = w - c.front_wgs;                                                                            \
+            if (c.perm_blocks) lw = (lw % c.perm_blocks) * c.perm_per + lw / c.perm_blocks;                           \
+            const uint32_t p0 = lw * c.fuse2, left = c.down.programs - p0;                                            \
+            gemvb_body<BITS, 1, 2>(c.down, p0, left < c.fuse2 ? left : c.fuse2, c.k2, m, y_mode, c.chunk2, c.inv_spb2, \
+                                   RotSrc{c.front.m[0].y, c.front.m[1].y, 2, c.front.m[0].n}, c.front.m[0].xh,        \
+                                   ChainCtx{c.state, c.state + FE_CHAIN_STRIDE, nbf, nbd, c.spin_limit});             \
+        }                                                                                                             \
+    }
+MLP_KERNEL(2)
+MLP_KERNEL(3)
+MLP_KERNEL(4)
+MLP_KERNEL(5)
+MLP_KERNEL(6)
+MLP_KERNEL(8)
 GEMVB_FAMILY(2)
 GEMVB_FAMILY(3)
 GEMVB_FAMILY(4)

@@ -146,6 +146,9 @@ __device__ __forceinline__ uint32_t silu_mul_bf16x2(uint32_t g, uint32_t u) {
 __device__ __forceinline__ void store_agent_f32x4(float* p, f32x4 v) {
     asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
 }
+__device__ __forceinline__ void store_agent_u32x2(void* p, u32x2 v) {
+    asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
 __device__ __forceinline__ void agent_stores_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ f32x4 load_agent_f32x4(const float* p) {
     const uint64_t a = __hip_atomic_load((const uint64_t*)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -316,8 +316,25 @@ def forward_group_launches(linears, rows: int, ws: "Workspace") -> int:
     return _lib.lib().fe_exl3_linear_forward_group_launches(_group_handles(linears), len(linears), rows, ws.h)
 
 
+def mlp_forward(gate, up, down, x, x_dtype: Dtype, yg, yu, y, y_dtype: Dtype, rows: int, ws: "Workspace", stream=None):
+    """The decode MLP block: yg = x @ W_gate, yu = x @ W_up (bf16), y (+)= SwiGLU(yg, yu) @ W_down; one launch where
+    mlp_forward_launches says so, else the grouped gate + up launch followed by down's forward_swiglu (the same bits)."""
+    check(_lib.lib().fe_exl3_mlp_forward(gate.h, up.h, down.h, gate.kern.h, _stream(stream), x.data_ptr(), int(x_dtype),
+                                         yg.data_ptr(), yu.data_ptr(), y.data_ptr(), int(y_dtype), rows, ws.h))
+
+
+def mlp_forward_launches(gate, up, down, rows: int, y_dtype: Dtype, ws: "Workspace") -> int:
+    return _lib.lib().fe_exl3_mlp_forward_launches(gate.h, up.h, down.h, rows, int(y_dtype), ws.h)
+
+
 class Workspace:
     """Scratch shared by every Linear on one stream (linear.rs:136-161)."""
+
+    def chain_status(self) -> int:
+        """Synchronizes and returns the error word of the one-launch MLP (0: all its bounded waits were met); clears it."""
+        e = C.c_uint32()
+        check(_lib.lib().fe_exl3_workspace_chain_status(self.h, C.byref(e)))
+        return e.value
 
     def __init__(self, linears, max_rows: int):
         _lib.init()

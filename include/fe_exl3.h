@@ -56,7 +56,7 @@ int fe_exl3_kernels_destroy(fe_exl3_kernels *k);
 /* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
  * "fused_rot" 0/1 (FE_EXL3_NO_FUSED_ROT), "fused_rot_pairs" (FE_EXL3_FUSED_ROT_PAIRS), "group" 0/1 (FE_EXL3_NO_GROUP),
  * "hat_rows" (FE_EXL3_HAT_ROWS; 0 = never), "lds_pad" 0/1 (FE_EXL3_NO_LDS_PAD), "fuse" 0/1 (FE_EXL3_NO_FUSE), "gemm_group_m" (FE_EXL3_GROUP),
- * "gemm_splits" (FE_GEMM_SPLITS), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the prefill GEMM never / where it
+ * "gemm_splits" (FE_GEMM_SPLITS), "mlp_chain" 0/1 (FE_EXL3_NO_CHAIN), "chain_spin" (FE_EXL3_CHAIN_SPIN), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the prefill GEMM never / where it
  * is the faster one / over all tiles / whole rounds then runs, the last two for tests). forward() reads no environment variable; tests and tuners flip a switch here. Not for
  * use while launches with this handle are being issued from another thread. No counterpart in the reference, which reads
  * its switches (FE_EXL3_NOSPLIT, FE_EXL3_UNTUNED, ...) from the environment at plan time. */
@@ -126,6 +126,28 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
 /* Launches of that call: 1, 2, or 0 when the members run one after the other. */
 int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_t count, uint32_t rows,
                                           const fe_exl3_workspace *ws);
+/* The decode MLP block in one launch: yg = x @ W_gate, yu = x @ W_up (bf16 [rows][n]), y (+)= SwiGLU(yg, yu) @ W_down,
+ * with the bits of fe_exl3_linear_forward_group on {gate, up} followed by fe_exl3_linear_forward_swiglu on down, which is
+ * what it falls back to (two launches) whenever the one launch does not apply. This is the MLP block of a decode row
+ * (crates/fe-model/src/model.rs:3184-3199), where the reference launches seven kernels; the entry point has no
+ * counterpart there. In the one launch the programs of the down projection follow those of gate and up in the grid:
+ * they request their first weights at once, wait until the column blocks of gate and up that hold their input channels
+ * are published (every finished block of the front stage is written through to memory and then announced by a ready
+ * word), and rotate SwiGLU(gate, up) from there; start-up, launch overhead and tail of the second launch disappear
+ * under the first. The wait is bounded ("chain_spin" polls, about a microsecond each): when it runs out the program sets
+ * the workspace's chain error word and goes on, the launch still ends normally, and its results are void;
+ * fe_exl3_workspace_chain_status reports and clears that. It applies to 1..16 rows where all three linears rotate their
+ * own input (fe_exl3_linear_forward_is_one_launch), with the same width, gate and up of one shape, and a workspace
+ * created from (at least) these three linears; "mlp_chain" 0 (FE_EXL3_NO_CHAIN=1) turns it off.
+ * fe_exl3_mlp_forward_launches: 1 if the call is the one launch, else 0. */
+int fe_exl3_mlp_forward(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down,
+                        const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype, fe_devptr_t yg, fe_devptr_t yu,
+                        fe_devptr_t y, int y_dtype, uint32_t rows, const fe_exl3_workspace *ws);
+int fe_exl3_mlp_forward_launches(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down, uint32_t rows,
+                                 int y_dtype, const fe_exl3_workspace *ws);
+/* Synchronizes the device and returns the chain error word of the workspace (0: every bounded wait of the one-launch MLP
+ * calls so far was met), clearing it and the launch state behind it when it is set. */
+int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error);
 /* forward() for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc). No counterpart in the reference, whose forward always takes a Workspace. The
  * rotated inputs, split partial sums and arrival counters live in one static device array of FE_EXL3_STATIC_BYTES that
