@@ -6,17 +6,20 @@
 Workload (BASELINE.json configs[1]): the EXL3 decode MLP of a Qwen3.8-27B-shaped layer at M = 1, at 3, 4 and 5 bits per
 weight: gate and up are K=5120 N=17408, down is K=17408 N=5120. One step = the forward (input rotation + trellis GEMV)
 of all nine linears on seeded synthetic layers, inputs and weights resident in HBM, launched as the MLP block launches
-them: gate and up, two linears of the same input, as one grouped call (fe_exl3_linear_forward_group), down as
-Linear::forward. `value` is the trellis bytes streamed per second (the reference's numerator,
-crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole step, launch gaps and input rotations included. The nine
-weight sets total 401 MB, more than L2 plus the 256 MB Infinity Cache, so every step streams its weights from HBM.
+them: per width one call of fe_exl3_mlp_forward, y = down(SwiGLU(gate(x), up(x))), which is one kernel launch (the
+programs of down follow those of gate and up in the grid and wait for the column blocks they need). `value` is the
+trellis bytes streamed per second (the reference's numerator, crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole
+step, launch gaps and input rotations included. The nine weight sets total 401 MB, more than L2 plus the 256 MB Infinity
+Cache, so every step streams its weights from HBM. `separate_launches` is the same nine linears launched as six kernels
+(gate + up grouped, then down on an input of its own), the step of the earlier rounds of this bench.
 
-`roofline` is the dominant kernel alone (the 4-bit GEMV launch of the two 5120x17408 projections): its trellis bytes
+`roofline` is the dominant kernel alone (exl3_mlp_b4, the three 4-bit projections in one launch): its trellis bytes
 over its average launch duration, measured with HIP event pairs on the launch stream in a second pass of the same K
 steps in which every launch carries such a pair (which is also where `per_launch` comes from; `value` is taken from the
-first pass, without events: a pair costs the eager step 3.5 us a launch). It also carries the single 5120x17408 linear
-the target names and the measured decode-only ceiling of the vector ALUs (`alu_ceiling_GBs`), which splits the distance to
-the HBM roofline into "ceiling against HBM" and "kernel against ceiling".
+first pass, without events: a pair costs the eager step 3.5 us a launch). It also carries the grouped gate + up launch
+and the single 5120x17408 linear the target names, each timed alone, and the measured decode-only ceiling of the
+vector ALUs (`alu_ceiling_*`), which splits the distance to the HBM roofline into "ceiling against HBM" and "kernel
+against ceiling".
 `cpu_baseline` times the CPU oracle (the reference's factored f64 linear, threaded over 128-column blocks) on the host;
 `configs` holds, per BASELINE configuration, a CPU figure of the same kind and the parity of the GPU result against it
 (W_hat mismatches on sampled tiles, max |y - ref| / rms(ref), max relative error with the denominator floored at the rms).
@@ -181,6 +184,8 @@ def main():
     ap.add_argument("--no-configs", action="store_true", help="leave out the per-configuration CPU figures and parity")
     ap.add_argument("--bracket-events", action="store_true",
                     help="time the roofline kernel with events recorded before and after its launch instead of events attached to its dispatch")
+    ap.add_argument("--separate", action="store_true",
+                    help="the step as six launches (gate + up grouped, then down on an input of its own) instead of one launch per MLP")
     ap.add_argument("--step-only", action="store_true",
                     help="only the timed passes of the step (for a kernel trace in which every GEMV dispatch is one of the step's six launches)")
     ap.add_argument("--no-sweep", action="store_true", help="leave out the M = 1, 4, 8, 16 sweep (for a kernel trace of the step alone)")
@@ -221,14 +226,16 @@ def main():
     ws = exl3.Workspace([l[2] for l in linears], 1)
     total_bytes = sum(l[2].weight_bytes() for l in linears)
 
-    # The step's launches: per bit width, gate + up of one input as a grouped call, then down. Every argument of the calls
-    # into the C ABI is prepared once.
-    f_group, f_forward, f_rotate, f_rotated, f_record = (lib.fe_exl3_linear_forward_group, lib.fe_exl3_linear_forward,
-                                                        lib.fe_exl3_linear_rotate_input, lib.fe_exl3_linear_gemv_rotated,
-                                                        lib.fe_hip_event_record)
+    # The step's launches. Headline: per bit width one call of fe_exl3_mlp_forward, down on SwiGLU(gate(x), up(x)): one
+    # kernel launch each. Beside it the step of this bench's earlier rounds: gate + up of one input as a grouped call, then
+    # down on an input of its own, six launches. Every argument of the calls into the C ABI is prepared once.
+    f_group, f_forward, f_rotate, f_rotated, f_record, f_mlp = (lib.fe_exl3_linear_forward_group, lib.fe_exl3_linear_forward,
+                                                               lib.fe_exl3_linear_rotate_input, lib.fe_exl3_linear_gemv_rotated,
+                                                               lib.fe_hip_event_record, lib.fe_exl3_mlp_forward)
     bf16 = int(exl3.Dtype.Bf16)
     by = {(name, bits): (lin, x, y) for name, bits, lin, x, y in linears}
     launches = []  # (label, bytes, dominant, kernel launches, [(fn, args)...], keepalive)
+    chain = []
     for bits in BITS:
         (g, xg, yg), (u, _, yu), (d, xd, yd) = by[("gate", bits)], by[("up", bits)], by[("down", bits)]
         hs = (C.c_void_p * 2)(g.h, u.h)
@@ -243,6 +250,14 @@ def main():
             calls = [(f_rotate, (d.h, kern.h, stream, xd.data_ptr(), bf16, 1, ws.h)),
                      (f_rotated, (d.h, stream, ws.xh_ptr, yd.data_ptr(), bf16, 1, ws.h))]
         launches.append((f"down_b{bits}", d.weight_bytes(), False, len(calls), calls, None))
+        if exl3.mlp_forward_launches(g, u, d, 1, exl3.Dtype.Bf16, ws) == 1:
+            chain.append((f"mlp_b{bits}", g.weight_bytes() + u.weight_bytes() + d.weight_bytes(), bits == 4, 1,
+                          [(f_mlp, (g.h, u.h, d.h, kern.h, stream, xg.data_ptr(), bf16, yg.data_ptr(), yu.data_ptr(), yd.data_ptr(),
+                                    bf16, 1, ws.h))], None))
+    separate = launches
+    one_launch_mlp = len(chain) == len(BITS) and not args.separate
+    if one_launch_mlp:
+        launches = chain
 
     # Event pairs on the launch stream, one per launch of a second pass of the same K steps. A pair is attached to the dispatch of the
     # launch's last kernel (the GEMV), so it reads that kernel's own begin and end as a kernel trace does and puts no
@@ -252,69 +267,79 @@ def main():
     # of its own on the queue, which adds the dispatch gap and the packets to the reading.
     attached = not args.bracket_events
     f_time_next = lib.fe_hip_time_next_launch
-    events = [[(ev.new(), ev.new()) for _ in launches] for _ in range(args.steps)]
 
-    def step(pairs=None):
-        rc = 0
-        for li, la in enumerate(launches):
-            calls = la[4]
-            for fn, a in calls[:-1]:
+    def measure(launches):
+        """W + K steps right after the host work, the ramp, W + K steps again (`value`), then K steps with an event pair on
+        every launch."""
+        events = [[(ev.new(), ev.new()) for _ in launches] for _ in range(args.steps)]
+
+        def step(pairs=None):
+            rc = 0
+            for li, la in enumerate(launches):
+                calls = la[4]
+                for fn, a in calls[:-1]:
+                    rc |= fn(*a)
+                pair = pairs[li] if pairs is not None else None
+                attach = pair is not None and attached and la[3] == len(calls)  # the last call is one kernel launch
+                if attach:
+                    rc |= f_time_next(pair[0], pair[1])
+                elif pair is not None:
+                    rc |= f_record(pair[0], stream)
+                fn, a = calls[-1]
                 rc |= fn(*a)
-            pair = pairs[li] if pairs is not None else None
-            attach = pair is not None and attached and la[3] == len(calls)  # the last call is one kernel launch
-            if attach:
-                rc |= f_time_next(pair[0], pair[1])
-            elif pair is not None:
-                rc |= f_record(pair[0], stream)
-            fn, a = calls[-1]
-            rc |= fn(*a)
-            if pair is not None and not attach:
-                rc |= f_record(pair[1], stream)
-        _lib.check(rc)
+                if pair is not None and not attach:
+                    rc |= f_record(pair[1], stream)
+            _lib.check(rc)
 
-    def timed_steps():  # W untimed steps, then exactly K steps between two synchronizations
-        for _ in range(args.warmup):
+        def timed_steps():  # W untimed steps, then exactly K steps between two synchronizations
+            for _ in range(args.warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                step()
+            torch.cuda.synchronize()
+            return time.perf_counter() - t0
+
+        # The GPU comes out of the host work before this point (the CPU baseline, the uploads) at its idle clocks and takes
+        # about 30 ms of continuous launches to reach the clocks it then holds: the same K steps read 2230 GB/s right after
+        # idle, 2400 after 8 ms, 2500 after 16 ms and 2560 from 32 ms on (no further change up to 250 ms). A decode loop runs
+        # in that steady state, so `value` is taken there: `after_idle` is the reading right after the host work, then the
+        # steps run untimed for --ramp-ms, then W + K steps again.
+        r = {}
+        r["dt_idle"] = timed_steps()
+        r["ramp_steps"] = int(args.ramp_ms * 1e-3 / (r["dt_idle"] / args.steps)) + 1 if args.ramp_ms > 0 else 0
+        for _ in range(r["ramp_steps"]):
             step()
-        torch.cuda.synchronize()
+        r["dt"] = timed_steps() if r["ramp_steps"] else r["dt_idle"]
+        # the same K steps once more with an event pair on every launch, for the roofline kernel's own duration and the
+        # per-launch table (the pairs cost the eager step 3.5 us a launch, so `value` is taken without them)
         t0 = time.perf_counter()
         for i in range(args.steps):
-            step()
+            step(events[i])
         torch.cuda.synchronize()
-        return time.perf_counter() - t0
+        r["ms_per_step_timed"] = (time.perf_counter() - t0) * 1e3 / args.steps
+        r["dom_ms"] = []
+        for li, la in enumerate(launches):
+            if la[2]:
+                r["dom_ms"] += [ev.ms(*events[i][li]) for i in range(args.steps)]
+                r["dom_bytes"] = la[1]
+        r["per"] = {}
+        for li, la in enumerate(launches):  # every launch of the timed region, by its own events
+            us = sum(ev.ms(*events[i][li]) for i in range(args.steps)) / args.steps * 1e3
+            r["per"][la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
+        return r
 
-    # The GPU comes out of the host work before this point (the CPU baseline, the uploads) at its idle clocks and takes
-    # about 30 ms of continuous launches to reach the clocks it then holds: the same K steps read 2230 GB/s right after
-    # idle, 2400 after 8 ms, 2500 after 16 ms and 2560 from 32 ms on (no further change up to 250 ms). A decode loop runs
-    # in that steady state, so `value` is taken there: `after_idle` is the reading right after the host work, then the
-    # steps run untimed for --ramp-ms, then W + K steps again.
-    dt_idle = timed_steps()
-    ramp_steps = int(args.ramp_ms * 1e-3 / (dt_idle / args.steps)) + 1 if args.ramp_ms > 0 else 0
-    for _ in range(ramp_steps):
-        step()
-    dt = timed_steps() if ramp_steps else dt_idle
+    head = measure(launches)
+    dt_idle, dt, ramp_steps, ms_per_step_timed, per = head["dt_idle"], head["dt"], head["ramp_steps"], head["ms_per_step_timed"], head["per"]
     ms_per_step = dt * 1e3 / args.steps
     value = total_bytes / (dt / args.steps) / 1e9
-    # the same K steps once more with an event pair on every launch, for the roofline kernel's own duration and the
-    # per-launch table (the pairs cost the eager step 3.5 us a launch, so `value` is taken without them)
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(events[i])
-    torch.cuda.synchronize()
-    ms_per_step_timed = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    dom_ms = []
-    for li, la in enumerate(launches):
-        if la[2]:
-            dom_ms += [ev.ms(*events[i][li]) for i in range(args.steps)]
-            dom_bytes = la[1]
-    dom_kernel = "exl3_gemvb_b4_r1"
+    dom_ms, dom_bytes = head["dom_ms"], head["dom_bytes"]
+    dom_kernel = "exl3_mlp_b4" if one_launch_mlp else "exl3_gemvb_b4_r1"
     dom_avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (dom_avg_ms * 1e-3) / 1e9
-
-    per = {}
-    for li, la in enumerate(launches):  # every launch of the timed region, by its own events
-        us = sum(ev.ms(*events[i][li]) for i in range(args.steps)) / args.steps * 1e3
-        per[la[0]] = {"us": round(us, 2), "GB/s": round(la[1] / us / 1e3, 1), "launches": la[3]}
+    if one_launch_mlp:
+        assert ws.chain_status() == 0, "a bounded wait of the one-launch MLP ran out"
 
     if args.step_only:
         print(json.dumps({"metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048", "value": round(value, 2),
@@ -324,35 +349,53 @@ def main():
                                        "achieved": round(achieved, 2), "frac": round(achieved / HBM_PEAK_GBS, 4)},
                           "per_launch": per}))
         return
+    # the six-launch step of the earlier rounds, measured the same way
+    sep = measure(separate) if one_launch_mlp else head
+    sep_value = total_bytes / (sep["dt"] / args.steps) / 1e9
+    sep_dom_us = sum(sep["dom_ms"]) / len(sep["dom_ms"]) * 1e3
 
-    # The dominant launch and the single linear the target names, each alone and back to back between one pair of
-    # events, cycling over weight copies past the caches: the kernel's duration plus the gap between two launches.
-    g4, u4 = by[("gate", 4)][0], by[("up", 4)][0]
+    # The dominant launch, the grouped gate + up launch and the single linear the target names, each alone: back to back
+    # between one pair of events, eagerly launched and replayed from a graph (no host time between the launches), cycling
+    # over weight copies past the caches. A launch period is an upper bound of the kernel's duration.
+    g4, u4, d4 = by[("gate", 4)][0], by[("up", 4)][0], by[("down", 4)][0]
     x4 = by[("gate", 4)][1]
-    pair_sets, keep1 = cold_copies(torch, exl3, kern, [g4, u4])
-    ws_pair = exl3.Workspace([g4, u4], 1)
+    mlp_sets, keep1 = cold_copies(torch, exl3, kern, [g4, u4, d4])
+    ws_alone = exl3.Workspace([g4, u4, d4], 1)
     ys_pair = [by[("gate", 4)][2], by[("up", 4)][2]]
+    y_down = by[("down", 4)][2]
     at = [0]
 
-    def dom_call():
-        exl3.forward_group(pair_sets[at[0] % len(pair_sets)], x4, exl3.Dtype.Bf16, ys_pair, exl3.Dtype.Bf16, 1, ws_pair, stream=stream)
+    def mlp_call(s=stream):
+        g, u, d = mlp_sets[at[0] % len(mlp_sets)]
+        exl3.mlp_forward(g, u, d, x4, exl3.Dtype.Bf16, ys_pair[0], ys_pair[1], y_down, exl3.Dtype.Bf16, 1, ws_alone, stream=s)
         at[0] += 1
 
-    dom_b2b_us = ev.loop_us(stream, dom_call, 4 * len(pair_sets))
-
-    def single_call():
-        pair_sets[at[0] % len(pair_sets)][0].forward(x4, exl3.Dtype.Bf16, ys_pair[0], exl3.Dtype.Bf16, 1, ws_pair, stream=stream)
+    def pair_call(s=stream):
+        exl3.forward_group(mlp_sets[at[0] % len(mlp_sets)][:2], x4, exl3.Dtype.Bf16, ys_pair, exl3.Dtype.Bf16, 1, ws_alone, stream=s)
         at[0] += 1
 
-    single_us = ev.loop_us(stream, single_call, 8 * len(pair_sets))
-    # ... and its kernel alone, by events attached to the dispatch (what a kernel trace reports)
-    one_pairs = [(ev.new(), ev.new()) for _ in range(2 * len(pair_sets))]
+    def single_call(s=stream):
+        mlp_sets[at[0] % len(mlp_sets)][0].forward(x4, exl3.Dtype.Bf16, ys_pair[0], exl3.Dtype.Bf16, 1, ws_alone, stream=s)
+        at[0] += 1
+
+    alone = {}
+    for name, fn, nbytes in (("mlp_b4", mlp_call, dom_bytes if one_launch_mlp else g4.weight_bytes() + u4.weight_bytes() + d4.weight_bytes()),
+                             ("gate_up_b4", pair_call, g4.weight_bytes() + u4.weight_bytes()),
+                             ("single_5120x17408_b4", single_call, g4.weight_bytes())):
+        eager_us = ev.loop_us(stream, fn, 4 * len(mlp_sets))
+        replay_us = graph_us(lib, _lib.check, ev, fn, 2 * len(mlp_sets))
+        alone[name] = {"bytes_per_launch": nbytes, "eager_period_us": round(eager_us, 3), "graph_replay_period_us": round(replay_us, 3),
+                       "GB/s": round(nbytes / replay_us / 1e3, 1), "frac": round(nbytes / replay_us / 1e3 / HBM_PEAK_GBS, 4)}
+    alone["mlp_b4"]["launches"] = 1 if one_launch_mlp else 2
+    # ... and the single linear's kernel by events attached to its dispatch, every launch carrying a pair. The host cannot
+    # keep the queue full at this pace (a launch with a pair costs it more than the kernel lasts), so each kernel starts on
+    # an idle GPU and reads longer than the launch period above: reported, not used.
+    one_pairs = [(ev.new(), ev.new()) for _ in range(2 * len(mlp_sets))]
     for a, b in one_pairs:
         _lib.check(f_time_next(a, b))
         single_call()
-    single_kernel_us = sum(ev.ms(a, b) for a, b in one_pairs) / len(one_pairs) * 1e3
-    single_bytes = g4.weight_bytes()
-    del pair_sets, keep1
+    alone["single_5120x17408_b4"]["attached_events_on_an_idle_queue_us"] = round(sum(ev.ms(a, b) for a, b in one_pairs) / len(one_pairs) * 1e3, 3)
+    del mlp_sets, keep1, ws_alone
 
     # the decode-only ceiling of the vector ALUs: the GEMV's decode at the GEMV's occupancy with no memory traffic
     ceiling = {}
@@ -364,33 +407,48 @@ def main():
         ms = kern.probe_decode(bits, grid, iters, 20)
         ceiling[f"b{bits}"] = round(grid * 256 * 32 * iters * bits / 8 / (ms * 1e-3) / 1e9, 1)
 
+    single, pair = alone["single_5120x17408_b4"], alone["gate_up_b4"]
+    untimed = 2 * args.warmup + args.steps + ramp_steps  # steps in front of the K steps of `value`
     out = {
         "metric": "quant linear GB/s (%HBM peak) at M=1; TFLOP/s (%MFMA peak) at M=2048",
         "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ramp_steps": ramp_steps, "untimed_steps_total": untimed,
+        "after_idle_value": round(total_bytes / (dt_idle / args.steps) / 1e9, 2),
         "ms_per_step": round(ms_per_step, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "EXL3 decode MLP, Qwen3.8-27B-shaped layer, M=1, 3/4/5 bpw (gate, up 5120x17408; down 17408x5120)",
-                   "linears_per_step": len(linears), "trellis_bytes_per_step": total_bytes, "seed": SEED,
-                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2)},
-        "roofline": {"bound": "hbm", "kernel": f"{dom_kernel} (gate + up in one launch, 5120x17408 each, 4 bits, M=1)",
+                   "linears_per_step": len(linears), "kernel_launches_per_step": sum(la[3] for la in launches),
+                   "trellis_bytes_per_step": total_bytes, "seed": SEED,
+                   "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+                   "untimed_steps_total": untimed, "ramp_steps": ramp_steps,
+                   "after_idle_value": round(total_bytes / (dt_idle / args.steps) / 1e9, 2),
+                   "separate_launches_value": round(sep_value, 2)},
+        "roofline": {"bound": "hbm",
+                     "kernel": (f"{dom_kernel} (gate, up and down of the 4-bit MLP in one launch, M=1)" if one_launch_mlp else
+                                f"{dom_kernel} (gate + up in one launch, 5120x17408 each, 4 bits, M=1)"),
                      "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": ROOFLINE_TRAFFIC_BYTES, "traffic_source": ROOFLINE_TRAFFIC_SOURCE,
+                     "traffic": ROOFLINE_TRAFFIC_BYTES if one_launch_mlp else None, "traffic_source": ROOFLINE_TRAFFIC_SOURCE,
                      "avg_launch_us": round(dom_avg_ms * 1e3, 3), "bytes_per_launch": dom_bytes, "launches": len(dom_ms),
                      "timed_in": f"a second pass of the {args.steps} steps with an event pair on every launch ({ms_per_step_timed:.5f} ms a step)",
-                     "back_to_back_cold_us": round(dom_b2b_us, 3),
                      "events": "recorded around the launch" if args.bracket_events else "attached to the kernel's dispatch",
-                     "alu_ceiling_GBs": ceiling,
+                     "alu_ceiling_b3_GBs": ceiling["b3"], "alu_ceiling_b4_GBs": ceiling["b4"], "alu_ceiling_b5_GBs": ceiling["b5"],
                      "frac_of_alu_ceiling": round(achieved / ceiling["b4"], 4),
-                     "single_linear_5120x17408_b4_m1": {
-                         "kernel_us": round(single_kernel_us, 3), "GB/s": round(single_bytes / single_kernel_us / 1e3, 1),
-                         "frac": round(single_bytes / single_kernel_us / 1e3 / HBM_PEAK_GBS, 4),
-                         "back_to_back_cold_us": round(single_us, 3), "bytes_per_launch": single_bytes}},
+                     "graph_replay_period_us": alone["mlp_b4"]["graph_replay_period_us"],
+                     "gate_up_launch_us": round(sep_dom_us, 3),
+                     "gate_up_launch_frac": round(pair["bytes_per_launch"] / sep_dom_us / 1e3 / HBM_PEAK_GBS, 4),
+                     "gate_up_launch_period_us": pair["graph_replay_period_us"],
+                     "single_linear_us": single["graph_replay_period_us"], "single_linear_frac": single["frac"],
+                     "alone": alone},
         "cpu_baseline": cpu,
         "per_launch": per,
         "after_idle": {"value": round(total_bytes / (dt_idle / args.steps) / 1e9, 2), "unit": "GB/s",
                        "ms_per_step": round(dt_idle * 1e3 / args.steps, 5),
                        "what": f"the same {args.warmup} + {args.steps} steps right after the host work, before the {ramp_steps} "
                                f"untimed steps ({args.ramp_ms:g} ms) that bring the GPU to the clocks it holds in a decode loop"},
+        "separate_launches": {"value": round(sep_value, 2), "unit": "GB/s", "ms_per_step": round(sep["dt"] * 1e3 / args.steps, 5),
+                              "kernel_launches_per_step": sum(la[3] for la in separate), "per_launch": sep["per"],
+                              "what": "gate + up as one grouped launch, then down on an input of its own: the step of this bench's "
+                                      "earlier rounds"},
     }
 
     out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup, ramp_steps)
@@ -530,26 +588,26 @@ def configs(torch, np, exl3, fp4, synth, kern, ev, stream, tensors, by, ws):
 
 def traffic_pass(torch, np, exl3, synth):
     """Three rounds of: evict (an elementwise update of 600 MiB: reads 600 MiB, writes 600 MiB), exl3_probe_v4 reading
-    exactly the roofline kernel's algorithmic bytes, evict, the roofline kernel. Prints the known sizes."""
+    exactly the roofline kernel's algorithmic bytes, evict, the roofline kernel (the 4-bit MLP in one launch). Prints the
+    known sizes."""
     kern = exl3.Kernels.load()
-    k, n = 5120, 17408
     blocks = exl3.default_blocks(exl3.cu_count())
-    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, n, 4, SEED, name)), blocks) for name in ("gate", "up")]
+    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(k, n, 4, SEED, name)), blocks) for name, k, n in MLP]
     ws = exl3.Workspace(lins, 1)
-    x = torch.from_numpy(synth.activations(1, k, SEED).view(np.int16)).cuda()
-    ys = [torch.zeros((1, n), dtype=torch.bfloat16, device="cuda") for _ in lins]
+    x = torch.from_numpy(synth.activations(1, 5120, SEED).view(np.int16)).cuda()
+    ys = [torch.zeros((1, l.n), dtype=torch.bfloat16, device="cuda") for l in lins]
     nbytes = sum(l.weight_bytes() for l in lins)
     buf = torch.zeros(nbytes, dtype=torch.uint8, device="cuda")
     big = torch.zeros(600 << 20, dtype=torch.uint8, device="cuda")
-    assert exl3.forward_group_launches(lins, 1, ws) == 1
+    assert exl3.mlp_forward_launches(*lins, 1, exl3.Dtype.Bf16, ws) == 1
     for _ in range(3):
         big.add_(1)
         kern.probe_stream_read(buf, 1024, 1)
         big.add_(1)
-        exl3.forward_group(lins, x, exl3.Dtype.Bf16, ys, exl3.Dtype.Bf16, 1, ws)
+        exl3.mlp_forward(*lins, x, exl3.Dtype.Bf16, ys[0], ys[1], ys[2], exl3.Dtype.Bf16, 1, ws)
     torch.cuda.synchronize()
     print(json.dumps({"exl3_probe_v4_reads_KiB": nbytes / 1024, "elementwise_reads_and_writes_KiB": (600 << 20) / 1024,
-                      "roofline_kernel": "exl3_gemvb_b4_r1", "algorithmic_KiB": nbytes / 1024}))
+                      "roofline_kernel": "exl3_mlp_b4", "algorithmic_KiB": nbytes / 1024}))
 
 
 def graph_us(lib, check, ev, fn, inner, reps=5):
@@ -581,7 +639,8 @@ def graph_us(lib, check, ev, fn, inner, reps=5):
 
 
 def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
-    """The 4-bit MLP and the attention projections at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts):
+    """The 4-bit MLP and the attention projections at M = 1, 4, 8, 16 (BASELINE's decode / speculative-verify row counts)
+    and 32, 64 (the reference's all-linear times, crates/fe-exl3/BENCH.md:103):
     microseconds per linear, launched back to back as the step launches them (gate + up grouped, then down; q, k, v grouped,
     then o), cycling over weight copies of at least 512 MB in all, eagerly launched and replayed from a graph. Not part of
     `value`."""
@@ -595,7 +654,7 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
     abytes = sum(l.weight_bytes() for l in (q, kk, v, o))
     nbytes = (g.weight_bytes() + u.weight_bytes() + d.weight_bytes()) / 3
     res = {"weight_copies_cycled": {"mlp": len(mlp_sets), "attn": len(attn_sets)}}
-    for m in (1, 4, 8, 16):
+    for m in (1, 4, 8, 16, 32, 64):
         ws = exl3.Workspace([g, u, d, q, kk, v, o], m)
         x = torch.from_numpy(synth.activations(m, g.k, SEED).view(np.int16)).cuda()
         xd = torch.from_numpy(synth.activations(m, d.k, SEED).view(np.int16)).cuda()
@@ -617,8 +676,7 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
         def block(s=stream):
             gg, uu, dd = mlp_sets[at[0] % len(mlp_sets)]
             at[0] += 1
-            exl3.forward_group([gg, uu], x, exl3.Dtype.Bf16, [yg, yu], exl3.Dtype.Bf16, m, ws, stream=s)
-            dd.forward_swiglu(yg, yu, g.n, resid, exl3.Dtype.Bf16Add, m, ws, stream=s)
+            exl3.mlp_forward(gg, uu, dd, x, exl3.Dtype.Bf16, yg, yu, resid, exl3.Dtype.Bf16Add, m, ws, stream=s)
 
         def attn(s=stream):
             qq, k2, vv, oo = attn_sets[at[0] % len(attn_sets)]
@@ -628,7 +686,8 @@ def rows_sweep(torch, np, exl3, synth, kern, ev, stream, lib, check, linears):
 
         us = ev.loop_us(stream, mlp, 3 * len(mlp_sets)) / 3
         r = {"us_per_linear": round(us, 2), "GB/s": round(nbytes / us / 1e3, 1), "frac_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4),
-             "gate_up_launches": exl3.forward_group_launches([g, u], m, ws)}
+             "gate_up_launches": exl3.forward_group_launches([g, u], m, ws),
+             "mlp_block_is_one_launch": bool(exl3.mlp_forward_launches(g, u, d, m, exl3.Dtype.Bf16Add, ws))}
         r["mlp_block_us"] = round(ev.loop_us(stream, block, 3 * len(mlp_sets)), 2)
         r["mlp_block_graph_us"] = round(graph_us(lib, check, ev, block, 2 * len(mlp_sets)), 2)
         a_us = ev.loop_us(stream, attn, 2 * len(attn_sets))

@@ -79,6 +79,7 @@ struct fe_exl3_linear {
     fe_exl3_view view{};
     FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
     FeBuf hat;                // decoded fp16 tiles kept with the linear (fe_exl3_linear_keep_decoded), else empty
+    FeBuf chain_order;        // u32[programs]: the programs sorted by the last channel block their run reads (one-launch MLP)
     const fe_exl3_kernels *kern = nullptr;
 };
 
@@ -264,6 +265,21 @@ static uint32_t plan_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p
     return std::max(1u, std::min(progs, units));
 }
 
+// The programs of the linear's partition in the order in which, as the down projection of a one-launch MLP, their inputs
+// get ready: sorted by the last 128-channel block their run reads (a run that crosses into the next column block reads
+// the last block of all), then by where the run starts.
+static int make_chain_order(fe_exl3_linear *l) {
+    const uint32_t upb = l->k / 128, units = upb * (l->n / 128), base = units / l->programs, rem = units % l->programs;
+    std::vector<uint32_t> order(l->programs), last(l->programs);
+    for (uint32_t p = 0; p < l->programs; p++) {
+        const uint32_t u0 = p * base + std::min(p, rem), len = base + (p < rem ? 1 : 0), kb0 = u0 % upb;
+        order[p] = p;
+        last[p] = kb0 + len > upb ? upb - 1 : kb0 + len - 1;
+    }
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return last[a] < last[b]; });
+    return l->chain_order.from_host(order.data(), order.size() * 4);
+}
+
 static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, const fe_exl3_plan &p) {
     char msg[160];
     if (bits_slot(bits) < 0) {
@@ -291,6 +307,10 @@ int fe_exl3_linear_from_view(fe_exl3_linear **out, const fe_exl3_kernels *kern, 
     l->view = *view;
     l->kern = kern;
     l->programs = plan_programs(kern, *plan, view->k, view->n);
+    if (int c = make_chain_order(l)) {
+        delete l;
+        return c;
+    }
     *out = l;
     return 0;
 }
@@ -323,6 +343,7 @@ int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, con
     }
     if (!c) c = l->suh.from_host(suh, (size_t)k * 2);
     if (!c) c = l->svh.from_host(svh, (size_t)n * 2);
+    if (!c) c = make_chain_order(l);
     if (c) {
         delete l;
         return c;
@@ -740,13 +761,13 @@ int fe_exl3_linear_forward_group(const fe_exl3_linear *const *ls, size_t count, 
 struct MlpChainArgs {
     GemvJobArgs front;
     GemvJobArgs::Member down;
-    fe_devptr_t state;
+    fe_devptr_t state, perm;
     uint32_t front_wgs, interleave;
     uint32_t k1, chunk1, inv_spb1, fuse1;
     uint32_t k2, chunk2, inv_spb2, fuse2;
-    uint32_t perm_blocks, perm_per, spin_limit, pad;
+    uint32_t spin_limit, pad;
 };
-static_assert(sizeof(MlpChainArgs) == 24 + kGroupMax * 88 + 88 + 8 + 14 * 4, "MlpChain layout");
+static_assert(sizeof(MlpChainArgs) == 24 + kGroupMax * 88 + 88 + 16 + 12 * 4, "MlpChain layout");
 
 static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, fe_devptr_t xh, fe_devptr_t y, fe_devptr_t z,
                         fe_devptr_t counters) {
@@ -818,9 +839,8 @@ static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe
     a.chunk2 = chunk_of(2 * a.fuse2 * units_per_program(d));
     uint32_t lds = red + rows * (std::max(a.chunk1, a.chunk2) * 128 + 16);
     if (occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
-    // the down stage's programs in the order in which their inputs get ready: all column blocks of the first channels first
-    const uint32_t nbd = d->n / 128;
-    if (kern->opt.chain_perm && d->programs % nbd == 0 && d->programs / nbd > 1) a.perm_blocks = nbd, a.perm_per = d->programs / nbd;
+    // the down stage's programs in the order in which their inputs get ready (the linear's table)
+    a.perm = kern->opt.chain_perm ? d->chain_order.p : 0;
     a.spin_limit = kern->opt.chain_spin;
     const uint32_t grid = a.front_wgs + (d->programs + a.fuse2 - 1) / a.fuse2;
     uint32_t x_mode = (uint32_t)x_dtype & 1, ldx = g->k, mode = (uint32_t)y_dtype;

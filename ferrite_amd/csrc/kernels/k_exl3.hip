@@ -926,17 +926,18 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
 #define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
 
 // The decode MLP in one launch, 1..16 rows: grid = the front stage's workgroups (gate and up, alternating when their
-// counts are equal, so that block b of both is finished at about the same time), then the down stage's. With perm_blocks
-// set, down workgroup w runs program (w % perm_blocks) * perm_per + w / perm_blocks: the programs of all column blocks for
-// the first channels come first, in the order in which the front stage finishes them.
+// counts are equal, so that block b of both is finished at about the same time), then the down stage's. Down workgroup
+// w runs program perm[w] (the host's table: the programs sorted by the last channel block their run reads, so that they
+// come in the order in which the front stage finishes their inputs; null: program w).
 struct MlpChain {
     GemvJob front;
     GemvMember down;
     uint32_t* state;
+    const uint32_t* perm;
     uint32_t front_wgs, interleave;
     uint32_t k1, chunk1, inv_spb1, fuse1;
     uint32_t k2, chunk2, inv_spb2, fuse2;
-    uint32_t perm_blocks, perm_per, spin_limit, pad;
+    uint32_t spin_limit, pad;
 };
 #define MLP_KERNEL(BITS)                                                                                              \
     extern "C" __global__ __launch_bounds__(256, 4) void exl3_mlp_b##BITS(MlpChain c, const void* x, uint32_t x_mode,  \
@@ -956,7 +957,7 @@ struct MlpChain {
                                    ChainCtx{c.state, c.state + (1 + i * nbf) * FE_CHAIN_STRIDE, nbf, nbd, c.spin_limit}); \
         } else {                                                                                                      \
             uint32_t lw = w - c.front_wgs;                                                                            \
-            if (c.perm_blocks) lw = (lw % c.perm_blocks) * c.perm_per + lw / c.perm_blocks;                           \
+            if (c.perm) lw = c.perm[lw];                                                                              \
             const uint32_t p0 = lw * c.fuse2, left = c.down.programs - p0;                                            \
             gemvb_body<BITS, 1, 2>(c.down, p0, left < c.fuse2 ? left : c.fuse2, c.k2, m, y_mode, c.chunk2, c.inv_spb2, \
                                    RotSrc{c.front.m[0].y, c.front.m[1].y, 2, c.front.m[0].n}, c.front.m[0].xh,        \

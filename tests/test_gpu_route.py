@@ -333,6 +333,13 @@ def test_mlp_block_routes_as_the_reference(env, oracle):
     assert np.array_equal(got12[:12], by_hand_decode(12)[0]) and np.array_equal(got12[12:], x_b[12:])
     assert np.array_equal(got12[:dec], got[:dec])  # a decode row's bits do not depend on the batch around it
 
+    # a single decode row: the three trellis linears as one launch (fe_exl3_mlp_forward), the bits of the steps by hand
+    assert exl3.mlp_forward_launches(e.q_gate, e.q_up, e.q_down, 1, exl3.Dtype.Bf16Add, e.xws) == 1
+    got1 = run(1, 0, e.p_sw)
+    assert np.array_equal(got1[:1], by_hand_decode(1)[0]) and np.array_equal(got1[1:], x_b[1:])
+    assert np.array_equal(got1[:1], got[:1])
+    assert e.xws.chain_status() == 0
+
     # without the fused front: prompt rows through the fused gate|up GEMM, fe_silu_mul and down's prompt linear
     got_unfused = run(rows, dec, None)
     assert np.array_equal(got_unfused[:dec], hand_dec)
