@@ -42,6 +42,7 @@ SYMBOLS = {
     "fe_hip_malloc": (I, [C.POINTER(U64), SZ]),
     "fe_hip_free": (I, [U64]),
     "fe_hip_canary_on": (I, []),
+    "fe_hip_zero_alloc_on": (I, []),
     "fe_hip_canary_tails": (I, [P, SZ, C.POINTER(SZ)]),
     "fe_hip_memset_d8": (I, [U64, C.c_uint8, SZ, P]),
     "fe_hip_memset_d32": (I, [U64, U32, SZ, P]),
@@ -85,6 +86,7 @@ SYMBOLS = {
     "fe_exl3_linear_forward_static": (I, [P, P, P, U64, I, U64, I, U32]),
     "fe_exl3_linear_forward_is_one_launch": (I, [P, U32]),
     "fe_exl3_linear_keep_decoded": (I, [P, P, I]),
+    "fe_exl3_linear_decoded": (I, [P, C.POINTER(U64), C.POINTER(SZ)]),
     "fe_exl3_linear_forward_swiglu": (I, [P, P, P, U64, U64, U32, U64, I, U32, P]),
     "fe_exl3_linear_forward_group": (I, [PP, SZ, P, P, U64, I, C.POINTER(U64), I, U32, P]),
     "fe_exl3_linear_forward_group_launches": (I, [PP, SZ, U32, P]),

@@ -672,6 +672,13 @@ int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on) {
     return c;
 }
 
+int fe_exl3_linear_decoded(const fe_exl3_linear *l, fe_devptr_t *tiles, size_t *bytes) {
+    if (!l) return fe_set_error(FE_ERR_ARG, "fe_exl3_linear_decoded", "null linear");
+    if (tiles) *tiles = l->hat.p;
+    if (bytes) *bytes = l->hat.bytes;
+    return 0;
+}
+
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows) { return l && fused_rotation_fits(l, rows); }
 
 int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype,

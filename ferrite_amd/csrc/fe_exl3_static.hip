@@ -7,6 +7,7 @@
 // hipGetSymbolAddress returned for the current device (static_base), as kernel argument and for clearing.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdio>
 
 #include "fe_exl3.h"
@@ -22,38 +23,30 @@ constexpr size_t kXhBytes = (size_t)FE_EXL3_STATIC_ROWS * 32768 * 2;  // fp16 [r
 static_assert(kCounterBytes + kXhBytes < FE_EXL3_STATIC_BYTES, "no room for partial sums");
 constexpr int kMaxDevices = 64;
 
-void *g_base[kMaxDevices];  // device address of `scratch` on each device, once set up
+std::atomic<void *> g_base[kMaxDevices];  // device address of `scratch` on each device, once taken
 
-__global__ void fe_static_zero(uint32_t *p, uint32_t n) {
-    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) p[i] = 0;
-}
-
-// Once per device, with that device current: the array's address on this device, counters cleared (they are zero at
-// rest afterwards: the kernel that finishes a column block re-arms its counter).
-int static_setup(int dev, hipStream_t s) {
+// The array's address on the current device `dev`. Nothing is cleared: a file-scope device array is zero when its
+// module is loaded, the arrival counters are zero at rest (the program that finishes a column block re-arms its
+// counter), and the other two areas are written before they are read. Threads that come here together take the same
+// address and store the same value.
+int static_setup(int dev) {
     void *p = nullptr;
     hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !p) return fe_check_hip(e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol, "hipGetSymbolAddress(scratch)");
-    // a fill kernel, not hipMemsetAsync: the first call may come under stream capture
-    fe_static_zero<<<(uint32_t)(kCounterBytes / 4 / 256), 256, 0, s>>>((uint32_t *)p, (uint32_t)(kCounterBytes / 4));
-    e = hipGetLastError();
-    if (e != hipSuccess) return fe_check_hip((int)e, "fe_static_zero");
-    g_base[dev] = p;
+    g_base[dev].store(p, std::memory_order_release);
     return 0;
 }
 
 }  // namespace
 
-// Called by fe_hip_init for the device it binds (set-up outside any capture, synchronized).
+// Called by fe_hip_init for the device it binds (outside any capture).
 int fe_exl3_static_setup_current_device() {
     int dev = -1;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fe_check_hip((int)e, "hipGetDevice");
     if (dev < 0 || dev >= kMaxDevices) return fe_set_error(FE_ERR_UNSUPPORTED, "fe_exl3_static_setup", "device ordinal above 63");
-    if (g_base[dev]) return 0;
-    FE_TRY(static_setup(dev, nullptr));
-    return fe_check_hip((int)hipDeviceSynchronize(), "hipDeviceSynchronize");
+    if (g_base[dev].load(std::memory_order_acquire)) return 0;
+    return static_setup(dev);
 }
 
 extern "C" int fe_exl3_linear_forward_static(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
@@ -64,9 +57,10 @@ extern "C" int fe_exl3_linear_forward_static(const fe_exl3_linear *l, const fe_e
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fe_check_hip((int)e, "hipGetDevice");
     if (dev < 0 || dev >= kMaxDevices) return fe_set_error(FE_ERR_UNSUPPORTED, fn, "device ordinal above 63");
-    // a device the caller made current without fe_hip_init: set up on the call's stream, ahead of the kernels
-    if (!g_base[dev]) FE_TRY(static_setup(dev, (hipStream_t)s));
-    const fe_devptr_t base = (fe_devptr_t)(uintptr_t)g_base[dev];
+    // a device the caller made current without fe_hip_init: take the address now (under stream capture HIP may refuse
+    // that; fe_hip_init on the device beforehand avoids it)
+    if (!g_base[dev].load(std::memory_order_acquire)) FE_TRY(static_setup(dev));
+    const fe_devptr_t base = (fe_devptr_t)(uintptr_t)g_base[dev].load(std::memory_order_acquire);
     return fe_exl3_forward_over(l, kern, s, x, x_dtype, y, y_dtype, rows, FE_EXL3_STATIC_ROWS, base, kCounterBytes,
                                 base + kCounterBytes, kXhBytes, base + kCounterBytes + kXhBytes,
                                 FE_EXL3_STATIC_BYTES - kCounterBytes - kXhBytes, fn);

@@ -80,31 +80,41 @@ namespace {
 constexpr size_t kCanaryPad = 64 << 10;
 std::mutex g_canary_lock;
 std::vector<std::pair<fe_devptr_t, size_t>> g_canary_live;
-bool env_flag(const char *name, bool fallback) {
+// The reference's reading of the two variables (crates/fe-cuda/src/lib.rs:307-316): zeroing is on unless FE_ZERO_ALLOC is
+// exactly "0", the canary is on only when FE_CANARY is exactly "1".
+bool env_equals(const char *name, const char *value) {
     const char *e = getenv(name);
-    return e && *e ? atoi(e) != 0 : fallback;
+    return e && strcmp(e, value) == 0;
 }
 bool canary_on() {
-    static const bool on = env_flag("FE_CANARY", false);
+    static const bool on = env_equals("FE_CANARY", "1");
     return on;
 }
 bool zero_alloc() {
-    static const bool on = env_flag("FE_ZERO_ALLOC", true);
+    static const bool on = !env_equals("FE_ZERO_ALLOC", "0");
     return on;
 }
 }  // namespace
+
+int fe_hip_zero_alloc_on(void) { return zero_alloc() ? 1 : 0; }
 
 int fe_hip_malloc(fe_devptr_t *out, size_t bytes) {
     void *p = nullptr;
     const size_t n = bytes ? bytes : 1;
     HIPCHK(hipMalloc(&p, n + (canary_on() ? kCanaryPad : 0)));
-    if (zero_alloc()) HIPCHK(hipMemsetD8Async((hipDeviceptr_t)p, 0, n, nullptr));
+    // (a failure from here on gives the block back before it is reported)
+    hipError_t e = hipSuccess;
+    if (zero_alloc()) e = hipMemsetD8Async((hipDeviceptr_t)p, 0, n, nullptr);
+    if (e == hipSuccess && canary_on()) e = hipMemsetD8Async((hipDeviceptr_t)((char *)p + bytes), 0xA5, kCanaryPad, nullptr);
+    if (e == hipSuccess && (zero_alloc() || canary_on())) e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess) {
+        (void)hipFree(p);
+        return fe_check_hip((int)e, "fe_hip_malloc: clearing the new block");
+    }
     if (canary_on()) {
-        HIPCHK(hipMemsetD8Async((hipDeviceptr_t)((char *)p + bytes), 0xA5, kCanaryPad, nullptr));
         std::lock_guard<std::mutex> g(g_canary_lock);
         g_canary_live.emplace_back((fe_devptr_t)p, bytes);
     }
-    if (zero_alloc() || canary_on()) HIPCHK(hipStreamSynchronize(nullptr));
     *out = (fe_devptr_t)p;
     return 0;
 }

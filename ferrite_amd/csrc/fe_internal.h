@@ -48,6 +48,7 @@ struct FeBuf {
     }
     int zeroed(size_t n) {
         FE_TRY(alloc(n));
+        if (fe_hip_zero_alloc_on()) return 0;  // fe_hip_malloc has cleared the block and synchronized
         FE_TRY(fe_hip_memset_d8(p, 0, n, nullptr));
         return fe_hip_synchronize();
     }

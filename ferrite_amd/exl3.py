@@ -285,6 +285,24 @@ class Linear:
         then run the GEMM over them without decoding."""
         check(_lib.lib().fe_exl3_linear_keep_decoded(self.h, _stream(stream), int(on)))
 
+    def decoded_w_hat(self):
+        """The kept tiles un-swizzled: W_hat as fp16 bits [k][n] (host uint16 array), exactly the values the decoder of
+        the hot loops produced (keep_decoded() first)."""
+        ptr, nbytes = C.c_uint64(), C.c_size_t()
+        check(_lib.lib().fe_exl3_linear_decoded(self.h, C.byref(ptr), C.byref(nbytes)))
+        if not ptr.value:
+            raise FeError(-1, "no decoded tiles: call keep_decoded() first")
+        raw = np.empty(nbytes.value // 2, np.uint16)
+        check(_lib.lib().fe_hip_synchronize())
+        check(_lib.lib().fe_hip_memcpy_dtoh(raw.ctypes.data_as(C.c_void_p), ptr.value, nbytes.value))
+        ktiles, tiles_n = self.k // 64, (self.n // 128 + 1) // 2
+        blocks = raw.reshape(tiles_n, ktiles, 256, 8, 8)  # [tn][kt][column r][position][8 values]
+        r = np.arange(256)[:, None]
+        pos = np.arange(8)[None, :] ^ (r & 7) ^ ((r >> 3) & 1)  # where chunk c of column r lies
+        chunks = np.take_along_axis(blocks, np.broadcast_to(pos[None, None, :, :, None], blocks.shape), axis=3)  # [tn][kt][r][c][8]
+        w = chunks.reshape(tiles_n, ktiles, 256, 64).transpose(1, 3, 0, 2).reshape(self.k, tiles_n * 256)
+        return np.ascontiguousarray(w[:, :self.n])
+
     def forward_is_one_launch(self, rows: int) -> bool:
         """Whether forward() with this many rows is the decode GEMV alone, rotating its own input."""
         return bool(_lib.lib().fe_exl3_linear_forward_is_one_launch(self.h, rows))

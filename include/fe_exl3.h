@@ -99,6 +99,11 @@ int fe_exl3_linear_forward(const fe_exl3_linear *l, const fe_exl3_kernels *kern,
  * (reconstruct_bf16 into Linear.w, crates/fe-model/src/model.rs:262-266), for callers that have the memory: 178 MB for
  * 5120 x 17408. on == 0 frees them. Stream-ordered; the first GEMM may follow on the same stream. */
 int fe_exl3_linear_keep_decoded(fe_exl3_linear *l, fe_stream_t s, int on);
+/* The kept tiles (null / 0 when there are none), for checks of the decoder that runs in the hot loops against
+ * decode_tile (crates/fe-exl3/src/cpu.rs:57-69): fp16 W_hat, block (tn, kt) of 32 KB at ((tn * (k / 64)) + kt) * 32768 =
+ * columns 256 tn .. + 255 of channels 64 kt .. + 63, 128 bytes a column r, the 16-byte chunk c (channels 8 c .. 8 c + 7)
+ * of column r at byte r * 128 + 16 * (c ^ (r & 7) ^ ((r >> 3) & 1)). */
+int fe_exl3_linear_decoded(const fe_exl3_linear *l, fe_devptr_t *tiles, size_t *bytes);
 /* 1 if forward() with this many rows is a single launch (the decode GEMV rotates its own input: every program's K range
  * is whole 128-element Hadamard blocks), 0 if it is rotate_input followed by gemv_rotated. Same bits either way. */
 int fe_exl3_linear_forward_is_one_launch(const fe_exl3_linear *l, uint32_t rows);
@@ -153,9 +158,11 @@ int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error);
  * rotated inputs, split partial sums and arrival counters live in one static device array of FE_EXL3_STATIC_BYTES that
  * every GPU the library runs on holds until the process ends; the call allocates and frees nothing. Same kernels and
  * the same bits as fe_exl3_linear_forward. Limits: 1..FE_EXL3_STATIC_ROWS rows, rows * k * 2 <= 1 MiB of rotated inputs,
- * (programs + n / 128) * rows * 512 bytes of partial sums (programs: about 4 per CU) <= FE_EXL3_STATIC_BYTES - 1 MiB - 16 KiB, n <= 524288; anything larger is
- * FE_ERR_WORKSPACE. All calls on one GPU share the array: calls that overlap on one GPU (two streams) race; order them. */
-#define FE_EXL3_STATIC_BYTES (12u << 20)
+ * (programs + n / 128) * rows * 512 bytes of partial sums <= FE_EXL3_STATIC_BYTES - 1 MiB - 16 KiB, n <= 524288; anything
+ * larger is FE_ERR_WORKSPACE. `programs` follows the linear's plan (occ programs a CU, 1..5): the array is sized for the
+ * widest tuned shape, 5120 x 17408, at 16 rows under occ 5 (1280 programs on 256 CUs: 11.06 MiB of partial sums). All
+ * calls on one GPU share the array: calls that overlap on one GPU (two streams) race; order them. */
+#define FE_EXL3_STATIC_BYTES (13u << 20)
 #define FE_EXL3_STATIC_ROWS 16
 int fe_exl3_linear_forward_static(const fe_exl3_linear *l, const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x,
                                   int x_dtype, fe_devptr_t y, int y_dtype, uint32_t rows);

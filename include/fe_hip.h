@@ -49,6 +49,7 @@ typedef struct fe_canary_tail {
     size_t bytes, first, damaged;
 } fe_canary_tail;
 int fe_hip_canary_on(void);
+int fe_hip_zero_alloc_on(void); /* 1 unless FE_ZERO_ALLOC is exactly "0" (the canary: on only for FE_CANARY exactly "1") */
 int fe_hip_canary_tails(fe_canary_tail *out, size_t cap, size_t *count);
 int fe_hip_memset_d8(fe_devptr_t p, uint8_t v, size_t n, fe_stream_t s);
 int fe_hip_memset_d32(fe_devptr_t p, uint32_t v, size_t n, fe_stream_t s);

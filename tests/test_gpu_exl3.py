@@ -44,6 +44,25 @@ def test_reconstruct_hat_is_bit_exact(env, oracle, bits):
     assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} values differ"
 
 
+@pytest.mark.parametrize("bits", [2, 3, 4, 5, 6, 8])
+@pytest.mark.parametrize("strips", [True, False])
+def test_hot_loop_decoder_is_bit_exact(env, oracle, bits, strips):
+    """The decoder of the hot loops (decode_lane: boundary windows, one extract per state; the GEMV, the decoding GEMM
+    and exl3_hat_tiles_b* all run it) bit for bit against decode_tile (crates/fe-exl3/src/cpu.rs:57-69): the tiles that
+    exl3_hat_tiles_b* leaves with the linear are exactly decode_lane's fp16 values, read back and un-swizzled. An odd
+    count of column blocks (the last 256-column tile half empty) and both trellis layouts."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    t = synth.exl3_tensor(384, 384, bits, 300 + bits)
+    d = exl3.DeviceExl3.upload_strips(t) if strips else exl3.DeviceExl3.upload(t)
+    lin = exl3.Linear.new(kern, d, 64)
+    lin.keep_decoded()
+    got = lin.decoded_w_hat()
+    want = oracle.w_hat_f16(to_oracle(oracle, t))
+    assert got.shape == want.shape
+    assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} values differ"
+
+
 def test_reconstruct_bf16_within_one_ulp(env, oracle):
     """crates/fe-exl3/src/bin/exl3-gpucheck.rs:58-98: GPU f32 math vs the f64 reference: at most 1 bf16 ulp apart, more
     only as f32 cancellation noise near zero (absolute error below 1e-4 of the tensor's rms); [n][k] is the exact

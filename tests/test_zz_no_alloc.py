@@ -1,6 +1,9 @@
 """The entry point that allocates nothing (fe_exl3_linear_forward_static): its output has the bits of
-fe_exl3_linear_forward over a workspace object, call after call on the shared static scratch array, and shapes beyond
-the array are refused with an error."""
+fe_exl3_linear_forward over a workspace object, call after call on the shared static scratch array; the free device
+memory does not move across its calls; it records into a HIP graph and replays; and shapes beyond the array are refused
+with an error."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -56,6 +59,63 @@ def test_the_benchmark_shape_at_one_and_sixteen_rows():
     for rows in (16, 1):
         _, got, want = both(torch, exl3, synth, kern, 5120, 17408, 4, rows, 13, exl3.Dtype.Bf16)
         same_bits(torch, got, want, rows)
+
+
+def test_no_device_memory_moves_and_the_widest_plan_fits():
+    """Free device memory (hipMemGetInfo) reads the same before and after a run of calls; 5120 x 17408 at 16 rows under a
+    plan of 5 programs a CU (1280 programs: the most room a tuned shape asks of the array) is served."""
+    import torch
+    from ferrite_amd import exl3, synth
+    kern = exl3.Kernels.load()
+    t = synth.exl3_tensor(5120, 17408, 4, 13)
+    w = exl3.DeviceExl3.upload_strips(t)
+    lin5 = exl3.Linear.with_plan(kern, w, exl3.Plan(10, 4, 3, 5))
+    lin = exl3.Linear.new(kern, w, exl3.default_blocks(exl3.cu_count()))
+    x = dev_u16(torch, synth.activations(16, 5120, 3))
+    want = torch.zeros((16, 17408), dtype=torch.bfloat16, device="cuda")
+    got = torch.zeros((16, 17408), dtype=torch.bfloat16, device="cuda")
+    ws = exl3.Workspace([lin5], 16)
+    lin5.forward(x, exl3.Dtype.Bf16, want, exl3.Dtype.Bf16, 16, ws)
+    lin5.forward_static(x, exl3.Dtype.Bf16, got, exl3.Dtype.Bf16, 16)  # (first call: any lazy set-up is behind us)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    free0 = torch.cuda.mem_get_info()[0]
+    for rows in (1, 16, 3, 16, 1):
+        lin5.forward_static(x, exl3.Dtype.Bf16, got, exl3.Dtype.Bf16, rows)
+        lin.forward_static(x, exl3.Dtype.Bf16, got, exl3.Dtype.Bf16, rows)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "a forward_static call changed the free device memory"
+
+
+def test_records_into_a_graph_and_replays():
+    import torch
+    from ferrite_amd import _lib, exl3, synth
+    lib, check = _lib.lib(), _lib.check
+    kern = exl3.Kernels.load()
+    t = synth.exl3_tensor(2048, 1024, 4, 21)
+    lin = exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(4))  # split K: counters and partial sums in use
+    x = dev_u16(torch, synth.activations(5, 2048, 22))
+    ws = exl3.Workspace([lin], 5)
+    want = torch.zeros((5, 1024), dtype=torch.float32, device="cuda")
+    lin.forward(x, exl3.Dtype.Bf16, want, exl3.Dtype.F32, 5, ws)
+    got = torch.zeros((5, 1024), dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    s, g = C.c_void_p(), C.c_void_p()
+    check(lib.fe_hip_stream_create(C.byref(s)))
+    check(lib.fe_hip_graph_begin(s))
+    lin.forward_static(x, exl3.Dtype.Bf16, got, exl3.Dtype.F32, 5, stream=s)
+    check(lib.fe_hip_graph_end(s, C.byref(g)))
+    for rep in range(3):
+        got.fill_(9.0)
+        torch.cuda.synchronize()
+        check(lib.fe_hip_graph_launch(g, s))
+        check(lib.fe_hip_stream_sync(s))
+        assert torch.equal(got.view(torch.int32), want.view(torch.int32)), rep
+        # an eager call on the same array between the replays
+        lin.forward_static(x, exl3.Dtype.Bf16, got, exl3.Dtype.F32, 2)
+        torch.cuda.synchronize()
+    check(lib.fe_hip_graph_destroy(g))
+    check(lib.fe_hip_stream_destroy(s))
 
 
 def test_sizes_beyond_the_array_are_errors():
