@@ -742,6 +742,21 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
         timed.after_idle = first
         return ev.loop_us(stream, fn, n_warm, ramp_ms=0) / 1e3
 
+    # What the matrix units sustain on this board with nothing else running: the register-only probe (4 x 4 independent
+    # v_mfma_f32_32x32x16_f16 per wavefront, one wavefront a SIMD as in the GEMM core) after the same 0.15 s of launches, with
+    # operands of 0.5 and 1 (the published peak's conditions: hardly a bit toggles), with random signs and mantissas (what
+    # rotated activations and 11-bit codebook values feed the unit) and with five random mantissa bits (the six
+    # significant bits of an NVFP4 operand). The clock is what rocm-smi reports during the sustained window.
+    from ferrite_amd import probes
+    fk = fp4.Kernels.load()
+    peak = {}
+    for label, kind, seed in (("f16_constant_operands", "f16", 0), ("f16_random_operands", "f16", 12345),
+                              ("f16_five_mantissa_bits", "f16", 12346), ("f8_random_operands", "f8", 12345)):
+        p = probes.mfma_peak(fk, kind, exl3.cu_count(), seed=seed)
+        peak[label] = {"TFLOP/s": p["sustained_TFLOPs"], "burst_TFLOP/s": p["burst_TFLOPs"], "sclk_MHz": p.get("sclk_MHz_median")}
+    res["mfma_sustained"] = peak
+    sus16, sus16_5, sus8 = peak["f16_random_operands"]["TFLOP/s"], peak["f16_five_mantissa_bits"]["TFLOP/s"], peak["f8_random_operands"]["TFLOP/s"]
+
     # EXL3
     t = synth.exl3_tensor(k, n, 4, SEED, "gate")
     lin = exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), 1024)
@@ -774,7 +789,6 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
                                          "what": "torch.matmul (hipBLASLt), f16 x f16^T, random normal operands"}
     del a16, w16, y16
     # NVFP4
-    fk = fp4.Kernels.load()
     flin = synth.fp4_linear(n, k, SEED, input_scale=1.0).upload()
     fws = fp4.Workspace(m, k)
     xf = torch.from_numpy(synth.activations(m, k, SEED).view(np.int16)).cuda()
@@ -867,6 +881,11 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
         us = ev.loop_us(stream, gv, 30)
         res[f"bf16_5120x17408_m{rows}"] = {"gemv_us": round(us, 2), "GB/s": round(2.0 * n * k / us / 1e3, 1),
                                           "frac_hbm_peak": round(2.0 * n * k / us / 1e3 / HBM_PEAK_GBS, 4)}
+    # every GEMM against what the matrix units sustain alone on operands that toggle like its own
+    for name, e in res.items():
+        if isinstance(e, dict) and "TFLOP/s" in e and name != "mfma_sustained":
+            ceiling = sus8 if name.startswith("fp8") else sus16_5 if name.startswith("nvfp4") else sus16
+            e["frac_of_mfma_sustained"] = round(e["TFLOP/s"] / ceiling, 4)
     return res
 
 

@@ -99,6 +99,7 @@ SYMBOLS = {
     "fe_exl3_reconstruct_bf16": (I, [P, P, C.POINTER(View), U64, I, U64, SZ]),
     "fe_exl3_probe_stream_read": (I, [P, P, U64, SZ, U32, U32, C.POINTER(F)]),
     "fe_exl3_probe_decode": (I, [P, P, U32, U32, U32, U32, C.POINTER(F)]),
+    "fe_exl3_probe_op": (I, [P, P, C.c_char_p, U32, U32, U32, C.POINTER(F)]),
     # fe_fp4.h
     "fe_fp4_kernels_load": (I, [PP]),
     "fe_fp4_kernels_destroy": (I, [P]),
@@ -118,6 +119,7 @@ SYMBOLS = {
     "fe_fp4_linear_quantize": (I, [P, P, P, P, U64, U32, U32]),
     "fe_fp4_linear_gemm": (I, [P, P, P, P, U64, U32, U32, U64]),
     "fe_fp4_linear_forward_swiglu": (I, [P, P, P, P, P, U64, U32, U32, F]),
+    "fe_fp4_mfma_peak": (I, [P, P, I, U32, U32, U32, U32, C.POINTER(F)]),
     # fe_route.h
     "fe_route_ctx_create": (I, [PP, P, P, P, P, P, U32]),
     "fe_route_ctx_destroy": (I, [P]),

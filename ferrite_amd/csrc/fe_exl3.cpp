@@ -971,6 +971,30 @@ int fe_exl3_probe_stream_read(const fe_exl3_kernels *kern, fe_stream_t s, fe_dev
                          &ctx);
 }
 
+int fe_exl3_probe_op(const fe_exl3_kernels *kern, fe_stream_t s, const char *op, uint32_t grid, uint32_t iters,
+                     uint32_t launches, float *ms) {
+    if (!kern || !op || !grid || !launches || strlen(op) > 32) return fe_set_error(FE_ERR_ARG, "fe_exl3_probe_op", "bad argument");
+    char nm[64];
+    snprintf(nm, sizeof nm, "exl3_probe_op_%s", op);
+    struct Ctx {
+        fe_function_t f;
+        fe_stream_t s;
+        fe_devptr_t out;
+        uint32_t grid, iters, seed;
+    } ctx{nullptr, s, 0, grid, iters, 7u};
+    FE_TRY(fe_hip_module_get_function(&ctx.f, kern->module, nm));
+    FeBuf out;
+    FE_TRY(out.zeroed(64));
+    ctx.out = out.p;
+    return time_launches(s, launches, ms,
+                         [](void *p) {
+                             Ctx *c = (Ctx *)p;
+                             void *args[] = {&c->out, &c->iters, &c->seed};
+                             return fe_hip_launch(c->f, c->grid, 1, 1, 256, 1, 1, 0, c->s, args);
+                         },
+                         &ctx);
+}
+
 int fe_exl3_probe_decode(const fe_exl3_kernels *kern, fe_stream_t s, uint32_t bits, uint32_t grid, uint32_t iters,
                          uint32_t launches, float *ms) {
     if (!kern || bits < 3 || bits > 5 || !grid || !launches) return fe_set_error(FE_ERR_ARG, "fe_exl3_probe_decode", "bits 3..5");

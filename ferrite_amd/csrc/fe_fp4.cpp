@@ -422,3 +422,31 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
 }
 
 }  // extern "C"
+
+// Matrix-unit peak (fe_mfma_peak_*): `launches` launches of grid x 256 threads between two events, after one warm-up.
+extern "C" int fe_fp4_mfma_peak(const fe_fp4_kernels *kern, fe_stream_t s, int kind, uint32_t seed, uint32_t grid, uint32_t iters,
+                                uint32_t launches, float *ms) {
+    const char *fn = "fe_fp4_mfma_peak";
+    if (!kern || kind < 0 || kind > 2 || !grid || !launches) return fe_set_error(FE_ERR_ARG, fn, "kind 0 (f16), 1 (bf16), 2 (f8)");
+    static const char *names[] = {"fe_mfma_peak_f16", "fe_mfma_peak_bf16", "fe_mfma_peak_f8"};
+    fe_function_t f = nullptr;
+    FE_TRY(fe_hip_module_get_function(&f, kern->module, names[kind]));
+    FeBuf out;
+    FE_TRY(out.alloc((size_t)grid * 256 * 4));
+    fe_devptr_t o = out.p;
+    void *args[] = {&o, &iters, &seed};
+    fe_event_t a = nullptr, b = nullptr;
+    FE_TRY(fe_hip_event_create(&a));
+    int c = fe_hip_event_create(&b);
+    if (!c) c = fe_hip_launch(f, grid, 1, 1, 256, 1, 1, 0, s, args);
+    if (!c) c = fe_hip_event_record(a, s);
+    for (uint32_t i = 0; !c && i < launches; i++) c = fe_hip_launch(f, grid, 1, 1, 256, 1, 1, 0, s, args);
+    if (!c) c = fe_hip_event_record(b, s);
+    if (!c) c = fe_hip_event_sync(b);
+    float t = 0;
+    if (!c) c = fe_hip_event_elapsed_ms(&t, a, b);
+    fe_hip_event_destroy(a);
+    fe_hip_event_destroy(b);
+    if (!c && ms) *ms = t / (float)launches;
+    return c;
+}

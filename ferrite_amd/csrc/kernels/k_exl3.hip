@@ -1270,3 +1270,31 @@ extern "C" __global__ __launch_bounds__(256, 4) void exl3_probe_decode_b4(uint32
 extern "C" __global__ __launch_bounds__(256, 4) void exl3_probe_decode_b5(uint32_t* out, uint32_t iters, uint32_t seed) {
     probe_decode_body<5>(out, iters, seed);
 }
+
+// Instruction throughput probes: 8 independent chains of `iters` dependent instructions a lane, no memory traffic
+// (kernels/k-exl3/src/probe.rs:38-67 measures its decode's instructions the same way). The instructions are the ones the
+// trellis decode is made of, plus an add and an and as the plain 32-bit yardsticks; the issue rate of an instruction is
+// lanes x 8 x iters over the launch time.
+#define OP_PROBE(NAME, ASM)                                                                                            \
+    extern "C" __global__ __launch_bounds__(256) void exl3_probe_op_##NAME(uint32_t* out, uint32_t iters, uint32_t seed) { \
+        uint32_t x[8];                                                                                                 \
+        _Pragma("unroll") for (int j = 0; j < 8; j++) x[j] = (seed + j) ^ (threadIdx.x * 0x9e3779b9u);                 \
+        const uint32_t c = 0x83DCD12Du;                                                                                \
+        for (uint32_t i = 0; i < iters; i++) {                                                                         \
+            _Pragma("unroll") for (int j = 0; j < 8; j++) asm volatile(ASM : "+v"(x[j]) : "v"(c));                     \
+        }                                                                                                              \
+        const uint32_t r = x[0] ^ x[1] ^ x[2] ^ x[3] ^ x[4] ^ x[5] ^ x[6] ^ x[7];                                      \
+        if (r == 0x12345678u) *out = r;                                                                                \
+    }
+OP_PROBE(add, "v_add_u32 %0, %0, %1")
+OP_PROBE(and, "v_and_b32 %0, %0, %1")
+OP_PROBE(mul_lo, "v_mul_lo_u32 %0, %0, %1")
+OP_PROBE(mad_u24, "v_mad_u32_u24 %0, %0, %1, %1")
+OP_PROBE(bfe, "v_bfe_u32 %0, %0, 5, 16")
+OP_PROBE(alignbit, "v_alignbit_b32 %0, %0, %1, 16")
+OP_PROBE(perm, "v_perm_b32 %0, %0, %1, %1")
+OP_PROBE(sad_u8, "v_sad_u8 %0, %0, 0, %1")
+OP_PROBE(sad_hi_u8, "v_sad_hi_u8 %0, %0, 0, %1")
+OP_PROBE(pk_fma_f16, "v_pk_fma_f16 %0, %0, %1, %1")
+OP_PROBE(fma_f32, "v_fma_f32 %0, %0, %1, %1")
+OP_PROBE(dpp_mov, "v_mov_b32_dpp %0, %0 row_shr:1 row_mask:0xf bank_mask:0xf")

@@ -791,3 +791,77 @@ __device__ __forceinline__ void gemv_nvfp4_body(uint16_t* c, const _Float16* aq,
 FP4_GEMV_KERNEL(1)
 FP4_GEMV_KERNEL(2)
 FP4_GEMV_KERNEL(3)  // (four groups of rows would not fit the registers of two programs a CU)
+
+// ---- matrix-unit peak probe ---------------------------------------------------------------------------------------------
+//
+// Every wavefront issues iters x 16 independent matrix instructions (the GEMM core's 4 x 4 accumulator pieces, 256
+// accumulator registers) on operands that stay in registers: no memory traffic, no LDS (kernels/k-fp4/src/lib.rs:866-916,
+// fe_fp4_peak). KIND 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_32x32x16_bf16, 2: v_mfma_f32_32x32x64_f8f6f4 on e4m3
+// codes (the unscaled form). seed == 0: every operand element is 0.5 or 1 (few bits toggle from one instruction to the
+// next, the reference's kind of pattern); otherwise signs and mantissas are random bits of the seed (an even seed:
+// only the top five mantissa bits of the 16-bit kinds), magnitudes in [0.5, 2), as the operands of a GEMM on real data toggle: the clock the board holds under its power limit depends on
+// it. One float a lane is written so that nothing is dead code. Flops of a launch: wavefronts x iters x 16 x 2 x 32 x 32 x
+// (16 or 64).
+template <int KIND>
+__device__ __forceinline__ void mfma_peak_body(float* out, uint32_t iters, uint32_t seed) {
+    const uint32_t lane = threadIdx.x & 63;
+    f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
+    uint32_t rs = seed * 0x9e3779b9u + (blockIdx.x * 256 + threadIdx.x) * 0x85ebca6bu;
+    auto rnd = [&]() {
+        rs ^= rs << 13, rs ^= rs >> 17, rs ^= rs << 5;
+        return seed ? rs : 0u;
+    };
+    // 16-bit pairs: sign and mantissa from the random word, exponent of 0.5 or 1; e4m3 quadruples likewise
+    // (an even seed keeps only the top five mantissa bits of the 16-bit kinds: the six significant bits of an NVFP4 operand)
+    const uint32_t keep16 = seed & 1 ? (KIND == 1 ? 0x80ff80ffu : 0x87ff87ffu) : (KIND == 1 ? 0x80fc80fcu : 0x87e087e0u);
+    const uint32_t base16 = KIND == 1 ? 0x3f003f00u : 0x38003800u;
+    auto h = [&](uint32_t flip) { return ((rnd() & keep16) | base16) ^ flip; };
+    auto c = [&](uint32_t flip) { return (int)(((rnd() & 0x8f8f8f8fu) | 0x30303030u) ^ flip); };
+    u32x4 a16[4], b16[4];
+    gm_i32x8 a8[4], b8[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a16[i] = (u32x4){h(0), h((lane & 1) << 15), h(0), h((uint32_t)i << 31)};
+        b16[i] = (u32x4){h((lane & 2) << 14), h(0), h((uint32_t)i << 15), h(0)};
+        a8[i] = (gm_i32x8){c(0), c((lane & 1) << 7), c((uint32_t)i << 31), c(0), c(0), c(0), c(0), c(0)};
+        b8[i] = (gm_i32x8){c(0), c((lane & 2) << 6), c(0), c(0), c(0), c((uint32_t)i << 15), c(0), c(0)};
+    }
+    for (uint32_t it = 0; it < iters; it++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (KIND == 0)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a16[i]), __builtin_bit_cast(f16x8, b16[j]),
+                                                                      acc[i][j], 0, 0, 0);
+                else if constexpr (KIND == 1)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a16[i]), __builtin_bit_cast(bf16x8, b16[j]),
+                                                                       acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[i], b8[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+            }
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) sum += acc[i][j][e];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = sum;
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_mfma_peak_f16(float* out, uint32_t iters, uint32_t seed) {
+    mfma_peak_body<0>(out, iters, seed);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_mfma_peak_bf16(float* out, uint32_t iters, uint32_t seed) {
+    mfma_peak_body<1>(out, iters, seed);
+}
+extern "C" __global__ __launch_bounds__(256, 1) void fe_mfma_peak_f8(float* out, uint32_t iters, uint32_t seed) {
+    mfma_peak_body<2>(out, iters, seed);
+}

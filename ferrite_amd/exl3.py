@@ -212,6 +212,14 @@ class Kernels:
                                                    launches, C.byref(ms)))
         return ms.value
 
+    PROBE_OPS = ("add", "and", "mul_lo", "mad_u24", "bfe", "alignbit", "perm", "sad_u8", "sad_hi_u8", "pk_fma_f16", "fma_f32", "dpp_mov")
+
+    def probe_op(self, op, grid, iters, launches, stream=None):
+        """Milliseconds per launch of grid x 256 lanes x 8 chains x iters dependent instructions `op` (PROBE_OPS)."""
+        ms = C.c_float()
+        check(_lib.lib().fe_exl3_probe_op(self.h, _stream(stream), op.encode(), grid, iters, launches, C.byref(ms)))
+        return ms.value
+
     def probe_decode(self, bits, grid, iters, launches, stream=None):
         ms = C.c_float()
         check(_lib.lib().fe_exl3_probe_decode(self.h, _stream(stream), bits, grid, iters, launches, C.byref(ms)))

@@ -135,6 +135,19 @@ class Kernels:
         """A switch of the launch paths, by name (the header lists them)."""
         check(_lib.lib().fe_fp4_kernels_set_option(self.h, name.encode(), int(value)))
 
+    MFMA_KINDS = {"f16": (0, 16), "bf16": (1, 16), "f8": (2, 64)}  # kind, k of the instruction (32 x 32 x k)
+
+    def mfma_peak(self, kind: str, grid: int, iters: int, launches: int, seed: int = 0, stream=None):
+        """(milliseconds per launch, TFLOP/s) of the register-only matrix-unit probe (fp4-peak.rs:11-31): grid x 4 wavefronts
+        x iters x 16 independent v_mfma_f32_32x32x{16,64} of the given operand kind; seed 0: operands of 0.5 and 1, else
+        random signs and mantissas."""
+        from .exl3 import _stream
+        code, k = self.MFMA_KINDS[kind]
+        ms = C.c_float()
+        check(_lib.lib().fe_fp4_mfma_peak(self.h, _stream(stream), code, seed, grid, iters, launches, C.byref(ms)))
+        flops = grid * 4 * iters * 16 * 2.0 * 32 * 32 * k
+        return ms.value, flops / (ms.value * 1e-3) / 1e12
+
     def __del__(self):
         if getattr(self, "h", None) and _lib is not None and _lib._lib is not None:
             _lib._lib.fe_fp4_kernels_destroy(self.h)

@@ -186,6 +186,12 @@ int fe_exl3_probe_stream_read(const fe_exl3_kernels *kern, fe_stream_t s, fe_dev
                               uint32_t launches, float *ms);
 int fe_exl3_probe_decode(const fe_exl3_kernels *kern, fe_stream_t s, uint32_t bits, uint32_t grid, uint32_t iters,
                          uint32_t launches, float *ms);
+/* Issue rate of one vector instruction of the decode (kernels/k-exl3/src/probe.rs:38-67, exl3_probe_{imad,idp,lop,...}):
+ * grid x 256 lanes run 8 independent chains of `iters` dependent instructions each; op is one of "add", "and",
+ * "mul_lo" (v_mul_lo_u32), "mad_u24", "bfe", "alignbit", "perm", "sad_u8", "sad_hi_u8", "pk_fma_f16", "fma_f32",
+ * "dpp_mov". Lane-operations per second = grid * 256 * 8 * iters / (ms * 1e-3). */
+int fe_exl3_probe_op(const fe_exl3_kernels *kern, fe_stream_t s, const char *op, uint32_t grid, uint32_t iters,
+                     uint32_t launches, float *ms);
 
 #ifdef __cplusplus
 }

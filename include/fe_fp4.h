@@ -86,6 +86,15 @@ int fe_fp4_linear_forward_swiglu(const fe_fp4_linear *l, const fe_fp4_kernels *k
                                  const fe_fp4_workspace *ws, const fe_fp4_workspace *act, fe_devptr_t x, uint32_t lda,
                                  uint32_t m, float down_g);
 
+/* Matrix-unit peak probe (fe_fp4_peak, kernels/k-fp4/src/lib.rs:866-916, driven by crates/fe-fp4/src/bin/fp4-peak.rs):
+ * grid x 4 wavefronts issue iters x 16 independent matrix instructions each on register operands, no memory traffic.
+ * kind 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_f32_32x32x16_bf16, 2: v_mfma_f32_32x32x64_f8f6f4 (e4m3 x e4m3).
+ * seed 0: operands of 0.5 and 1 (few bits toggle, the reference's kind of pattern); otherwise random signs and mantissas, as
+ * a GEMM on real data toggles its operands (the clock held under the board's power limit depends on it).
+ * ms: average milliseconds of `launches` launches; flops of one = grid * 4 * iters * 16 * 2 * 32 * 32 * (kind == 2 ? 64 : 16). */
+int fe_fp4_mfma_peak(const fe_fp4_kernels *kern, fe_stream_t s, int kind, uint32_t seed, uint32_t grid, uint32_t iters,
+                     uint32_t launches, float *ms);
+
 #ifdef __cplusplus
 }
 #endif
