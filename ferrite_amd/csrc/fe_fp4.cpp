@@ -21,6 +21,7 @@ constexpr uint32_t kTileN = 256;                        // GM_BN
 struct fe_fp4_kernels {
     fe_module_t module = nullptr;
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4[3] = {nullptr, nullptr, nullptr};
+    fe_function_t strip4 = nullptr;  // the GEMV over strips of 16 weight rows, up to 16 activation rows (no hand-off)
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
     fe_function_t gemm4_sk = nullptr, gemm8_sk = nullptr, gemm8c_sk = nullptr, swiglu4_sk = nullptr;  // the same on the stream-K schedule
@@ -29,7 +30,9 @@ struct fe_fp4_kernels {
     // afterwards. No forward call reads the environment.
     uint32_t group_m = 8;      // raster group height in row tiles; 0 = all (FE_FP4_GROUP, lib.rs:31-32, 68)
     uint32_t gemv = 1;         // up to 64 rows run the GEMV (FE_FP4_NO_GEMV=1: the GEMM's single tile row)
-    uint32_t gemv_sk = 0;      // K splits of the GEMV; 0 = two programs a CU (FE_FP4_GEMV_SK)
+    uint32_t gemv_sk = 0;      // K splits of the GEMV over weight tiles; 0 = two programs a CU (FE_FP4_GEMV_SK)
+    uint32_t gemv_strips = 1;  // the GEMV runs over strips of 16 weight rows, K split inside the workgroup (FE_FP4_NO_STRIPS=1: over weight tiles and K splits)
+    uint32_t gemv_waves = 0;   // wavefronts of a strip's workgroup: 4, 8 or 16; 0 = four or more wavefronts a SIMD (FE_FP4_GEMV_WAVES)
     int32_t xcd = -1;          // column tiles dealt to the XCDs: -1 = where the weights are the larger operand (FE_FP4_XCD)
     uint32_t fp8_f16 = 0;      // FP8 linears as fp16 expansion on the 16-bit matrix instruction (FE_FP8_F16=1)
     uint32_t gemm_splits = 8;  // most pieces a cut output tile takes (FE_GEMM_SPLITS; 1: never cut)
@@ -69,6 +72,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
         snprintf(nm, sizeof nm, "fe_gemv_nvfp4_x%d", xr);
         c = fe_hip_module_get_function(&k->gemv4[xr - 1], k->module, nm);
     }
+    if (!c) c = fe_hip_module_get_function(&k->strip4, k->module, "fe_gemv_nvfp4_strips");
+    if (!c) c = fe_hip_func_set_max_dyn_lds(k->strip4, 48 * 1024);
     if (!c) c = fe_hip_module_get_function(&k->quant8, k->module, "fe_fp8_quant");
     if (!c) c = fe_hip_module_get_function(&k->gemm8, k->module, "fe_gemm_fp8");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
@@ -90,6 +95,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (const char *g = getenv("FE_FP4_GROUP")) k->group_m = (uint32_t)atoi(g);
     if (const char *e = getenv("FE_FP4_NO_GEMV")) k->gemv = atoi(e) ? 0 : 1;
     if (const char *e = getenv("FE_FP4_GEMV_SK")) k->gemv_sk = (uint32_t)atoi(e);
+    if (const char *e = getenv("FE_FP4_NO_STRIPS")) k->gemv_strips = atoi(e) ? 0 : 1;
+    if (const char *e = getenv("FE_FP4_GEMV_WAVES")) k->gemv_waves = (uint32_t)atoi(e);
     if (const char *e = getenv("FE_FP4_XCD")) k->xcd = atoi(e) ? 1 : 0;
     if (const char *e = getenv("FE_FP8_F16")) k->fp8_f16 = atoi(e) ? 1 : 0;
     if (const char *e = getenv("FE_GEMM_SPLITS")) k->gemm_splits = (uint32_t)atoi(e);
@@ -115,6 +122,8 @@ int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value
     if (nm == "group_m") k->group_m = (uint32_t)value;
     else if (nm == "gemv") k->gemv = value ? 1 : 0;
     else if (nm == "gemv_sk") k->gemv_sk = (uint32_t)value;
+    else if (nm == "gemv_strips") k->gemv_strips = (uint32_t)value;
+    else if (nm == "gemv_waves") k->gemv_waves = (uint32_t)value;
     else if (nm == "xcd") k->xcd = value;
     else if (nm == "fp8_f16") k->fp8_f16 = value ? 1 : 0;
     else if (nm == "gemm_splits") k->gemm_splits = (uint32_t)value;
@@ -325,6 +334,29 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         // decode-sized: the weight-read-bound GEMV, up to 48 rows a pass. Two programs fit a CU: as many programs as run
         // at once, not more (a second round of short programs costs more than idle CUs in the first).
         const uint32_t nts = n / kTile, kts = k / 64;
+        // Strips of 16 weight rows over all of K, one a workgroup, the activations staged in LDS: no hand-off between
+        // programs. Every program stages all m rows of activations, so it pays where that is small beside the weights:
+        // one row, or up to four on narrow linears (measured, cold weights: 5120 x 17408 at 1 row 14.3 against 15.4 us for
+        // the weight tiles with K splits, 5120 x 5120 at 1..4 rows 7.2-7.8 against 9.7-10.0; at k = 17408 the staging
+        // costs more than the hand-off it saves: 17.0 against 15.8). gemv_strips 2 forces it wherever it fits.
+        const bool strips_fit = k % 256 == 0 && (size_t)m * k * 2 <= 48 * 1024 && m <= 16;
+        const bool strips_pay = k <= 8192 && (m == 1 || (n <= 8192 && m <= 4));
+        if (kern->gemv_strips && strips_fit && (strips_pay || kern->gemv_strips == 2)) {
+            const uint32_t strips = n / 16;
+            uint32_t waves = 4;  // wavefronts of a workgroup: two or more a SIMD in all
+            while (waves < 16 && strips * waves < 8 * kern->cus) waves *= 2;
+            if (kern->gemv_waves && kern->gemv_waves <= 16 && !(kern->gemv_waves & (kern->gemv_waves - 1))) waves = kern->gemv_waves;
+            while (waves > 1 && waves > kts / 4) waves /= 2;
+            fe_devptr_t w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
+            uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
+            for (uint32_t r0 = 0; r0 < m; r0 += kGemvRows) {
+                uint32_t rows = m - r0 < kGemvRows ? m - r0 : kGemvRows;
+                fe_devptr_t yy = y + (size_t)r0 * ldy * 2, aq = ws->aq.p + (size_t)r0 * k * 2, rr = res ? res + (size_t)r0 * ldy * 2 : 0;
+                void *args[] = {&yy, &aq, &w, &sw, &alpha, &rr, &rows, &n, &k, &ldy, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr};
+                FE_TRY(fe_hip_launch(kern->strip4, strips, 1, 1, 64 * waves, 1, 1, rows * k * 2, s, args));
+            }
+            return 0;
+        }
         uint32_t sk = 2 * kern->cus / nts;
         if (kern->gemv_sk) sk = kern->gemv_sk;
         if (sk > 16) sk = 16;

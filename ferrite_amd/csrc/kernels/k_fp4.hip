@@ -792,6 +792,110 @@ FP4_GEMV_KERNEL(1)
 FP4_GEMV_KERNEL(2)
 FP4_GEMV_KERNEL(3)  // (four groups of rows would not fit the registers of two programs a CU)
 
+// ---- GEMV over strips of 16 weight rows (1..16 rows): no hand-off between programs ------------------------------------------
+//
+// A program takes one strip of 16 weight rows over all of K; its W wavefronts (blockDim.x / 64: 4, 8 or 16, the host's
+// choice, so that a launch has four or more wavefronts a SIMD) take groups of four k tiles in turn and their sums meet
+// in LDS. Nothing crosses between programs: no partial sums in memory, no arrival counters, no finisher.
+//
+// What bounds a kernel that reads 9/16 byte a weight is the address unit: a vector memory instruction occupies it for
+// 16 clocks whatever it fetches. So a load step of a wavefront is four k tiles at once: lane L = 16 g + r takes row r
+// of k tile kt0 + g whole, 32 bytes of codes as two 16-byte loads and its four scale bytes as one dword (three
+// instructions per 2 KB of codes, where a lane that takes 16 codes of one k tile needs two per 512 bytes); the MFMA's k
+// index is only a summation index, so step s of the group multiplies, in lane group g, the 16 codes of scale block s of
+// k tile kt0 + g with the same 16 activations. The activations (m rows of k fp16: the host takes this kernel only where
+// they fit in 48 KB) are staged in LDS once per program and read from there. A row's bits depend on (k, W) only.
+struct Fp4StripStage {
+    u32x4 c[2];   // the lane's row of k tile kt0 + g: 64 codes
+    uint32_t sc;  // its four scale bytes
+};
+#define FP4_STRIP_WAVES_MAX 16
+
+__device__ __forceinline__ void gemv_nvfp4_strip_body(uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw,
+                                                      const float* alpha, const uint16_t* res, uint32_t m, uint32_t n, uint32_t k,
+                                                      uint32_t ldc, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt,
+                                                      uint32_t s_skt, uint32_t s_sr) {
+    constexpr int XR = 1;  // up to 16 activation rows
+    __shared__ f32x4 red[FP4_STRIP_WAVES_MAX][64];
+    __shared__ u32x2 scale_lut[128];
+    extern __shared__ __attribute__((aligned(16))) unsigned char xs[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6, r = lane & 15, g = lane >> 4;
+    fp4_scale_lut_fill(scale_lut);
+    for (uint32_t i = tid; i < m * (k / 8); i += blockDim.x) ((u32x4*)xs)[i] = ((const u32x4*)aq)[i];
+    const uint32_t strip = blockIdx.x, nt = strip >> 3, rg = strip & 7;  // the strip: 16-row group rg of weight tile nt
+    const uint32_t groups = k / 256;                                      // groups of four k tiles
+    const uint8_t* wp = w + (size_t)nt * w_snt + (size_t)(16 * rg + r) * w_sr + (size_t)g * w_skt;
+    const uint8_t* sp = sw + (size_t)nt * s_snt + (size_t)(16 * rg + r) * s_sr + (size_t)g * s_skt;
+    uint32_t xo[XR];  // byte offset in xs of the lane's activation row at k tile g
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++) xo[xr] = ((16 * xr + r < m ? 16 * xr + r : m - 1) * k + 64 * g) * 2;
+
+    auto load = [&](Fp4StripStage& st, uint32_t gi) {
+        const uint8_t* p = wp + (size_t)gi * 4 * w_skt;
+        st.c[0] = __builtin_nontemporal_load((const u32x4*)p);
+        st.c[1] = __builtin_nontemporal_load((const u32x4*)(p + 16));
+        st.sc = __builtin_nontemporal_load((const uint32_t*)(sp + (size_t)gi * 4 * s_skt));
+    };
+    f32x4 acc[XR];
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++) acc[xr] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const Fp4StripStage& st, uint32_t gi) {
+#pragma unroll
+        for (int blk = 0; blk < 4; blk++) {  // scale block blk of the lane's k tile: codes 16 blk .. 16 blk + 15
+            const Fp4Scale s = fp4_scale_lut(scale_lut, __builtin_amdgcn_ubfe(st.sc, 8 * blk, 8) << 3);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                u32x4 a = fp4x8_to_f16(st.c[blk >> 1][2 * (blk & 1) + j], s);
+#pragma unroll
+                for (int xr = 0; xr < XR; xr++) {
+                    const f16x8 x = *(const f16x8*)(xs + xo[xr] + gi * 512 + 32 * blk + 16 * j);
+                    acc[xr] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), x, acc[xr], 0, 0, 0);
+                }
+            }
+        }
+    };
+    constexpr int NS = 4;  // groups in flight a wavefront (16 k tiles)
+    Fp4StripStage st[NS];
+    uint32_t gi = wave;
+#pragma unroll
+    for (int i = 0; i < NS; i++)
+        if (gi + waves * i < groups) load(st[i], gi + waves * i);
+    __syncthreads();  // scale_lut, xs
+    for (; gi < groups; gi += waves * NS) {
+#pragma unroll
+        for (int i = 0; i < NS; i++) {
+            if (gi + waves * i < groups) compute(st[i], gi + waves * i);
+            __builtin_amdgcn_sched_barrier(0);
+            if (gi + waves * (i + NS) < groups) load(st[i], gi + waves * (i + NS));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // The wavefronts' sums meet in LDS, one group of activation rows at a time; wavefront 0 adds them in wavefront order.
+    // Lane (r, g) holds output row 16 xr + r, columns 16 strip + 4 g .. + 3.
+    const uint32_t col = 16 * strip + 4 * g;
+#pragma unroll
+    for (int xr = 0; xr < XR; xr++) {
+        if (xr) __syncthreads();
+        red[wave][lane] = acc[xr];
+        __syncthreads();
+        const uint32_t row = 16 * xr + r;
+        if (wave == 0 && row < m) {
+            f32x4 sum = red[0][lane];
+            for (uint32_t v = 1; v < waves; v++) sum += red[v][lane];
+            float o[4] = {sum[0], sum[1], sum[2], sum[3]};
+            fp4_store4(c, res, (size_t)row * ldc + col, o, *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE);
+        }
+    }
+}
+
+extern "C" __global__ __launch_bounds__(1024) void fe_gemv_nvfp4_strips(uint16_t* c, const _Float16* aq, const uint8_t* w,
+                                                                        const uint8_t* sw, const float* alpha, const uint16_t* res,
+                                                                        uint32_t m, uint32_t n, uint32_t k, uint32_t ldc, uint32_t w_snt,
+                                                                        uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, uint32_t s_skt,
+                                                                        uint32_t s_sr) {
+    gemv_nvfp4_strip_body(c, aq, w, sw, alpha, res, m, n, k, ldc, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
+}
+
 // ---- matrix-unit peak probe ---------------------------------------------------------------------------------------------
 //
 // Every wavefront issues iters x 16 independent matrix instructions (the GEMM core's 4 x 4 accumulator pieces, 256

@@ -259,6 +259,50 @@ def test_fp4_gemv_agrees_with_the_gemm(env, oracle):
     assert np.array_equal(outs[(64, 0)][48:55], outs[(7, 48)]) and np.array_equal(outs[(64, 0)][48:], outs[(16, 48)])
 
 
+@pytest.mark.parametrize("n,k", [(384, 2048), (128, 256), (1024, 5120)])
+def test_fp4_gemv_over_strips_agrees_with_the_weight_tiles(env, oracle, n, k):
+    """The GEMV over strips of 16 weight rows (a workgroup a strip over all of K, activations staged in LDS, nothing
+    handed between programs; option gemv_strips = 2 takes it wherever it fits, 0 never) against the GEMV over weight tiles
+    and K splits: the same exact products summed in another order; both weight layouts; the residual epilogue; rows past m
+    untouched; repeats bit-equal; and against the f64 reference over the dequantized operands (fp4-check.rs:134-144)."""
+    torch, fp4, kern = env
+    from ferrite_amd import synth
+    host = synth.fp4_linear(n, k, 51, input_scale=1.0)
+    lin = host.upload()
+    view = fp4.PromptLinear.from_view("view", n, k, torch.from_numpy(host.codes).cuda(), torch.from_numpy(host.sf).cuda(),
+                                      torch.from_numpy(host.alpha).cuda(), host.g)
+    wdq = oracle.dequant_fp4(host.codes, host.sf, 1.0)
+    try:
+        for m in (1, 2, 4, 9, 16):
+            if m * k * 2 > 48 * 1024:
+                continue
+            ws = fp4.Workspace(m, k)
+            xb = fp4_check_activations(m, k, lin.g, 60 + m)
+            xd = dev_u16(torch, xb)
+            res = dev_u16(torch, bf16_bits(np.random.default_rng(m).normal(size=(m + 1, n)).astype(np.float32)))
+
+            def run(l, strips, r=None):
+                kern.set_option("gemv_strips", strips)
+                y = torch.full((m + 1, n), -3.0, dtype=torch.bfloat16, device="cuda")
+                l.forward(kern, ws, y, n, xd, k, m, res=r)
+                torch.cuda.synchronize()
+                out = y.view(torch.int16).cpu().numpy().view(np.uint16)
+                assert (out[m:] == bf16_bits(np.float32([-3.0]))[0]).all()
+                return out[:m]
+
+            tiles, strips = run(lin, 0), run(lin, 2)
+            assert np.array_equal(strips, run(lin, 2)) and np.array_equal(strips, run(view, 2))
+            a, b = bf16_to_f32(strips).astype(np.float64), bf16_to_f32(tiles).astype(np.float64)
+            assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all(), m
+            with_res = run(lin, 2, res)
+            assert np.array_equal(with_res, bf16_bits(bf16_to_f32(strips) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m])))
+            codes, sf = oracle.quant_fp4(xb, host.g)
+            ref = oracle.ref_gemm(oracle.dequant_fp4(codes, sf, 1.0), wdq).astype(np.float64) * host.alpha.astype(np.float64)[None, :]
+            assert (np.abs(a - ref) / np.abs(ref).max(axis=1, keepdims=True)).max() < 8e-3, m
+    finally:
+        kern.set_option("gemv_strips", 1)
+
+
 def test_quantizer_on_special_values(env, oracle):
     """Ties between codes, the saturation boundary, signed zeros, infinities and NaN (a NaN element has magnitude 0 and
     keeps its sign, format.rs:28-41, 66-69; it does not enter the block maximum, format.rs:76): codes and scales as the
