@@ -51,6 +51,7 @@ struct fe_exl3_options {
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
     uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
+    uint32_t handoff_fenced = 0;   // 1..16 rows through the kernels whose hand-off uses release / acquire fences (a slow cross-check)
     uint32_t mlp_chain = 1;        // the decode MLP (gate, up, down) as one launch where it applies (FE_EXL3_NO_CHAIN=1: off)
     uint32_t chain_perm = 1;       // the down stage's workgroups in the order in which their inputs get ready (FE_EXL3_CHAIN_PERM)
     uint32_t chain_spin = 1u << 16;  // polls a program of the down stage waits for the front stage's outputs (FE_EXL3_CHAIN_SPIN)
@@ -62,6 +63,7 @@ struct fe_exl3_kernels {
     fe_function_t rot_in = nullptr, rot_in_group = nullptr, probe_v4 = nullptr;
     fe_function_t probe_decode[3] = {nullptr, nullptr, nullptr};  // 3, 4, 5 bits
     fe_function_t gemvb[6][4] = {};                               // the decode GEMV, [bits slot][row groups - 1]
+    fe_function_t gemvb_fenced[6] = {};                           // the same for 1..16 rows with the fenced hand-off
     fe_function_t mlp[6] = {};                                    // the decode MLP in one launch, [bits slot]
     uint32_t cus = 0;
     fe_function_t gemm[6] = {}, gemm_sk[6] = {};  // decode inside the GEMM: one piece a program / stream-K
@@ -142,6 +144,9 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
             get(&k->gemvb[i][rg - 1], nm);
             if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemvb[i][rg - 1], 84 * 1024);
         }
+        snprintf(nm, sizeof nm, "exl3_gemvb_b%d_r1_fenced", kBits[i]);
+        get(&k->gemvb_fenced[i], nm);
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemvb_fenced[i], 84 * 1024);
         snprintf(nm, sizeof nm, "exl3_mlp_b%d", kBits[i]);
         get(&k->mlp[i], nm);
         if (!c) c = fe_hip_func_set_max_dyn_lds(k->mlp[i], 84 * 1024);
@@ -206,6 +211,7 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     else if (nm == "gemm_splits") o.gemm_splits = value;
     else if (nm == "gemm_sk") o.gemm_sk = value;
     else if (nm == "mlp_chain") o.mlp_chain = value;
+    else if (nm == "handoff_fenced") o.handoff_fenced = value;
     else if (nm == "chain_spin") o.chain_spin = value;
     else if (nm == "chain_perm") o.chain_perm = value;
     else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
@@ -581,7 +587,9 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     uint32_t k = ls[0]->k, mode = (uint32_t)y_dtype, x_mode = in.mode, ldx = in.ld, inv_spb = 0xffffffffu / (k / 64);
     fe_devptr_t x = in.x, x2 = in.x2;
     void *args[] = {&g, &x, &x2, &x_mode, &ldx, &k, &rows, &mode, &chunk, &inv_spb, &fuse};
-    return fe_hip_launch(kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1], programs, 1, 1, 256, 1, 1, lds, s, args);
+    const fe_function_t f = kern->opt.handoff_fenced && rows <= 16 ? kern->gemvb_fenced[bits_slot(ls[0]->bits)]
+                                                                   : kern->gemvb[bits_slot(ls[0]->bits)][(rows + 15) / 16 - 1];
+    return fe_hip_launch(f, programs, 1, 1, 256, 1, 1, lds, s, args);
 }
 
 // Decode-sized rows run the GEMV (with in.x != 0 it rotates that input itself and leaves the rotated rows in xh; callers
@@ -796,7 +804,7 @@ static uint32_t units_per_program(const fe_exl3_linear *l) {
 // within the 32 units a wavefront watches, and a workspace with room for the three side by side.
 static bool mlp_chain_fits(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe_exl3_linear *d, uint32_t rows,
                            const fe_exl3_workspace *ws, int y_dtype) {
-    if (!g || !u || !d || !ws || !g->kern->opt.mlp_chain) return false;
+    if (!g || !u || !d || !ws || !g->kern->opt.mlp_chain || g->kern->opt.handoff_fenced) return false;
     if (g->kern != u->kern || g->kern != d->kern || g->bits != u->bits || g->bits != d->bits) return false;
     if (g->k != u->k || g->n != u->n || d->k != g->n) return false;
     if (rows < 1 || rows > 16 || rows > ws->max_rows || y_dtype < 0 || y_dtype > 3) return false;

@@ -532,7 +532,10 @@ __device__ __forceinline__ uint32_t load_agent_u32(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <int BITS, int RG, int CHAIN = 0>
+// FENCED: the hand-off written with the memory model's own means (plain stores, a release fence at agent scope, the
+// arrival, an acquire fence, plain loads) instead of write-through stores and loads that pass the L2: the slow form
+// (the release writes the whole L2 back), kept as a cross-check of the fast one (option "handoff_fenced").
+template <int BITS, int RG, int CHAIN = 0, bool FENCED = false>
 __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, uint32_t np, uint32_t k, uint32_t m, uint32_t y_mode,
                                            uint32_t chunk, uint32_t inv_spb, const RotSrc src, uint16_t* stamp_base,
                                            const ChainCtx ch = ChainCtx{}) {
@@ -770,9 +773,15 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         //     after the barrier that publishes last_flag.
         // Every byte that crosses is written through and read through, so no cache write-back or invalidate is needed.
         float* zseg = mb.z + (size_t)(p + fnb) * m * 128;
-        for (uint32_t row = hw; row < m; row += 8)
-            store_agent_f32x4(zseg + row * 128 + 4 * l32, *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32));
-        agent_stores_wait();
+        if constexpr (FENCED) {
+            for (uint32_t row = hw; row < m; row += 8)
+                *(f32x4*)(zseg + row * 128 + 4 * l32) = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        } else {
+            for (uint32_t row = hw; row < m; row += 8)
+                store_agent_f32x4(zseg + row * 128 + 4 * l32, *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32));
+            agent_stores_wait();
+        }
         FE_STAMP(5);
         __syncthreads();
         if (tid == 0) {
@@ -782,6 +791,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         __syncthreads();
         FE_STAMP(6);
         if (last_flag) {
+            if constexpr (FENCED) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
             // A half wavefront finishes rows hw, hw + 8, ...: RB of them at a time with SB segments each, 8 or 12 agent-scope
             // loads in flight (each takes a trip to memory: the trips overlap); every row's segments are added in program
             // order (as many in flight as the registers hold without costing the kernel a resident wavefront). Up to 8 rows
@@ -802,7 +812,9 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
                             const uint32_t row = row0 + 8 * j < m ? row0 + 8 * j : row0;
 #pragma unroll
                             for (int b = 0; b < SB; b++)  // (past the last segment: out of the buffer's range, reads zero)
-                                t[j * SB + b] = load_agent_f32x4(zrs, row * 512 + 16 * l32, (sp0 + b) * m * 512);
+                                t[j * SB + b] = FENCED ? __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(
+                                                             zrs, row * 512 + 16 * l32, (sp0 + b) * m * 512, 0))
+                                                       : load_agent_f32x4(zrs, row * 512 + 16 * l32, (sp0 + b) * m * 512);
                         }
 #pragma unroll
                         for (int j = 0; j < RB; j++)
@@ -923,7 +935,17 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         gemvb_body<BITS, RG>(job.m[i], p0, left < fuse ? left : fuse, k, m, y_mode, chunk, inv_spb,                   \
                              RotSrc{x, x2, x_mode, ldx}, job.m[0].xh);                                                \
     }
-#define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4)
+#define GEMVB_FENCED_KERNEL(BITS)                                                                                     \
+    extern "C" __global__ __launch_bounds__(256, 4) void exl3_gemvb_b##BITS##_r1_fenced(                              \
+        GemvJob job, const void* x, const void* x2, uint32_t x_mode, uint32_t ldx, uint32_t k, uint32_t m,             \
+        uint32_t y_mode, uint32_t chunk, uint32_t inv_spb, uint32_t fuse) {                                            \
+        uint32_t i = 0;                                                                                               \
+        while (i + 1 < job.count && blockIdx.x >= job.first[i + 1]) i++;                                              \
+        const uint32_t p0 = (blockIdx.x - job.first[i]) * fuse, left = job.m[i].programs - p0;                        \
+        gemvb_body<BITS, 1, 0, true>(job.m[i], p0, left < fuse ? left : fuse, k, m, y_mode, chunk, inv_spb,           \
+                                     RotSrc{x, x2, x_mode, ldx}, job.m[0].xh);                                        \
+    }
+#define GEMVB_FAMILY(BITS) GEMVB_KERNEL(BITS, 1) GEMVB_KERNEL(BITS, 2) GEMVB_KERNEL(BITS, 3) GEMVB_KERNEL(BITS, 4) GEMVB_FENCED_KERNEL(BITS)
 
 // The decode MLP in one launch, 1..16 rows: grid = the front stage's workgroups (gate and up, alternating when their
 // counts are equal, so that block b of both is finished at about the same time), then the down stage's. Down workgroup

@@ -56,7 +56,9 @@ int fe_exl3_kernels_destroy(fe_exl3_kernels *k);
 /* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
  * "fused_rot" 0/1 (FE_EXL3_NO_FUSED_ROT), "fused_rot_pairs" (FE_EXL3_FUSED_ROT_PAIRS), "group" 0/1 (FE_EXL3_NO_GROUP),
  * "hat_rows" (FE_EXL3_HAT_ROWS; 0 = never), "lds_pad" 0/1 (FE_EXL3_NO_LDS_PAD), "fuse" 0/1 (FE_EXL3_NO_FUSE), "gemm_group_m" (FE_EXL3_GROUP),
- * "gemm_splits" (FE_GEMM_SPLITS), "mlp_chain" 0/1 (FE_EXL3_NO_CHAIN), "chain_spin" (FE_EXL3_CHAIN_SPIN), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the prefill GEMM never / where it
+ * "gemm_splits" (FE_GEMM_SPLITS), "mlp_chain" 0/1 (FE_EXL3_NO_CHAIN), "chain_spin" (FE_EXL3_CHAIN_SPIN),
+ * "handoff_fenced" 0/1 (the decode GEMV for 1..16 rows with its hand-off between programs written with release / acquire fences
+ * at agent scope and plain accesses instead of write-through stores and loads that pass the L2: several times slower, a cross-check), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the prefill GEMM never / where it
  * is the faster one / over all tiles / whole rounds then runs, the last two for tests). forward() reads no environment variable; tests and tuners flip a switch here. Not for
  * use while launches with this handle are being issued from another thread. No counterpart in the reference, which reads
  * its switches (FE_EXL3_NOSPLIT, FE_EXL3_UNTUNED, ...) from the environment at plan time. */

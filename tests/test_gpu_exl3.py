@@ -63,6 +63,38 @@ def test_hot_loop_decoder_is_bit_exact(env, oracle, bits, strips):
     assert np.array_equal(got, want), f"{(got != want).sum()} of {got.size} values differ"
 
 
+@pytest.mark.parametrize("bits", [3, 4, 5])
+def test_fenced_handoff_gives_the_same_bits(env, bits):
+    """The hand-off of segment sums between programs is written with write-through stores, acknowledged, a relaxed
+    agent-scope arrival, and loads that pass the L2. Option handoff_fenced runs the same partition with the memory model's
+    own means instead (plain stores, release fence, arrival, acquire fence, plain loads): slow, and required to give the
+    same bits, single linears and grouped launches, call after call on one workspace."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    ts = [synth.exl3_tensor(1024, n, bits, 500 + bits + i) for i, n in enumerate((640, 384))]
+    lins = [exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(t), exl3.Plan(11 + 4 * i, 1, 4, 4)) for i, t in enumerate(ts)]  # uneven runs
+    ws = exl3.Workspace(lins, 16)
+    try:
+        for rows in (1, 5, 16):
+            x = dev_u16(torch, synth.activations(rows, 1024, rows))
+            outs = {}
+            for fenced in (0, 1, 0, 1):
+                kern.set_option("handoff_fenced", fenced)
+                ys = [torch.zeros((rows, l.n), dtype=torch.float32, device="cuda") for l in lins]
+                single = torch.zeros((rows, lins[0].n), dtype=torch.float32, device="cuda")
+                lins[0].forward(x, exl3.Dtype.Bf16, single, exl3.Dtype.F32, rows, ws)
+                exl3.forward_group(lins, x, exl3.Dtype.Bf16, ys, exl3.Dtype.F32, rows, ws)
+                torch.cuda.synchronize()
+                got = [single.cpu()] + [y.cpu() for y in ys]
+                if fenced in outs:
+                    assert all(torch.equal(a, b) for a, b in zip(got, outs[fenced]))
+                outs[fenced] = got
+            assert all(torch.equal(a, b) for a, b in zip(outs[0], outs[1])), rows
+            assert torch.equal(outs[0][0], outs[0][1])  # a member of a group has the bits of its own forward
+    finally:
+        kern.set_option("handoff_fenced", 0)
+
+
 def test_reconstruct_bf16_within_one_ulp(env, oracle):
     """crates/fe-exl3/src/bin/exl3-gpucheck.rs:58-98: GPU f32 math vs the f64 reference: at most 1 bf16 ulp apart, more
     only as f32 cancellation noise near zero (absolute error below 1e-4 of the tensor's rms); [n][k] is the exact
