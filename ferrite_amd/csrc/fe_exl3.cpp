@@ -53,6 +53,7 @@ struct fe_exl3_options {
     uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
     uint32_t handoff_fenced = 0;   // 1..16 rows through the kernels whose hand-off uses release / acquire fences (a slow cross-check)
     uint32_t mlp_chain = 1;        // the decode MLP (gate, up, down) as one launch where it applies (FE_EXL3_NO_CHAIN=1: off)
+    uint32_t chain_rot_pairs = 32; // (row, 128-channel block) pairs a program rotates at most inside the one-launch MLP (FE_EXL3_CHAIN_ROT_PAIRS)
     uint32_t chain_perm = 1;       // the down stage's workgroups in the order in which their inputs get ready (FE_EXL3_CHAIN_PERM)
     uint32_t chain_spin = 1u << 16;  // polls a program of the down stage waits for the front stage's outputs (FE_EXL3_CHAIN_SPIN)
 };
@@ -177,6 +178,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     o.mlp_chain = env_u32("FE_EXL3_NO_CHAIN", 0) ? 0 : 1;
     o.chain_spin = env_u32("FE_EXL3_CHAIN_SPIN", o.chain_spin);
     o.chain_perm = env_u32("FE_EXL3_CHAIN_PERM", o.chain_perm);
+    o.chain_rot_pairs = env_u32("FE_EXL3_CHAIN_ROT_PAIRS", o.chain_rot_pairs);
     if (!c) {
         int cus = 0;
         c = fe_hip_cu_count(&cus);
@@ -214,6 +216,7 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     else if (nm == "handoff_fenced") o.handoff_fenced = value;
     else if (nm == "chain_spin") o.chain_spin = value;
     else if (nm == "chain_perm") o.chain_perm = value;
+    else if (nm == "chain_rot_pairs") o.chain_rot_pairs = value;
     else return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", name);
     return 0;
 }
@@ -808,7 +811,12 @@ static bool mlp_chain_fits(const fe_exl3_linear *g, const fe_exl3_linear *u, con
     if (g->kern != u->kern || g->kern != d->kern || g->bits != u->bits || g->bits != d->bits) return false;
     if (g->k != u->k || g->n != u->n || d->k != g->n) return false;
     if (rows < 1 || rows > 16 || rows > ws->max_rows || y_dtype < 0 || y_dtype > 3) return false;
-    if (!fused_rotation_fits(g, rows) || !fused_rotation_fits(u, rows) || !fused_rotation_fits(d, rows)) return false;
+    // every stage rotates its own input inside the launch: (row, 128-channel block) pairs a program. As separate launches
+    // that pays up to 16 pairs (fused_rotation_fits); inside the one launch up to 32, i.e. up to 4 rows on the 27B-shaped
+    // MLP (measured at 4 bits, cold weights: 4 rows 53.6 us against 56.8 us for rotation and GEMV launches; 8 rows 65.1 / 60.1)
+    const fe_exl3_options &o = g->kern->opt;
+    for (const fe_exl3_linear *l : {g, u, d})
+        if (!o.fused_rot || rows * units_per_program(l) > o.chain_rot_pairs) return false;
     if (units_per_program(d) > 32) return false;
     if (std::max(g->k, d->k) > ws->max_k || (size_t)2 * rows * g->k * 2 > ws->xh.bytes) return false;
     if (job_z(g, rows) + job_z(u, rows) + job_z(d, rows) > ws->z_len) return false;

@@ -143,9 +143,10 @@ int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_
  * word), and rotate SwiGLU(gate, up) from there; start-up, launch overhead and tail of the second launch disappear
  * under the first. The wait is bounded ("chain_spin" polls, about a microsecond each): when it runs out the program sets
  * the workspace's chain error word and goes on, the launch still ends normally, and its results are void;
- * fe_exl3_workspace_chain_status reports and clears that. It applies to 1..16 rows where all three linears rotate their
- * own input (fe_exl3_linear_forward_is_one_launch), with the same width, gate and up of one shape, and a workspace
- * created from (at least) these three linears; "mlp_chain" 0 (FE_EXL3_NO_CHAIN=1) turns it off.
+ * fe_exl3_workspace_chain_status reports and clears that. It applies where every program rotates at most
+ * "chain_rot_pairs" (32) pairs of (row, 128-channel block) of its own input (up to 4 rows on a 5120 x 17408 MLP), with the
+ * same width, gate and up of one shape, and a workspace created from (at least) these three linears; "mlp_chain" 0
+ * (FE_EXL3_NO_CHAIN=1) turns it off.
  * fe_exl3_mlp_forward_launches: 1 if the call is the one launch, else 0. */
 int fe_exl3_mlp_forward(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down,
                         const fe_exl3_kernels *kern, fe_stream_t s, fe_devptr_t x, int x_dtype, fe_devptr_t yg, fe_devptr_t yu,

@@ -43,7 +43,7 @@ def run(torch, exl3, lins, x, rows, y_dtype, ws, y0=None, stream=None):
 
 @pytest.mark.parametrize("bits,hidden,inter,rows,y_dtype", [
     (4, 512, 1536, 1, 0), (4, 1024, 2048, 1, 2), (3, 512, 1536, 2, 1), (5, 768, 1280, 1, 3), (2, 512, 1024, 1, 0),
-    (6, 512, 1024, 1, 0), (8, 512, 1024, 1, 0)])
+    (6, 512, 1024, 1, 0), (8, 512, 1024, 1, 0), (4, 1024, 2048, 4, 0), (5, 512, 1536, 3, 2)])
 def test_one_launch_has_the_bits_of_the_two_launches(bits, hidden, inter, rows, y_dtype):
     import torch
     from ferrite_amd import exl3, synth
