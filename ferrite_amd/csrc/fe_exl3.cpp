@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -51,6 +52,7 @@ struct fe_exl3_options {
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
     uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
+    uint32_t chain_down_units = 4; // the one-launch MLP's down stage in programs of this many units where that divides a column block (0: the linear's own partition; FE_EXL3_CHAIN_DOWN_UNITS)
     uint32_t handoff_fenced = 0;   // 1..16 rows through the kernels whose hand-off uses release / acquire fences (a slow cross-check)
     uint32_t mlp_chain = 1;        // the decode MLP (gate, up, down) as one launch where it applies (FE_EXL3_NO_CHAIN=1: off)
     uint32_t chain_rot_pairs = 32; // (row, 128-channel block) pairs a program rotates at most inside the one-launch MLP (FE_EXL3_CHAIN_ROT_PAIRS)
@@ -82,7 +84,17 @@ struct fe_exl3_linear {
     fe_exl3_view view{};
     FeBuf trellis, suh, svh;  // owned copies (upload), empty for from_view
     FeBuf hat;                // decoded fp16 tiles kept with the linear (fe_exl3_linear_keep_decoded), else empty
-    FeBuf chain_order;        // u32[programs]: the programs sorted by the last channel block their run reads (one-launch MLP)
+    // The linear as the down projection of a one-launch MLP: its partition there (the linear's own, and partitions into
+    // programs of 2, 4 and 8 units where that divides a column block) with u32[programs], the programs sorted by the last
+    // channel block their run reads.
+    struct ChainPart {
+        uint32_t unit_len = 0, programs = 0;  // unit_len 0: the linear's own partition
+        FeBuf order;
+        // the same weights (no copies: the view) as a linear of this partition, for the launches of the MLP call that are
+        // not the one launch: every row count then sums down's segments in the same order
+        std::unique_ptr<fe_exl3_linear> as_linear;
+    };
+    std::vector<std::unique_ptr<ChainPart>> chain_parts;
     const fe_exl3_kernels *kern = nullptr;
 };
 
@@ -179,6 +191,7 @@ int fe_exl3_kernels_load(fe_exl3_kernels **out) {
     o.chain_spin = env_u32("FE_EXL3_CHAIN_SPIN", o.chain_spin);
     o.chain_perm = env_u32("FE_EXL3_CHAIN_PERM", o.chain_perm);
     o.chain_rot_pairs = env_u32("FE_EXL3_CHAIN_ROT_PAIRS", o.chain_rot_pairs);
+    o.chain_down_units = env_u32("FE_EXL3_CHAIN_DOWN_UNITS", o.chain_down_units);
     if (!c) {
         int cus = 0;
         c = fe_hip_cu_count(&cus);
@@ -203,7 +216,8 @@ int fe_exl3_kernels_set_option(fe_exl3_kernels *k, const char *name, uint32_t va
     if (!k || !name) return fe_set_error(FE_ERR_ARG, "fe_exl3_kernels_set_option", "null argument");
     fe_exl3_options &o = k->opt;
     const std::string nm = name;
-    if (nm == "fused_rot") o.fused_rot = value;
+    if (nm == "chain_down_units") o.chain_down_units = value;
+    else if (nm == "fused_rot") o.fused_rot = value;
     else if (nm == "fused_rot_pairs") o.fused_rot_pairs = value;
     else if (nm == "group") o.group = value;
     else if (nm == "hat_rows") o.hat_rows = value == 0 ? 0xffffffffu : std::max(value, kMaxRowsPerPass + 1);
@@ -274,19 +288,47 @@ static uint32_t plan_programs(const fe_exl3_kernels *kern, const fe_exl3_plan &p
     return std::max(1u, std::min(progs, units));
 }
 
-// The programs of the linear's partition in the order in which, as the down projection of a one-launch MLP, their inputs
-// get ready: sorted by the last 128-channel block their run reads (a run that crosses into the next column block reads
-// the last block of all), then by where the run starts.
-static int make_chain_order(fe_exl3_linear *l) {
-    const uint32_t upb = l->k / 128, units = upb * (l->n / 128), base = units / l->programs, rem = units % l->programs;
-    std::vector<uint32_t> order(l->programs), last(l->programs);
-    for (uint32_t p = 0; p < l->programs; p++) {
+// The programs of a partition of the linear in the order in which, as the down projection of a one-launch MLP, their
+// inputs get ready: sorted by the last 128-channel block their run reads (a run that crosses into the next column block
+// reads the last block of all), then by program number. A program of the down stage waits for lower-numbered programs'
+// inputs only through this order, which keeps every program behind the ones that started earlier in K.
+static int make_chain_part(fe_exl3_linear *l, uint32_t unit_len, uint32_t programs) {
+    const uint32_t upb = l->k / 128, units = upb * (l->n / 128), base = units / programs, rem = units % programs;
+    std::vector<uint32_t> order(programs), last(programs);
+    for (uint32_t p = 0; p < programs; p++) {
         const uint32_t u0 = p * base + std::min(p, rem), len = base + (p < rem ? 1 : 0), kb0 = u0 % upb;
         order[p] = p;
         last[p] = kb0 + len > upb ? upb - 1 : kb0 + len - 1;
     }
     std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return last[a] < last[b]; });
-    return l->chain_order.from_host(order.data(), order.size() * 4);
+    auto part = std::make_unique<fe_exl3_linear::ChainPart>();
+    part->unit_len = unit_len, part->programs = programs;
+    if (int c = part->order.from_host(order.data(), order.size() * 4)) return c;
+    if (unit_len) {
+        part->as_linear = std::make_unique<fe_exl3_linear>();
+        fe_exl3_linear &sh = *part->as_linear;
+        sh.name = l->name, sh.k = l->k, sh.n = l->n, sh.bits = l->bits, sh.plan = l->plan, sh.programs = programs;
+        sh.view = l->view, sh.kern = l->kern;
+    }
+    l->chain_parts.push_back(std::move(part));
+    return 0;
+}
+
+static int make_chain_order(fe_exl3_linear *l) {
+    if (int c = make_chain_part(l, 0, l->programs)) return c;
+    const uint32_t upb = l->k / 128, units = upb * (l->n / 128);
+    for (uint32_t len : {2u, 4u, 8u})
+        if (upb % len == 0 && units / len <= 8192 && units / len != l->programs)
+            if (int c = make_chain_part(l, len, units / len)) return c;
+    return 0;
+}
+
+// The partition the linear takes as the down stage of a one-launch MLP under the kernels' current options.
+static const fe_exl3_linear::ChainPart *chain_part(const fe_exl3_linear *l) {
+    const uint32_t want = l->kern->opt.chain_down_units;
+    for (const auto &part : l->chain_parts)
+        if (want && part->unit_len == want) return part.get();
+    return l->chain_parts[0].get();
 }
 
 static int check_fit(const char *name, uint32_t k, uint32_t n, uint32_t bits, const fe_exl3_plan &p) {
@@ -352,12 +394,12 @@ int fe_exl3_linear_upload(fe_exl3_linear **out, const fe_exl3_kernels *kern, con
     }
     if (!c) c = l->suh.from_host(suh, (size_t)k * 2);
     if (!c) c = l->svh.from_host(svh, (size_t)n * 2);
+    l->view = fe_exl3_view{k, n, bits, l->trellis.p, l->suh.p, l->svh.p, strips ? 1u : 0u};
     if (!c) c = make_chain_order(l);
     if (c) {
         delete l;
         return c;
     }
-    l->view = fe_exl3_view{k, n, bits, l->trellis.p, l->suh.p, l->svh.p, strips ? 1u : 0u};
     *out = l;
     return 0;
 }
@@ -385,6 +427,8 @@ static size_t hat_bytes(const fe_exl3_linear *l) { return (size_t)((l->n / 128 +
 
 // Room one linear's GEMV takes in a workspace at `rows` rows: a slot of 128 sums per (program, column block it touches).
 static size_t job_z(const fe_exl3_linear *l, uint32_t rows) { return (size_t)(l->programs + l->n / 128) * 128 * rows; }
+// ... as the down stage of a one-launch MLP
+static size_t chain_z(const fe_exl3_linear *l, uint32_t rows) { return (size_t)(chain_part(l)->programs + l->n / 128) * 128 * rows; }
 
 extern "C" {
 
@@ -395,7 +439,7 @@ int fe_exl3_workspace_create(fe_exl3_workspace **out, fe_exl3_linear *const *lin
     std::vector<size_t> zs, nbs;  // per linear; a launch of several linears needs room for the kGroupMax largest together
     for (size_t i = 0; i < count; i++) {
         const fe_exl3_linear *l = linears[i];
-        zs.push_back(job_z(l, 1));
+        zs.push_back(std::max(job_z(l, 1), chain_z(l, 1)));
         nbs.push_back(l->n / 128);
         max_hat = std::max(max_hat, hat_bytes(l));
         max_k = std::max<size_t>(max_k, l->k);
@@ -787,19 +831,19 @@ struct MlpChainArgs {
 };
 static_assert(sizeof(MlpChainArgs) == 24 + kGroupMax * 88 + 88 + 16 + 12 * 4, "MlpChain layout");
 
-static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, fe_devptr_t xh, fe_devptr_t y, fe_devptr_t z,
-                        fe_devptr_t counters) {
+static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, uint32_t programs, fe_devptr_t xh, fe_devptr_t y,
+                        fe_devptr_t z, fe_devptr_t counters) {
     m.trellis = l->view.trellis, m.svh = l->view.svh, m.suh = l->view.suh, m.xh = xh, m.y = y, m.z = z, m.counters = counters;
-    m.n = l->n, m.programs = l->programs;
+    m.n = l->n, m.programs = programs;
     view_strides(l->view, &m.stride_k, &m.stride_nb);
     const uint32_t units = (l->k / 128) * (l->n / 128);
-    m.base = units / l->programs, m.rem = units % l->programs;
+    m.base = units / programs, m.rem = units % programs;
     m.inv_base = 0xffffffffu / m.base, m.inv_base1 = 0xffffffffu / (m.base + 1);
 }
 
-static uint32_t units_per_program(const fe_exl3_linear *l) {
+static uint32_t units_per_program(const fe_exl3_linear *l, uint32_t programs) {
     const uint32_t units = (l->k / 128) * (l->n / 128);
-    return (units + l->programs - 1) / l->programs;
+    return (units + programs - 1) / programs;
 }
 
 // Whether the decode MLP gate, up -> SwiGLU -> down runs as one launch: trellis linears of one width, gate and up of one
@@ -815,11 +859,12 @@ static bool mlp_chain_fits(const fe_exl3_linear *g, const fe_exl3_linear *u, con
     // that pays up to 16 pairs (fused_rotation_fits); inside the one launch up to 32, i.e. up to 4 rows on the 27B-shaped
     // MLP (measured at 4 bits, cold weights: 4 rows 53.6 us against 56.8 us for rotation and GEMV launches; 8 rows 65.1 / 60.1)
     const fe_exl3_options &o = g->kern->opt;
-    for (const fe_exl3_linear *l : {g, u, d})
-        if (!o.fused_rot || rows * units_per_program(l) > o.chain_rot_pairs) return false;
-    if (units_per_program(d) > 32) return false;
+    const uint32_t d_units = units_per_program(d, chain_part(d)->programs);
+    if (!o.fused_rot || rows * std::max({units_per_program(g, g->programs), units_per_program(u, u->programs), d_units}) > o.chain_rot_pairs)
+        return false;
+    if (d_units > 32) return false;
     if (std::max(g->k, d->k) > ws->max_k || (size_t)2 * rows * g->k * 2 > ws->xh.bytes) return false;
-    if (job_z(g, rows) + job_z(u, rows) + job_z(d, rows) > ws->z_len) return false;
+    if (job_z(g, rows) + job_z(u, rows) + chain_z(d, rows) > ws->z_len) return false;
     if ((size_t)(2 * (g->n / 128) + d->n / 128) > ws->counters_len || kChainStride * (1 + 2 * (size_t)(g->n / 128)) > ws->chain_len) return false;
     return true;
 }
@@ -841,7 +886,8 @@ static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe
     a.front.count = 2;
     for (int i = 0; i < 2; i++) {
         const fe_exl3_linear *l = front[i];
-        fill_member(a.front.m[i], l, ws->xh.p + (size_t)i * rows * l->k * 2, ys[i], ws->z.p + z_at * 4, ws->counters.p + cnt_at * 4);
+        fill_member(a.front.m[i], l, l->programs, ws->xh.p + (size_t)i * rows * l->k * 2, ys[i], ws->z.p + z_at * 4,
+                    ws->counters.p + cnt_at * 4);
         a.front.first[i] = wgs;
         wgs += (l->programs + a.fuse1 - 1) / a.fuse1;
         z_at += job_z(l, rows), cnt_at += l->n / 128;
@@ -849,7 +895,8 @@ static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe
     for (size_t i = 2; i <= kGroupMax; i++) a.front.first[i] = wgs;
     a.front_wgs = wgs;
     a.interleave = g->programs == u->programs ? 1 : 0;
-    fill_member(a.down, d, ws->xh.p, y, ws->z.p + z_at * 4, ws->counters.p + cnt_at * 4);
+    const fe_exl3_linear::ChainPart *dp = chain_part(d);
+    fill_member(a.down, d, dp->programs, ws->xh.p, y, ws->z.p + z_at * 4, ws->counters.p + cnt_at * 4);
     a.state = ws->chain.p;
     a.k1 = g->k, a.k2 = d->k;
     a.inv_spb1 = 0xffffffffu / (a.k1 / 64), a.inv_spb2 = 0xffffffffu / (a.k2 / 64);
@@ -858,14 +905,14 @@ static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe
         const uint32_t c = std::max(4u, ((kJobLdsBudget - red) / rows - 16) / 128 / 4 * 4);
         return std::min(c, (run_steps + 3) / 4 * 4);
     };
-    a.chunk1 = chunk_of(2 * a.fuse1 * std::max(units_per_program(g), units_per_program(u)));
-    a.chunk2 = chunk_of(2 * a.fuse2 * units_per_program(d));
+    a.chunk1 = chunk_of(2 * a.fuse1 * std::max(units_per_program(g, g->programs), units_per_program(u, u->programs)));
+    a.chunk2 = chunk_of(2 * a.fuse2 * units_per_program(d, dp->programs));
     uint32_t lds = red + rows * (std::max(a.chunk1, a.chunk2) * 128 + 16);
     if (occ && kern->opt.lds_pad) lds = std::max(lds, kCuLds / (occ + 1) + 512);
     // the down stage's programs in the order in which their inputs get ready (the linear's table)
-    a.perm = kern->opt.chain_perm ? d->chain_order.p : 0;
+    a.perm = kern->opt.chain_perm ? dp->order.p : 0;
     a.spin_limit = kern->opt.chain_spin;
-    const uint32_t grid = a.front_wgs + (d->programs + a.fuse2 - 1) / a.fuse2;
+    const uint32_t grid = a.front_wgs + (dp->programs + a.fuse2 - 1) / a.fuse2;
     uint32_t x_mode = (uint32_t)x_dtype & 1, ldx = g->k, mode = (uint32_t)y_dtype;
     void *args[] = {&a, &x, &x_mode, &ldx, &rows, &mode};
     return fe_hip_launch(kern->mlp[bits_slot(g->bits)], grid, 1, 1, 256, 1, 1, lds, s, args);
@@ -891,7 +938,14 @@ int fe_exl3_mlp_forward(const fe_exl3_linear *gate, const fe_exl3_linear *up, co
     const fe_exl3_linear *front[2] = {gate, up};
     const fe_devptr_t ys[2] = {yg, yu};
     FE_TRY(fe_exl3_linear_forward_group(front, 2, kern, s, x, x_dtype, ys, FE_DTYPE_BF16, rows, ws));
-    return fe_exl3_linear_forward_swiglu(down, kern, s, yg, yu, gate->n, y, y_dtype, rows, ws);
+    // down in the partition it has in the one launch (where the GEMV runs and the workspace has the room), so that a row's
+    // bits are the same at every row count of this call
+    const fe_exl3_linear *dl = down;
+    if (rows <= kMaxRowsPerPass) {
+        const fe_exl3_linear::ChainPart *part = chain_part(down);
+        if (part->as_linear && job_z(part->as_linear.get(), rows) <= ws->z_len) dl = part->as_linear.get();
+    }
+    return fe_exl3_linear_forward_swiglu(dl, kern, s, yg, yu, gate->n, y, y_dtype, rows, ws);
 }
 
 int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error) {

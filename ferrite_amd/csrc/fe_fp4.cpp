@@ -2,6 +2,7 @@
 // are ferrite_amd/csrc/kernels/k_fp4.hip.
 #include "fe_fp4.h"
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -22,6 +23,7 @@ struct fe_fp4_kernels {
     fe_module_t module = nullptr;
     fe_function_t quant4 = nullptr, gemm4 = nullptr, reduce4 = nullptr, gemv4[3] = {nullptr, nullptr, nullptr};
     fe_function_t strip4 = nullptr;  // the GEMV over strips of 16 weight rows, up to 16 activation rows (no hand-off)
+    fe_function_t strip_once[5] = {};  // ... with every load of a workgroup issued before anything waits: 1..5 groups of K a wavefront
     fe_function_t quant8 = nullptr, gemm8 = nullptr, swiglu4 = nullptr, swiglu_reduce4 = nullptr;
     fe_function_t gemm8c = nullptr;  // FP8 on the 8-bit matrix instruction, operands as codes
     fe_function_t gemm4_sk = nullptr, gemm8_sk = nullptr, gemm8c_sk = nullptr, swiglu4_sk = nullptr;  // the same on the stream-K schedule
@@ -32,6 +34,7 @@ struct fe_fp4_kernels {
     uint32_t gemv = 1;         // up to 64 rows run the GEMV (FE_FP4_NO_GEMV=1: the GEMM's single tile row)
     uint32_t gemv_sk = 0;      // K splits of the GEMV over weight tiles; 0 = two programs a CU (FE_FP4_GEMV_SK)
     uint32_t gemv_strips = 1;  // the GEMV runs over strips of 16 weight rows, K split inside the workgroup (FE_FP4_NO_STRIPS=1: over weight tiles and K splits)
+    uint32_t gemv_once = 1;    // strips whose loads all go out at once, where a wavefront's share of K allows (FE_FP4_NO_ONCE=1: never)
     uint32_t gemv_waves = 0;   // wavefronts of a strip's workgroup: 4, 8 or 16; 0 = four or more wavefronts a SIMD (FE_FP4_GEMV_WAVES)
     int32_t xcd = -1;          // column tiles dealt to the XCDs: -1 = where the weights are the larger operand (FE_FP4_XCD)
     uint32_t fp8_f16 = 0;      // FP8 linears as fp16 expansion on the 16-bit matrix instruction (FE_FP8_F16=1)
@@ -74,6 +77,11 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     }
     if (!c) c = fe_hip_module_get_function(&k->strip4, k->module, "fe_gemv_nvfp4_strips");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->strip4, 48 * 1024);
+    for (int g = 1; g <= 5 && !c; g++) {
+        const std::string nm = "fe_gemv_nvfp4_strips_once_g" + std::to_string(g);
+        c = fe_hip_module_get_function(&k->strip_once[g - 1], k->module, nm.c_str());
+        if (!c) c = fe_hip_func_set_max_dyn_lds(k->strip_once[g - 1], 48 * 1024);
+    }
     if (!c) c = fe_hip_module_get_function(&k->quant8, k->module, "fe_fp8_quant");
     if (!c) c = fe_hip_module_get_function(&k->gemm8, k->module, "fe_gemm_fp8");
     if (!c) c = fe_hip_func_set_max_dyn_lds(k->gemm8, kGemmLds);
@@ -96,6 +104,7 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out) {
     if (const char *e = getenv("FE_FP4_NO_GEMV")) k->gemv = atoi(e) ? 0 : 1;
     if (const char *e = getenv("FE_FP4_GEMV_SK")) k->gemv_sk = (uint32_t)atoi(e);
     if (const char *e = getenv("FE_FP4_NO_STRIPS")) k->gemv_strips = atoi(e) ? 0 : 1;
+    if (const char *e = getenv("FE_FP4_NO_ONCE")) k->gemv_once = atoi(e) ? 0 : 1;
     if (const char *e = getenv("FE_FP4_GEMV_WAVES")) k->gemv_waves = (uint32_t)atoi(e);
     if (const char *e = getenv("FE_FP4_XCD")) k->xcd = atoi(e) ? 1 : 0;
     if (const char *e = getenv("FE_FP8_F16")) k->fp8_f16 = atoi(e) ? 1 : 0;
@@ -123,6 +132,7 @@ int fe_fp4_kernels_set_option(fe_fp4_kernels *k, const char *name, int32_t value
     else if (nm == "gemv") k->gemv = value ? 1 : 0;
     else if (nm == "gemv_sk") k->gemv_sk = (uint32_t)value;
     else if (nm == "gemv_strips") k->gemv_strips = (uint32_t)value;
+    else if (nm == "gemv_once") k->gemv_once = (uint32_t)value;
     else if (nm == "gemv_waves") k->gemv_waves = (uint32_t)value;
     else if (nm == "xcd") k->xcd = value;
     else if (nm == "fp8_f16") k->fp8_f16 = value ? 1 : 0;
@@ -347,13 +357,29 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
             while (waves < 16 && strips * waves < 8 * kern->cus) waves *= 2;
             if (kern->gemv_waves && kern->gemv_waves <= 16 && !(kern->gemv_waves & (kern->gemv_waves - 1))) waves = kern->gemv_waves;
             while (waves > 1 && waves > kts / 4) waves /= 2;
+            // Where a wavefront's share of K can be at most five groups of four k tiles and the activations at most four
+            // 16-byte pieces a thread, the kernel that issues every load at once, with the number of wavefronts (any, up to
+            // 16) that wastes the fewest loads: a wavefront with fewer groups than the others requests one again, and a
+            // load instruction costs the address unit the same either way (5120 x 5120: 8 wavefronts of 3 groups for 20
+            // groups 9.3 us, 10 of 2 groups measured faster).
+            fe_function_t strip_fn = kern->strip4;
+            if (kern->gemv_once) {
+                const uint32_t groups = k / 256, want = kern->gemv_waves ? waves : std::max(4u, (8 * kern->cus + strips - 1) / strips);
+                uint32_t best_w = 0, best_waste = ~0u;
+                for (uint32_t w1 = std::min(want, 16u); w1 <= (kern->gemv_waves ? want : 16u); w1++) {
+                    const uint32_t gpw = (groups + w1 - 1) / w1;
+                    if (gpw > 5 || w1 > groups || ((size_t)m * (k / 8) + 64 * w1 - 1) / (64 * w1) > 4) continue;
+                    if (w1 * gpw - groups < best_waste) best_waste = w1 * gpw - groups, best_w = w1;
+                }
+                if (best_w) waves = best_w, strip_fn = kern->strip_once[(groups + best_w - 1) / best_w - 1];
+            }
             fe_devptr_t w = l->w.p, sw = l->sw.p, alpha = l->alpha.p;
             uint32_t w_snt = l->w_snt, w_skt = l->w_skt, w_sr = l->w_sr, s_snt = l->s_snt, s_skt = l->s_skt, s_sr = l->s_sr;
             for (uint32_t r0 = 0; r0 < m; r0 += kGemvRows) {
                 uint32_t rows = m - r0 < kGemvRows ? m - r0 : kGemvRows;
                 fe_devptr_t yy = y + (size_t)r0 * ldy * 2, aq = ws->aq.p + (size_t)r0 * k * 2, rr = res ? res + (size_t)r0 * ldy * 2 : 0;
                 void *args[] = {&yy, &aq, &w, &sw, &alpha, &rr, &rows, &n, &k, &ldy, &w_snt, &w_skt, &w_sr, &s_snt, &s_skt, &s_sr};
-                FE_TRY(fe_hip_launch(kern->strip4, strips, 1, 1, 64 * waves, 1, 1, rows * k * 2, s, args));
+                FE_TRY(fe_hip_launch(strip_fn, strips, 1, 1, 64 * waves, 1, 1, rows * k * 2, s, args));
             }
             return 0;
         }

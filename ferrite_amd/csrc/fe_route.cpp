@@ -375,12 +375,14 @@ int fe_route_mlp_forward_w(const fe_route_ctx *c, const fe_route_proj *gate_up, 
     }
     const uint32_t n_rest = fused ? d : rows;
     if (n_rest > 0 && gate_up->lins.size() == 2 && !(gate_up->prompt && c->fp4() && n_rest > FE_X3_ROWS) && c->x3() && down->q) {
-        // Decode rows through three trellis linears, gate and up each one part: the whole block as one launch where
-        // that applies (fe_exl3_mlp_forward: the bits of the grouped gate + up launch and down's forward_swiglu below)
+        // Decode rows through three trellis linears, gate and up each one part, every row in one GEMV pass: the block
+        // through fe_exl3_mlp_forward at every such row count (one launch where that applies, else the grouped gate + up
+        // launch and down's forward_swiglu with down partitioned as in the one launch), so that a row's bits do not
+        // depend on the batch it is in
         const fe_route_linear *g = gate_up->lins[0].first, *u = gate_up->lins[1].first;
         if (g->q && u->q && g->k == hidden && u->k == hidden && g->n == inter && u->n == inter &&
-            gate_up->lins[0].second.size() == 1 && gate_up->lins[1].second.size() == 1 &&
-            fe_exl3_mlp_forward_launches(g->q, u->q, down->q, n_rest, FE_DTYPE_BF16_ADD, c->xws) == 1)
+            gate_up->lins[0].second.size() == 1 && gate_up->lins[1].second.size() == 1 && n_rest <= FE_X3_PASS &&
+            (n_rest <= FE_X3_ROWS || d >= n_rest))
             return fe_exl3_mlp_forward(g->q, u->q, down->q, c->xk, c->s, xn, FE_DTYPE_BF16, big, big + (size_t)n_rest * inter * 2, x,
                                        FE_DTYPE_BF16_ADD, n_rest, c->xws);
     }

@@ -896,6 +896,97 @@ extern "C" __global__ __launch_bounds__(1024) void fe_gemv_nvfp4_strips(uint16_t
     gemv_nvfp4_strip_body(c, aq, w, sw, alpha, res, m, n, k, ldc, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);
 }
 
+// The same strips when a wavefront's share of K is GPW <= 5 groups and the activations are at most four 16-byte pieces a
+// thread: every load of the workgroup goes out before anything waits. The activations' loads first (they
+// are few and mostly hit L2; loads return in order), then the wavefront's whole share of the strip, then the activations
+// go to LDS while the weights are on their way, and the groups are taken in the order they arrive. No load sits under a
+// condition (a wavefront with fewer groups than the others requests its last group again and does not use it; a thread
+// past the end of the activations requests the last piece again), so the compiler counts its waits exactly instead of
+// waiting for everything at the head of a loop. A vector memory instruction costs the address unit the same whether
+// its data is wanted or not, so the kernel exists per GPW and the host picks a number of wavefronts that divides the
+// groups where it can (any number up to 16, not only powers of two).
+template <int GPW>
+__device__ __forceinline__ void gemv_nvfp4_strip_once_body(uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw,
+                                                           const float* alpha, const uint16_t* res, uint32_t m, uint32_t k,
+                                                           uint32_t ldc, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr,
+                                                           uint32_t s_snt, uint32_t s_skt, uint32_t s_sr) {
+    __shared__ f32x4 red[FP4_STRIP_WAVES_MAX][64];
+    __shared__ u32x2 scale_lut[128];
+    extern __shared__ __attribute__((aligned(16))) unsigned char xs[];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6, r = lane & 15, g = lane >> 4;
+    constexpr int XV = 4;
+    const uint32_t xn = m * (k / 8);  // 16-byte pieces of the activations
+    u32x4 xv[XV];
+    uint32_t xi[XV];
+#pragma unroll
+    for (int i = 0; i < XV; i++) {
+        xi[i] = tid + i * blockDim.x;
+        xi[i] = xi[i] < xn ? xi[i] : xn - 1;
+        xv[i] = ((const u32x4*)aq)[xi[i]];
+    }
+    const uint32_t strip = blockIdx.x, nt = strip >> 3, rg = strip & 7;  // the strip: 16-row group rg of weight tile nt
+    const uint32_t groups = k / 256;                                      // groups of four k tiles
+    const uint8_t* wp = w + (size_t)nt * w_snt + (size_t)(16 * rg + r) * w_sr + (size_t)g * w_skt;
+    const uint8_t* sp = sw + (size_t)nt * s_snt + (size_t)(16 * rg + r) * s_sr + (size_t)g * s_skt;
+    Fp4StripStage st[GPW];
+#pragma unroll
+    for (int i = 0; i < GPW; i++) {
+        uint32_t gi = wave + waves * i;
+        gi = gi < groups ? gi : groups - 1;
+        const uint8_t* p = wp + (size_t)gi * 4 * w_skt;
+        st[i].c[0] = __builtin_nontemporal_load((const u32x4*)p);
+        st[i].c[1] = __builtin_nontemporal_load((const u32x4*)(p + 16));
+        st[i].sc = __builtin_nontemporal_load((const uint32_t*)(sp + (size_t)gi * 4 * s_skt));
+    }
+    fp4_scale_lut_fill(scale_lut);
+#pragma unroll
+    for (int i = 0; i < XV; i++) ((u32x4*)xs)[xi[i]] = xv[i];
+    __syncthreads();  // scale_lut, xs
+    const uint32_t xo = ((r < m ? r : m - 1) * k + 64 * g) * 2;  // byte offset in xs of the lane's activation row at k tile g
+    f32x4 acc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < GPW; i++) {
+        const uint32_t gi = wave + waves * i;
+        if (gi < groups) {
+#pragma unroll
+            for (int blk = 0; blk < 4; blk++) {  // scale block blk of the lane's k tile: codes 16 blk .. 16 blk + 15
+                const Fp4Scale sc = fp4_scale_lut(scale_lut, __builtin_amdgcn_ubfe(st[i].sc, 8 * blk, 8) << 3);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    u32x4 a = fp4x8_to_f16(st[i].c[blk >> 1][2 * (blk & 1) + j], sc);
+                    const f16x8 x = *(const f16x8*)(xs + xo + gi * 512 + 32 * blk + 16 * j);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), x, acc, 0, 0, 0);
+                }
+            }
+        }
+    }
+    // The wavefronts' sums meet in LDS; wavefront 0 adds them in wavefront order. Lane (r, g) holds output row r, columns
+    // 16 strip + 4 g .. + 3. (The groups of a wavefront are added in the order of the kernel above: the same bits.)
+    const uint32_t col = 16 * strip + 4 * g;
+    red[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && r < m) {
+        f32x4 sum = red[0][lane];
+        for (uint32_t v = 1; v < waves; v++) sum += red[v][lane];
+        float o[4] = {sum[0], sum[1], sum[2], sum[3]};
+        fp4_store4(c, res, (size_t)r * ldc + col, o, *(const f32x4*)(alpha + col) * FP4_OPERAND_SCALE);
+    }
+}
+
+#define FP4_STRIPS_ONCE_KERNEL(GPW)                                                                                       \
+    extern "C" __global__ __launch_bounds__(1024) void fe_gemv_nvfp4_strips_once_g##GPW(                                  \
+        uint16_t* c, const _Float16* aq, const uint8_t* w, const uint8_t* sw, const float* alpha, const uint16_t* res,   \
+        uint32_t m, uint32_t n, uint32_t k, uint32_t ldc, uint32_t w_snt, uint32_t w_skt, uint32_t w_sr, uint32_t s_snt, \
+        uint32_t s_skt, uint32_t s_sr) {                                                                                  \
+        (void)n;                                                                                                          \
+        gemv_nvfp4_strip_once_body<GPW>(c, aq, w, sw, alpha, res, m, k, ldc, w_snt, w_skt, w_sr, s_snt, s_skt, s_sr);     \
+    }
+FP4_STRIPS_ONCE_KERNEL(1)
+FP4_STRIPS_ONCE_KERNEL(2)
+FP4_STRIPS_ONCE_KERNEL(3)
+FP4_STRIPS_ONCE_KERNEL(4)
+FP4_STRIPS_ONCE_KERNEL(5)
+
 // ---- matrix-unit peak probe ---------------------------------------------------------------------------------------------
 //
 // Every wavefront issues iters x 16 independent matrix instructions (the GEMM core's 4 x 4 accumulator pieces, 256

@@ -26,7 +26,8 @@ int fe_fp4_kernels_load(fe_fp4_kernels **out);
 int fe_fp4_kernels_destroy(fe_fp4_kernels *k);
 /* Switches of the launch paths, by name (the environment variable that sets the same switch when the kernels are loaded):
  * "group_m" (FE_FP4_GROUP), "gemv" 0/1 (FE_FP4_NO_GEMV), "gemv_sk" (FE_FP4_GEMV_SK; 0 = automatic), "gemv_strips" 0/1/2 (FE_FP4_NO_STRIPS: the GEMV over strips of 16
- * weight rows never / where it pays / wherever it fits), "gemv_waves" (FE_FP4_GEMV_WAVES: wavefronts of a strip's workgroup; 0 = automatic), "xcd" -1/0/1
+ * weight rows never / where it pays / wherever it fits), "gemv_once" 0/1 (FE_FP4_NO_ONCE: the strips kernel that issues all of a workgroup's loads
+ * before it waits, where a wavefront's share of K is short enough; same bits), "gemv_waves" (FE_FP4_GEMV_WAVES: wavefronts of a strip's workgroup; 0 = automatic), "xcd" -1/0/1
  * (FE_FP4_XCD), "fp8_f16" 0/1 (FE_FP8_F16), "gemm_splits" (FE_GEMM_SPLITS), "gemm_sk" 0..3 (FE_GEMM_SK: the stream-K schedule of the
  * GEMM never / where it is the faster one / over all tiles / whole rounds then runs, the last two for tests). forward() reads no environment variable. No
  * counterpart in the reference (its FE_FP4_GROUP is read at load too, crates/fe-fp4/src/lib.rs:31-32, 68). */

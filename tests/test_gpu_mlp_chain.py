@@ -180,3 +180,34 @@ def test_cases_the_one_launch_does_not_take_fall_back():
     _, other = make(exl3, synth, kern, 512, 1536, 3, 6)
     ws2 = exl3.Workspace(lins + other, 1)
     assert exl3.mlp_forward_launches(lins[0], lins[1], other[2], 1, exl3.Dtype.Bf16, ws2) == 0  # widths differ
+
+
+def test_a_row_has_the_same_bits_at_every_row_count():
+    """The call partitions down as the one launch does at every row count it sends through the GEMV (1..64), whatever
+    plan the linear has of its own: row r of a batch has the bits of the single-row call, with the one launch on or off
+    (crates/fe-exl3/src/bin/exl3-rowcheck.rs:69-95, for the block)."""
+    import torch
+    from ferrite_amd import exl3, synth
+    kern = exl3.Kernels.load()
+    hidden, inter, bits = 512, 2048, 4
+    ts = [synth.exl3_tensor(hidden, inter, bits, 31, "gate"), synth.exl3_tensor(hidden, inter, bits, 32, "up"),
+          synth.exl3_tensor(inter, hidden, bits, 33, "down")]
+    blocks = exl3.default_blocks(exl3.cu_count())
+    lins = [exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(t), blocks) for t in ts[:2]]
+    # down with a partition of its own that is not the one launch's: 6 programs over its 64 units (runs of 10 and 11)
+    lins.append(exl3.Linear.with_plan(kern, exl3.DeviceExl3.upload_strips(ts[2]), exl3.Plan(6, 1, 4, 4)))
+    ws = exl3.Workspace(lins, 24)
+    xb = synth.activations(24, hidden, 8)
+    single = []
+    for r in range(24):
+        single.append(run(torch, exl3, lins, dev_u16(torch, xb[r:r + 1]), 1, exl3.Dtype.Bf16, ws)[2].clone())
+    assert exl3.mlp_forward_launches(*lins, 1, exl3.Dtype.Bf16, ws) == 1
+    for chain in (1, 0):
+        kern.set_option("mlp_chain", chain)
+        for m in (1, 2, 3, 8, 17, 24):
+            y = run(torch, exl3, lins, dev_u16(torch, xb[:m]), m, exl3.Dtype.Bf16, ws)[2]
+            torch.cuda.synchronize()
+            for r in range(m):
+                assert torch.equal(y[r], single[r][0]), (chain, m, r)
+    kern.set_option("mlp_chain", 1)
+    assert ws.chain_status() == 0
