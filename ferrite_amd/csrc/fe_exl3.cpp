@@ -561,6 +561,11 @@ static int launch_gemm(const fe_exl3_linear *l, fe_stream_t s, fe_devptr_t xh, f
 // The GEMV can rotate its own input: every program rotates the channels of its own run, (row, 128-channel block) pairs,
 // 8 at a time, so every column block repeats the rotation of its K range. Measured on 5120 x 17408: one launch wins up
 // to a few rows, the separate rotation launch from about 8 rows on.
+static uint32_t units_per_program(const fe_exl3_linear *l, uint32_t programs) {
+    const uint32_t units = (l->k / 128) * (l->n / 128);
+    return (units + programs - 1) / programs;
+}
+
 static bool fused_rotation_fits(const fe_exl3_linear *l, uint32_t rows) {
     const fe_exl3_options &o = l->kern->opt;
     if (!o.fused_rot || rows < 1 || rows > kMaxRowsPerPass) return false;
@@ -595,7 +600,8 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     for (size_t i = 0; i < count; i++) occ = std::max(occ, ls[i]->plan.occ), total += ls[i]->programs;
     const uint32_t places = std::max(1u, (occ ? occ : 4) * std::max(kern->cus, 1u));
     // (measured on gate + up, 4 bits: 34.1 against 35.6 us at 1 row, 36.8 / 38.2 at 4, even at 8, 44.8 / 41.9 at 16, where the
-    // longer run's inputs no longer fit the staging buffer in one piece: up to 4 rows)
+    // longer run's inputs no longer fit the staging buffer in one piece: up to 4 rows; 4-unit programs of 17408 x 5120 sharing a
+    // workgroup at 8 / 16 rows: 61.6 / 77.1 us a block against 65.2 / 75.8 without)
     uint32_t fuse = kern->opt.fuse && rows <= 4 ? std::min(4u, std::max(1u, (total + places - 1) / places)) : 1;
     uint32_t programs = 0, run_steps = 0;  // (programs: workgroups of the launch)
     size_t z_at = 0, cnt_at = 0;
@@ -841,10 +847,7 @@ static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, uint32_
     m.inv_base = 0xffffffffu / m.base, m.inv_base1 = 0xffffffffu / (m.base + 1);
 }
 
-static uint32_t units_per_program(const fe_exl3_linear *l, uint32_t programs) {
-    const uint32_t units = (l->k / 128) * (l->n / 128);
-    return (units + programs - 1) / programs;
-}
+
 
 // Whether the decode MLP gate, up -> SwiGLU -> down runs as one launch: trellis linears of one width, gate and up of one
 // shape whose outputs are down's input, every stage rotating its own input at this row count, a run of the down stage
