@@ -719,7 +719,7 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
             if (tid == 0) __hip_atomic_store(ch.ready + fnb * FE_CHAIN_STRIDE, chain_target, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #ifdef FE_GEMV_STAMPS
             if (tid == 0 && stamp_at)
-                ((unsigned long long*)(stamp_base + 65536))[8192 * 12 + (ch.ready - (ch.state + FE_CHAIN_STRIDE)) / FE_CHAIN_STRIDE + fnb] = __builtin_amdgcn_s_memrealtime();
+                ((unsigned long long*)(stamp_base + 65536))[16384 * 12 + (ch.ready - (ch.state + FE_CHAIN_STRIDE)) / FE_CHAIN_STRIDE + fnb] = __builtin_amdgcn_s_memrealtime();
 #endif
         } else if constexpr (CHAIN == 2) {
             if (tid == 0) {
