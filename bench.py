@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
 # `bench.py --traffic-pass`: KiB fetched x 2.0 (the factor that makes the counter read a streaming read and an
 # elementwise update of known size correctly) + KiB written x 1.0
-ROOFLINE_TRAFFIC_BYTES = int((69116 * 2.0 + 1632 * 1.0) * 1024)
+ROOFLINE_TRAFFIC_BYTES = int((70226 * 2.0 + 1993 * 1.0) * 1024)
 ROOFLINE_TRAFFIC_SOURCE = "profiles/exl3_mlp_b4_m1_hbm_traffic.md (rocprofv3 --pmc, not measured by this run)"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA peak of MI355X
@@ -816,8 +816,20 @@ def prefill(torch, np, exl3, fp4, synth, kern, ev, stream, m=2048, k=5120, n=174
         at[0] += 1
 
     us = ev.loop_us(stream, gemv1, 4 * len(copies))
+
+    def gemv1_on(s):
+        copies[at[0] % len(copies)].gemm(fk, fws, yf, n, 1, stream=s)
+        at[0] += 1
+
+    at[0] = 0
+    from ferrite_amd import _lib
+    us_graph = graph_us(_lib.lib(), _lib.check, ev, gemv1_on, 2 * len(copies))
     res["nvfp4_5120x17408_m1"] = {"gemv_us": round(us, 2), "GB/s": round(wbytes / us / 1e3, 1),
-                                  "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4), "weight_copies_cycled": len(copies)}
+                                  "frac_hbm_peak": round(wbytes / us / 1e3 / HBM_PEAK_GBS, 4),
+                                  # (the same launches replayed from a graph: the launch period without the eager loop's gaps)
+                                  "graph_replay_us": round(us_graph, 2),
+                                  "graph_replay_frac_hbm_peak": round(wbytes / us_graph / 1e3 / HBM_PEAK_GBS, 4),
+                                  "weight_copies_cycled": len(copies)}
     del copies, flin, yf, host1
     # the layer's other prefill shape, down (17408 x 5120): the same two GEMMs
     kd, nd = n, k
