@@ -281,8 +281,9 @@ def test_fp4_gemv_over_strips_agrees_with_the_weight_tiles(env, oracle, n, k):
             xd = dev_u16(torch, xb)
             res = dev_u16(torch, bf16_bits(np.random.default_rng(m).normal(size=(m + 1, n)).astype(np.float32)))
 
-            def run(l, strips, r=None):
+            def run(l, strips, r=None, once=1):
                 kern.set_option("gemv_strips", strips)
+                kern.set_option("gemv_once", once)  # (1: every load of a workgroup issued at once, where K allows)
                 y = torch.full((m + 1, n), -3.0, dtype=torch.bfloat16, device="cuda")
                 l.forward(kern, ws, y, n, xd, k, m, res=r)
                 torch.cuda.synchronize()
@@ -294,6 +295,8 @@ def test_fp4_gemv_over_strips_agrees_with_the_weight_tiles(env, oracle, n, k):
             assert np.array_equal(strips, run(lin, 2)) and np.array_equal(strips, run(view, 2))
             a, b = bf16_to_f32(strips).astype(np.float64), bf16_to_f32(tiles).astype(np.float64)
             assert (np.abs(a - b) <= np.abs(b) / 128.0 + 1e-30).all(), m
+            looped = bf16_to_f32(run(lin, 2, once=0)).astype(np.float64)  # the looped form: other wavefront counts, other order
+            assert (np.abs(looped - b) <= np.abs(b) / 128.0 + 1e-30).all(), m
             with_res = run(lin, 2, res)
             assert np.array_equal(with_res, bf16_bits(bf16_to_f32(strips) + bf16_to_f32(res.cpu().numpy().view(np.uint16)[:m])))
             codes, sf = oracle.quant_fp4(xb, host.g)
@@ -301,6 +304,7 @@ def test_fp4_gemv_over_strips_agrees_with_the_weight_tiles(env, oracle, n, k):
             assert (np.abs(a - ref) / np.abs(ref).max(axis=1, keepdims=True)).max() < 8e-3, m
     finally:
         kern.set_option("gemv_strips", 1)
+        kern.set_option("gemv_once", 1)
 
 
 def test_quantizer_on_special_values(env, oracle):

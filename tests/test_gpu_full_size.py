@@ -187,6 +187,71 @@ def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
     assert torch.equal(first[16][2][:1].view(torch.int16), first[1][2].view(torch.int16))
 
 
+@pytest.mark.parametrize("bits", [3, 4, 5])
+def test_exl3_decode_mlp_in_one_launch_at_full_size(env, oracle, bits):
+    """The decode MLP block of the benchmark (gate, up 5120 x 17408, down 17408 x 5120) through fe_exl3_mlp_forward: gate's
+    and up's outputs have the bits of their grouped launch (checked against the reference above); down is checked
+    against H(xh . W_hat) * svh / sqrt(128) over the activation the GPU formed, SwiGLU restated in numpy on gate's and
+    up's bf16 outputs and rotated by the oracle; the one launch and its two-launch form agree bit for bit at 1..16 rows,
+    and row r of every batch has the bits of the single-row call."""
+    torch, exl3, kern = env
+    from ferrite_amd import synth
+    blocks = exl3.default_blocks(exl3.cu_count())
+    g, u = (exl3.Linear.new(kern, exl3.DeviceExl3.upload_strips(synth.exl3_tensor(5120, 17408, bits, 70 + i, nm)), blocks)
+            for i, nm in enumerate(("gate", "up")))
+    down = Layer(env, oracle, 17408, 5120, bits, 72)
+    lins = [g, u, down.lin]
+    ws = exl3.Workspace(lins, 16)
+    xd = dev_u16(torch, synth.activations(16, 5120, 4))
+
+    def run(m, x=None):
+        yg, yu = (torch.zeros((m, 17408), dtype=torch.bfloat16, device="cuda") for _ in range(2))
+        y = torch.zeros((m, 5120), dtype=torch.float32, device="cuda")
+        exl3.mlp_forward(g, u, down.lin, xd[:m] if x is None else x, exl3.Dtype.Bf16, yg, yu, y, exl3.Dtype.F32, m, ws)
+        torch.cuda.synchronize()
+        return yg, yu, y
+
+    try:
+        assert exl3.mlp_forward_launches(g, u, down.lin, 1, exl3.Dtype.F32, ws) == 1
+        one = {m: run(m) for m in (1, 3, 8, 16)}
+        kern.set_option("mlp_chain", 0)
+        for m, got in one.items():
+            assert exl3.mlp_forward_launches(g, u, down.lin, m, exl3.Dtype.F32, ws) == 0
+            for a, b in zip(got, run(m)):
+                assert torch.equal(a, b), m
+        kern.set_option("mlp_chain", 1)
+        # gate and up: the grouped launch's bits
+        want = [torch.zeros((3, 17408), dtype=torch.bfloat16, device="cuda") for _ in range(2)]
+        exl3.forward_group([g, u], xd[:3], exl3.Dtype.Bf16, want, exl3.Dtype.Bf16, 3, ws)
+        torch.cuda.synchronize()
+        assert torch.equal(one[3][0], want[0]) and torch.equal(one[3][1], want[1])
+        # rows of a batch against the single-row call
+        for r in (0, 2, 7, 15):
+            single = run(1, xd[r:r + 1])
+            for m in (3, 8, 16):
+                if r < m:
+                    assert all(torch.equal(a[r], b[0]) for a, b in zip(one[m], single)), (m, r)
+        # down against the reference over the activation the GPU formed
+        yg, yu, y = one[3]
+        f64 = lambda t: (t.view(torch.int16).cpu().numpy().view(np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        def bf16r(a):
+            w = np.ascontiguousarray(a, np.float32).view(np.uint32)
+            return (((w + 0x7FFF + ((w >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32).astype(np.float64)
+        gq, uq = f64(yg), f64(yu)
+        act = bf16r(bf16r(gq / (1.0 + np.exp(-gq))) * uq)
+        o = oracle.Exl3(down.t.k, down.t.n, down.t.bits, down.t.trellis, down.t.suh, down.t.svh)
+        xh = oracle.rotate_input_ref(o, act)  # fp16 bits [m][k]
+        ref = down.reference(torch, torch.from_numpy(np.ascontiguousarray(xh).view(np.int16)).cuda().view(torch.float16), torch.float64)
+        got = y.cpu().numpy().astype(np.float64)
+        rms = np.sqrt((ref ** 2).mean())
+        # (the GPU's exponential is the hardware's approximate one: an activation can land on the other side of a bf16
+        # tie, which moves an output by about 1e-3 of the rms; the stage-wise bound of the plain linear is 1e-4)
+        assert np.abs(got - ref).max() / rms < 5e-3
+        assert ws.chain_status() == 0
+    finally:
+        kern.set_option("mlp_chain", 1)
+
+
 @pytest.mark.parametrize("shape", ["gate_up", "down"])
 @pytest.mark.parametrize("m", [128, 300, 512, 1024, 2048, 3072])
 def test_exl3_prefill_at_full_size(env, oracle, shape, m):
