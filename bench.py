@@ -11,7 +11,7 @@ programs of down follow those of gate and up in the grid and wait for the column
 trellis bytes streamed per second (the reference's numerator, crates/fe-exl3/src/bin/exl3-bench.rs:104) over the whole
 step, launch gaps and input rotations included. The nine weight sets total 401 MB, more than L2 plus the 256 MB Infinity
 Cache, so every step streams its weights from HBM. `separate_launches` is the same nine linears launched as six kernels
-(gate + up grouped, then down on an input of its own), the step of the earlier rounds of this bench.
+(gate + up grouped, then down on an input of its own), the step of earlier versions of this bench.
 
 `roofline` is the dominant kernel alone (exl3_mlp_b4, the three 4-bit projections in one launch): its trellis bytes
 over its average launch duration, measured with HIP event pairs on the launch stream in a second pass of the same K
@@ -227,7 +227,7 @@ def main():
     total_bytes = sum(l[2].weight_bytes() for l in linears)
 
     # The step's launches. Headline: per bit width one call of fe_exl3_mlp_forward, down on SwiGLU(gate(x), up(x)): one
-    # kernel launch each. Beside it the step of this bench's earlier rounds: gate + up of one input as a grouped call, then
+    # kernel launch each. Beside it the step of earlier versions of this bench: gate + up of one input as a grouped call, then
     # down on an input of its own, six launches. Every argument of the calls into the C ABI is prepared once.
     f_group, f_forward, f_rotate, f_rotated, f_record, f_mlp = (lib.fe_exl3_linear_forward_group, lib.fe_exl3_linear_forward,
                                                                lib.fe_exl3_linear_rotate_input, lib.fe_exl3_linear_gemv_rotated,
@@ -349,7 +349,7 @@ def main():
                                        "achieved": round(achieved, 2), "frac": round(achieved / HBM_PEAK_GBS, 4)},
                           "per_launch": per}))
         return
-    # the six-launch step of the earlier rounds, measured the same way
+    # the six-launch step of earlier versions, measured the same way
     sep = measure(separate) if one_launch_mlp else head
     sep_value = total_bytes / (sep["dt"] / args.steps) / 1e9
     sep_dom_us = sum(sep["dom_ms"]) / len(sep["dom_ms"]) * 1e3
@@ -447,8 +447,8 @@ def main():
                                f"untimed steps ({args.ramp_ms:g} ms) that bring the GPU to the clocks it holds in a decode loop"},
         "separate_launches": {"value": round(sep_value, 2), "unit": "GB/s", "ms_per_step": round(sep["dt"] * 1e3 / args.steps, 5),
                               "kernel_launches_per_step": sum(la[3] for la in separate), "per_launch": sep["per"],
-                              "what": "gate + up as one grouped launch, then down on an input of its own: the step of this bench's "
-                                      "earlier rounds"},
+                              "what": "gate + up as one grouped launch, then down on an input of its own: the step of earlier "
+                                      "versions of this bench"},
     }
 
     out["graph_replay"] = graph_replay(lib, _lib.check, ev, launches, stream, total_bytes, args.steps, args.warmup, ramp_steps)
