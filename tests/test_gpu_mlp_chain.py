@@ -211,3 +211,35 @@ def test_a_row_has_the_same_bits_at_every_row_count():
                 assert torch.equal(y[r], single[r][0]), (chain, m, r)
     kern.set_option("mlp_chain", 1)
     assert ws.chain_status() == 0
+
+
+@pytest.mark.parametrize("option,value", [("fuse", 0), ("lds_pad", 0), ("chain_perm", 0), ("chain_down_units", 0),
+                                          ("chain_down_units", 2), ("chain_down_units", 8), ("chain_rot_pairs", 8)])
+def test_switches_of_the_launch_change_no_bit(option, value):
+    """Every switch of the one launch (programs sharing a workgroup, the LDS request that sets the programs a CU, the order
+    of the down stage, the length of down's programs, the rows it takes) against the same call with the one launch off:
+    the same bits, whatever the launch looks like. The workspace is made after the switch is set, as the size of down's
+    partition asks."""
+    import torch
+    from ferrite_amd import exl3, synth
+    kern = exl3.Kernels.load()
+    defaults = {"fuse": 1, "lds_pad": 1, "chain_perm": 1, "chain_down_units": 4, "chain_rot_pairs": 32}
+    try:
+        kern.set_option(option, value)
+        _, lins = make(exl3, synth, kern, 1024, 4096, 4, 90)
+        for rows in (1, 2):
+            ws = exl3.Workspace(lins, rows)
+            x = dev_u16(torch, synth.activations(rows, 1024, 3))
+            kern.set_option("mlp_chain", 0)
+            want = [t.clone() for t in run(torch, exl3, lins, x, rows, exl3.Dtype.Bf16, ws)]
+            kern.set_option("mlp_chain", 1)
+            one = exl3.mlp_forward_launches(*lins, rows, exl3.Dtype.Bf16, ws)
+            for rep in range(2):
+                got = run(torch, exl3, lins, x, rows, exl3.Dtype.Bf16, ws)
+                torch.cuda.synchronize()
+                for a, b in zip(got, want):
+                    assert torch.equal(a, b), (option, value, rows, one, rep)
+            assert ws.chain_status() == 0
+    finally:
+        kern.set_option(option, defaults[option])
+        kern.set_option("mlp_chain", 1)
