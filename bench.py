@@ -43,7 +43,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes of one launch of the roofline kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE over
 # `bench.py --traffic-pass`: KiB fetched x 2.0 (the factor that makes the counter read a streaming read and an
 # elementwise update of known size correctly) + KiB written x 1.0
-ROOFLINE_TRAFFIC_BYTES = int((70226 * 2.0 + 1993 * 1.0) * 1024)
+ROOFLINE_TRAFFIC_BYTES = int((69125 * 2.0 + 1632 * 1.0) * 1024)
 ROOFLINE_TRAFFIC_SOURCE = "profiles/exl3_mlp_b4_m1_hbm_traffic.md (rocprofv3 --pmc, not measured by this run)"
 MFMA_F16_PEAK_TFLOPS = 2500.0
 MFMA_FP8_PEAK_TFLOPS = 5000.0  # dense fp8 MFMA peak of MI355X

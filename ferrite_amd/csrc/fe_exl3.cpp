@@ -52,7 +52,10 @@ struct fe_exl3_options {
     uint32_t gemm_group_m = 8;     // raster group of the prefill GEMM (FE_EXL3_GROUP)
     uint32_t gemm_splits = 8;      // most pieces a cut output tile of the prefill GEMM takes (FE_GEMM_SPLITS; 1: never cut)
     uint32_t gemm_sk = 1;          // stream-K schedule of the prefill GEMM: 0 never, 1 where measured faster, 2 always (FE_GEMM_SK)
-    uint32_t chain_down_units = 4; // the one-launch MLP's down stage in programs of this many units where that divides a column block (0: the linear's own partition; FE_EXL3_CHAIN_DOWN_UNITS)
+    // fe_exl3_mlp_forward runs down in programs of this many units where that divides a column block: 0 (the default) the
+    // linear's own partition; 2, 4, 8 shorter programs, which end the one launch sooner at one row and cost the two-launch
+    // form of the call time from 8 rows on (FE_EXL3_CHAIN_DOWN_UNITS)
+    uint32_t chain_down_units = 0;
     uint32_t handoff_fenced = 0;   // 1..16 rows through the kernels whose hand-off uses release / acquire fences (a slow cross-check)
     uint32_t mlp_chain = 1;        // the decode MLP (gate, up, down) as one launch where it applies (FE_EXL3_NO_CHAIN=1: off)
     uint32_t chain_rot_pairs = 32; // (row, 128-channel block) pairs a program rotates at most inside the one-launch MLP (FE_EXL3_CHAIN_ROT_PAIRS)

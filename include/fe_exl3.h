@@ -136,13 +136,13 @@ int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_
 /* The decode MLP block in one launch: yg = x @ W_gate, yu = x @ W_up (bf16 [rows][n]), y (+)= SwiGLU(yg, yu) @ W_down.
  * Whenever the one launch does not apply the call is fe_exl3_linear_forward_group on {gate, up} followed by
  * fe_exl3_linear_forward_swiglu on down (two launches), with the same bits: a row's result does not depend on the row
- * count of the call (1..64 rows). In this call down is partitioned into programs of "chain_down_units" (4) units of 128
- * channels x 128 columns where that divides its column blocks (0, or where it does not: the linear's own plan), at every
- * row count the GEMV takes; gate's and up's bits are those of their own forward, and down's are those of its own forward
- * only where the two partitions coincide. Short programs end the one launch sooner (5120 x 17408 MLP, 4 bits, 1 row:
- * 45.5 against 46.4 us) and cost the two-launch form time at 8 rows and more (8 / 16 / 64 rows: 65 / 76 / 184 us a
- * block against 60 / 69 / 161): set "chain_down_units" 0 (FE_EXL3_CHAIN_DOWN_UNITS=0, before the workspace is made)
- * where those batches matter more than the single row. This is the MLP block of a decode row
+ * count of the call (1..64 rows), and every output has the bits of the linear's own forward. Option "chain_down_units"
+ * (FE_EXL3_CHAIN_DOWN_UNITS; 2, 4 or 8; default 0 = off; set before the workspace is made) partitions down, in this call
+ * only, into programs of that many units of 128 channels x 128 columns where that divides its column blocks, at every row
+ * count the GEMV takes, so that rows still do not depend on the batch; down's bits are then its own forward's only where
+ * the two partitions coincide. Short programs end the one launch sooner at one row (5120 x 17408 MLP, 4 units: 45.5
+ * against 46.4 us at 4 bits, 53.2 against 55.7 at 5) and cost the two-launch form of the call from 8 rows on (4 bits, 8 /
+ * 16 / 64 rows: 65 / 76 / 184 us a block against 60 / 69 / 161): for deployments that only ever decode single rows. This is the MLP block of a decode row
  * (crates/fe-model/src/model.rs:3184-3199), where the reference launches seven kernels; the entry point has no
  * counterpart there. In the one launch the programs of the down projection follow those of gate and up in the grid:
  * they request their first weights at once, wait until the column blocks of gate and up that hold their input channels
@@ -151,7 +151,7 @@ int fe_exl3_linear_forward_group_launches(const fe_exl3_linear *const *ls, size_
  * under the first. The wait is bounded ("chain_spin" polls, about a microsecond each): when it runs out the program sets
  * the workspace's chain error word and goes on, the launch still ends normally, and its results are void;
  * fe_exl3_workspace_chain_status reports and clears that. It applies where every program rotates at most
- * "chain_rot_pairs" (32) pairs of (row, 128-channel block) of its own input (up to 5 rows on a 5120 x 17408 MLP), with the
+ * "chain_rot_pairs" (32) pairs of (row, 128-channel block) of its own input (up to 4 rows on a 5120 x 17408 MLP), with the
  * same width, gate and up of one shape, and a workspace created from (at least) these three linears; "mlp_chain" 0
  * (FE_EXL3_NO_CHAIN=1) turns it off.
  * fe_exl3_mlp_forward_launches: 1 if the call is the one launch, else 0. */

@@ -187,8 +187,8 @@ def test_exl3_decode_mlp_back_to_back_is_deterministic(env):
     assert torch.equal(first[16][2][:1].view(torch.int16), first[1][2].view(torch.int16))
 
 
-@pytest.mark.parametrize("bits", [3, 4, 5])
-def test_exl3_decode_mlp_in_one_launch_at_full_size(env, oracle, bits):
+@pytest.mark.parametrize("bits,down_units", [(3, 0), (4, 0), (5, 0), (4, 4), (5, 8)])
+def test_exl3_decode_mlp_in_one_launch_at_full_size(env, oracle, bits, down_units):
     """The decode MLP block of the benchmark (gate, up 5120 x 17408, down 17408 x 5120) through fe_exl3_mlp_forward: gate's
     and up's outputs have the bits of their grouped launch (checked against the reference above); down is checked
     against H(xh . W_hat) * svh / sqrt(128) over the activation the GPU formed, SwiGLU restated in numpy on gate's and
@@ -201,6 +201,7 @@ def test_exl3_decode_mlp_in_one_launch_at_full_size(env, oracle, bits):
             for i, nm in enumerate(("gate", "up")))
     down = Layer(env, oracle, 17408, 5120, bits, 72)
     lins = [g, u, down.lin]
+    kern.set_option("chain_down_units", down_units)  # (down in its own partition, or in shorter programs; before the workspace)
     ws = exl3.Workspace(lins, 16)
     xd = dev_u16(torch, synth.activations(16, 5120, 4))
 
@@ -250,6 +251,7 @@ def test_exl3_decode_mlp_in_one_launch_at_full_size(env, oracle, bits):
         assert ws.chain_status() == 0
     finally:
         kern.set_option("mlp_chain", 1)
+        kern.set_option("chain_down_units", 0)
 
 
 @pytest.mark.parametrize("shape", ["gate_up", "down"])

@@ -182,13 +182,16 @@ def test_cases_the_one_launch_does_not_take_fall_back():
     assert exl3.mlp_forward_launches(lins[0], lins[1], other[2], 1, exl3.Dtype.Bf16, ws2) == 0  # widths differ
 
 
-def test_a_row_has_the_same_bits_at_every_row_count():
-    """The call partitions down as the one launch does at every row count it sends through the GEMV (1..64), whatever
-    plan the linear has of its own: row r of a batch has the bits of the single-row call, with the one launch on or off
-    (crates/fe-exl3/src/bin/exl3-rowcheck.rs:69-95, for the block)."""
+@pytest.mark.parametrize("down_units", [0, 4])
+def test_a_row_has_the_same_bits_at_every_row_count(down_units):
+    """Row r of a batch has the bits of the single-row call, with the one launch on or off
+    (crates/fe-exl3/src/bin/exl3-rowcheck.rs:69-95, for the block): with down in its own partition (chain_down_units 0),
+    and with down in programs of 4 units, where the call keeps that partition at every row count it sends through the
+    GEMV, whatever plan the linear has of its own."""
     import torch
     from ferrite_amd import exl3, synth
     kern = exl3.Kernels.load()
+    kern.set_option("chain_down_units", down_units)  # (before the workspace is made)
     hidden, inter, bits = 512, 2048, 4
     ts = [synth.exl3_tensor(hidden, inter, bits, 31, "gate"), synth.exl3_tensor(hidden, inter, bits, 32, "up"),
           synth.exl3_tensor(inter, hidden, bits, 33, "down")]
@@ -210,11 +213,12 @@ def test_a_row_has_the_same_bits_at_every_row_count():
             for r in range(m):
                 assert torch.equal(y[r], single[r][0]), (chain, m, r)
     kern.set_option("mlp_chain", 1)
+    kern.set_option("chain_down_units", 0)
     assert ws.chain_status() == 0
 
 
-@pytest.mark.parametrize("option,value", [("fuse", 0), ("lds_pad", 0), ("chain_perm", 0), ("chain_down_units", 0),
-                                          ("chain_down_units", 2), ("chain_down_units", 8), ("chain_rot_pairs", 8)])
+@pytest.mark.parametrize("option,value", [("fuse", 0), ("lds_pad", 0), ("chain_perm", 0), ("chain_down_units", 2),
+                                          ("chain_down_units", 4), ("chain_down_units", 8), ("chain_rot_pairs", 8)])
 def test_switches_of_the_launch_change_no_bit(option, value):
     """Every switch of the one launch (programs sharing a workgroup, the LDS request that sets the programs a CU, the order
     of the down stage, the length of down's programs, the rows it takes) against the same call with the one launch off:
@@ -223,7 +227,7 @@ def test_switches_of_the_launch_change_no_bit(option, value):
     import torch
     from ferrite_amd import exl3, synth
     kern = exl3.Kernels.load()
-    defaults = {"fuse": 1, "lds_pad": 1, "chain_perm": 1, "chain_down_units": 4, "chain_rot_pairs": 32}
+    defaults = {"fuse": 1, "lds_pad": 1, "chain_perm": 1, "chain_down_units": 0, "chain_rot_pairs": 32}
     try:
         kern.set_option(option, value)
         _, lins = make(exl3, synth, kern, 1024, 4096, 4, 90)
