@@ -107,6 +107,7 @@ struct fe_exl3_workspace {
     FeBuf hat;                    // decoded fp16 weights of one linear (workspaces of hat_rows rows or more)
     FeBuf chain;                  // state of the one-launch MLP: sequence, error, finished blocks, ready words (u32)
     size_t z_len = 0, counters_len = 0, chain_len = 0;
+    bool chain_off = false;  // a bounded wait of the one-launch MLP ran out on this workspace: its calls are two launches from then on
 };
 
 int fe_load_module(fe_module_t *out, const char *env, const unsigned char *begin, const unsigned char *end) {
@@ -857,7 +858,7 @@ static void fill_member(GemvJobArgs::Member &m, const fe_exl3_linear *l, uint32_
 // within the 32 units a wavefront watches, and a workspace with room for the three side by side.
 static bool mlp_chain_fits(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe_exl3_linear *d, uint32_t rows,
                            const fe_exl3_workspace *ws, int y_dtype) {
-    if (!g || !u || !d || !ws || !g->kern->opt.mlp_chain || g->kern->opt.handoff_fenced) return false;
+    if (!g || !u || !d || !ws || ws->chain_off || !g->kern->opt.mlp_chain || g->kern->opt.handoff_fenced) return false;
     if (g->kern != u->kern || g->kern != d->kern || g->bits != u->bits || g->bits != d->bits) return false;
     if (g->k != u->k || g->n != u->n || d->k != g->n) return false;
     if (rows < 1 || rows > 16 || rows > ws->max_rows || y_dtype < 0 || y_dtype > 3) return false;
@@ -961,6 +962,7 @@ int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error) {
     FE_TRY(fe_hip_memcpy_dtoh(st, ws->chain.p, sizeof st));
     *error = st[1];
     if (st[1] || st[2]) {  // a wait ran out: the ready words and the count of that launch are void
+        ws->chain_off = true;  // (workgroups were not dispatched in grid order here: no further one-launch calls on this workspace)
         FE_TRY(fe_hip_memset_d8(ws->chain.p, 0, ws->chain_len * 4, nullptr));
         FE_TRY(fe_hip_memset_d8(ws->counters.p, 0, ws->counters_len * 4, nullptr));
         FE_TRY(fe_hip_synchronize());

@@ -161,7 +161,9 @@ int fe_exl3_mlp_forward(const fe_exl3_linear *gate, const fe_exl3_linear *up, co
 int fe_exl3_mlp_forward_launches(const fe_exl3_linear *gate, const fe_exl3_linear *up, const fe_exl3_linear *down, uint32_t rows,
                                  int y_dtype, const fe_exl3_workspace *ws);
 /* Synchronizes the device and returns the chain error word of the workspace (0: every bounded wait of the one-launch MLP
- * calls so far was met), clearing it and the launch state behind it when it is set. */
+ * calls so far was met). When it is set, the results of the calls since the last check are void; the word and the launch
+ * state behind it are cleared, and fe_exl3_mlp_forward on this workspace is its two-launch form from then on (the same
+ * bits): an expired wait means that this system does not dispatch workgroups in grid order, which the one launch needs. */
 int fe_exl3_workspace_chain_status(fe_exl3_workspace *ws, uint32_t *error);
 /* forward() for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
  * harnesses that forbid hipMalloc). No counterpart in the reference, whose forward always takes a Workspace. The

@@ -153,6 +153,9 @@ def test_expired_wait_is_reported_and_every_launch_ends():
     assert ws.chain_status() != 0
     assert ws.chain_status() == 0  # cleared
     kern.set_option("chain_spin", 1 << 16)
+    # ... and this workspace takes the two launches from now on; a new workspace takes the one launch again
+    assert exl3.mlp_forward_launches(*lins, 1, exl3.Dtype.Bf16, ws) == 0
+    assert exl3.mlp_forward_launches(*lins, 1, exl3.Dtype.Bf16, exl3.Workspace(lins, 1)) == 1
     got = run(torch, exl3, lins, x, 1, exl3.Dtype.Bf16, ws)
     torch.cuda.synchronize()
     for a, b in zip(got, want):
