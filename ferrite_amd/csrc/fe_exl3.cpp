@@ -19,7 +19,10 @@ namespace {
 constexpr uint32_t kMaxRowsPerPass = 64;       // 4 row groups of 16
 constexpr uint32_t kHatRows = 3072;            // rows from which the prefill decodes once into fp16 tiles (12 output tile rows)
 constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
-constexpr uint32_t kJobLdsBudget = 76 * 1024;  // LDS of one GEMV program
+// LDS of one GEMV program (sums of a segment + staged inputs of a chunk of the run): three programs fit a CU's 160 KB. Up
+// to 16 rows a whole run fits in far less; from 17 rows on a larger budget (76 KB: longer chunks, two programs a CU) was
+// measured slower: 37.8 against 30.9 us a linear at 32 rows on 5120 x 17408, the same at 64 rows (two a CU either way)
+constexpr uint32_t kJobLdsBudget = 53 * 1024;
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
 constexpr uint32_t kCuLds = 160 * 1024;        // LDS of a CU
@@ -633,7 +636,7 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
     // staged inputs: the whole run where the LDS budget holds it for `rows` rows, else chunks of a multiple of 4 load steps
     const uint32_t red = rows * kRedPitch * 4;
-    uint32_t chunk = std::max(4u, ((kJobLdsBudget - red) / rows - 16) / 128 / 4 * 4);
+    uint32_t chunk = std::max(4u, ((std::max(kJobLdsBudget, red + rows * 528) - red) / rows - 16) / 128 / 4 * 4);
     chunk = std::min(chunk, (run_steps + 3) / 4 * 4);
     uint32_t lds = red + rows * (chunk * 128 + 16);
     // Exactly occ programs a CU: the dispatcher fills a CU as far as registers and LDS allow (5 programs) before it moves
@@ -909,7 +912,7 @@ static int launch_mlp(const fe_exl3_linear *g, const fe_exl3_linear *u, const fe
     a.inv_spb1 = 0xffffffffu / (a.k1 / 64), a.inv_spb2 = 0xffffffffu / (a.k2 / 64);
     const uint32_t red = rows * kRedPitch * 4;
     auto chunk_of = [&](uint32_t run_steps) {
-        const uint32_t c = std::max(4u, ((kJobLdsBudget - red) / rows - 16) / 128 / 4 * 4);
+        const uint32_t c = std::max(4u, ((std::max(kJobLdsBudget, red + rows * 528) - red) / rows - 16) / 128 / 4 * 4);
         return std::min(c, (run_steps + 3) / 4 * 4);
     };
     a.chunk1 = chunk_of(2 * a.fuse1 * std::max(units_per_program(g, g->programs), units_per_program(u, u->programs)));
