@@ -21,7 +21,8 @@ constexpr uint32_t kHatRows = 3072;            // rows from which the prefill de
 constexpr uint32_t kGroupMax = 4;              // FE_EXL3_GROUP_MAX: linears of one launch
 // LDS of one GEMV program (sums of a segment + staged inputs of a chunk of the run): three programs fit a CU's 160 KB. Up
 // to 16 rows a whole run fits in far less; from 17 rows on a larger budget (76 KB: longer chunks, two programs a CU) was
-// measured slower: 37.8 against 30.9 us a linear at 32 rows on 5120 x 17408, the same at 64 rows (two a CU either way)
+// measured slower: 37.8 against 30.9 us a linear at 32 rows on 5120 x 17408; at 64 rows 52.7 against 45.2 once the sums'
+// buffer holds 32 rows at a time
 constexpr uint32_t kJobLdsBudget = 53 * 1024;
 constexpr uint32_t kRedPitch = 132;            // GEMV_RED_PITCH
 constexpr uint32_t kGemmLds = 2 * (256 + 256) * 64 * 2;  // two k tiles of A and W, 256 rows each; the epilogue reuses it
@@ -635,7 +636,7 @@ static int launch_job(const fe_exl3_linear *const *ls, size_t count, fe_stream_t
     }
     for (size_t i = count; i <= kGroupMax; i++) g.first[i] = programs;
     // staged inputs: the whole run where the LDS budget holds it for `rows` rows, else chunks of a multiple of 4 load steps
-    const uint32_t red = rows * kRedPitch * 4;
+    const uint32_t red = std::min(rows, 32u) * kRedPitch * 4;  // (more than 32 rows pass through it in two halves)
     uint32_t chunk = std::max(4u, ((std::max(kJobLdsBudget, red + rows * 528) - red) / rows - 16) / 128 / 4 * 4);
     chunk = std::min(chunk, (run_steps + 3) / 4 * 4);
     uint32_t lds = red + rows * (chunk * 128 + 16);

@@ -569,8 +569,11 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
     uint32_t nb = udiv_inv(2 * u0, spb, inv_spb), st = 2 * u0 - nb * spb;  // where the run stands: column block, load step
     const uint32_t nb_run0 = nb, st_run0 = st;
 
-    float* red = (float*)lds;                                        // [m][GEMV_RED_PITCH] sums of a finished segment
-    unsigned char* xs = (unsigned char*)(red + m * GEMV_RED_PITCH);  // [m][xpitch] rotated inputs of a chunk of the run
+    // [min(m, 32)][GEMV_RED_PITCH] sums of a finished segment: more than 32 rows pass through it in two halves, so that the
+    // programs of 33..64 rows still fit three to a CU
+    float* red = (float*)lds;
+    const uint32_t red_rows = RG > 2 ? 32 : m;
+    unsigned char* xs = (unsigned char*)(red + red_rows * GEMV_RED_PITCH);  // [m][xpitch] rotated inputs of a chunk of the run
     const uint32_t xpitch = chunk * 128 + 16;
 
     const uint32_t lane_word = g * mb.stride_k + (2 * wave + tau) * tw;
@@ -735,21 +738,46 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
 
     // The segment of column block fnb that ends here: its sums meet in LDS, and then either are the block's sums (the
     // block lies in this run alone) or go to z for the program that arrives last at the block.
-    auto flush = [&](uint32_t fnb, uint32_t p) {
-        __syncthreads();  // the previous segment's readers are done with `red`
-        // rows 4 g .. 4 g + 3 of A are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32 (tile g >> 1 of
-        // its pair, n = 4 (g & 1) + i + 8 h): a lane's four sums of either half are four neighbouring columns
+    // More than 32 rows (RG > 2): the sums of rows 0..31, then of rows 32.., meet in `red`; use(row, its sums) is called for
+    // each row by the half wavefront that takes it.
+    auto through_red_halves = [&](auto use) {
         float* rp = red + 32 * wave + 16 * (g >> 1) + 4 * (g & 1);
 #pragma unroll
-        for (int rg = 0; rg < RG; rg++) {
-            uint32_t row = 16 * rg + r;  // accumulator column = input row
-            if (row < m) {
-                *(f32x4*)(rp + row * GEMV_RED_PITCH) = acc[rg][0];
-                *(f32x4*)(rp + row * GEMV_RED_PITCH + 8) = acc[rg][1];
+        for (int h = 0; h < 2; h++) {
+            __syncthreads();  // the readers before are done with `red`
+#pragma unroll
+            for (int rg = 2 * h; rg < (2 * h + 2 < RG ? 2 * h + 2 : RG); rg++) {
+                const uint32_t row = 16 * rg + r;  // accumulator column = input row
+                if (row < m) {
+                    *(f32x4*)(rp + (row - 32 * h) * GEMV_RED_PITCH) = acc[rg][0];
+                    *(f32x4*)(rp + (row - 32 * h) * GEMV_RED_PITCH + 8) = acc[rg][1];
+                }
+                acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
             }
-            acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            __syncthreads();
+            const uint32_t end = m < 32u * h + 32 ? m : 32u * h + 32;
+            for (uint32_t row = 32 * h + hw; row < end; row += 8)
+                use(row, *(const f32x4*)(red + (row - 32 * h) * GEMV_RED_PITCH + 4 * l32));
         }
-        __syncthreads();
+    };
+
+    auto flush = [&](uint32_t fnb, uint32_t p) {
+        if constexpr (RG <= 2) __syncthreads();  // the previous segment's readers are done with `red`
+        // rows 4 g .. 4 g + 3 of A are columns 16 (g >> 1) + 4 (g & 1) + 8 h .. + 3 of the wavefront's 32 (tile g >> 1 of
+        // its pair, n = 4 (g & 1) + i + 8 h): a lane's four sums of either half are four neighbouring columns
+        if constexpr (RG <= 2) {
+            float* rp = red + 32 * wave + 16 * (g >> 1) + 4 * (g & 1);
+#pragma unroll
+            for (int rg = 0; rg < RG; rg++) {
+                uint32_t row = 16 * rg + r;  // accumulator column = input row
+                if (row < m) {
+                    *(f32x4*)(rp + row * GEMV_RED_PITCH) = acc[rg][0];
+                    *(f32x4*)(rp + row * GEMV_RED_PITCH + 8) = acc[rg][1];
+                }
+                acc[rg][0] = acc[rg][1] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            }
+            __syncthreads();
+        }
         FE_STAMP(4);
         const uint32_t col0 = fnb * 128;
         // programs of the block's first and last unit
@@ -757,10 +785,17 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         const uint32_t first_prog = ua < cut ? udiv_inv(ua, base + 1, mb.inv_base1) : rem + udiv_inv(ua - cut, base, mb.inv_base);
         const uint32_t last_prog = ub < cut ? udiv_inv(ub, base + 1, mb.inv_base1) : rem + udiv_inv(ub - cut, base, mb.inv_base);
         if (first_prog == last_prog) {
-            for (uint32_t row = hw; row < m; row += 8) {
-                f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
-                float v[4] = {t[0], t[1], t[2], t[3]};
-                finish(v, col0, row);
+            if constexpr (RG > 2) {
+                through_red_halves([&](uint32_t row, f32x4 t) {
+                    float v[4] = {t[0], t[1], t[2], t[3]};
+                    finish(v, col0, row);
+                });
+            } else {
+                for (uint32_t row = hw; row < m; row += 8) {
+                    f32x4 t = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
+                    float v[4] = {t[0], t[1], t[2], t[3]};
+                    finish(v, col0, row);
+                }
             }
             block_done(fnb);
             return;
@@ -773,7 +808,10 @@ __device__ __forceinline__ void gemvb_body(const GemvMember& mb, uint32_t p0, ui
         //     after the barrier that publishes last_flag.
         // Every byte that crosses is written through and read through, so no cache write-back or invalidate is needed.
         float* zseg = mb.z + (size_t)(p + fnb) * m * 128;
-        if constexpr (FENCED) {
+        if constexpr (RG > 2) {
+            through_red_halves([&](uint32_t row, f32x4 t) { store_agent_f32x4(zseg + row * 128 + 4 * l32, t); });
+            agent_stores_wait();
+        } else if constexpr (FENCED) {
             for (uint32_t row = hw; row < m; row += 8)
                 *(f32x4*)(zseg + row * 128 + 4 * l32) = *(const f32x4*)(red + row * GEMV_RED_PITCH + 4 * l32);
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
