@@ -346,11 +346,11 @@ int fe_fp4_linear_gemm(const fe_fp4_linear *l, const fe_fp4_kernels *kern, fe_st
         const uint32_t nts = n / kTile, kts = k / 64;
         // Strips of 16 weight rows over all of K, one a workgroup, the activations staged in LDS: no hand-off between
         // programs. Every program stages all m rows of activations, so it pays where that is small beside the weights:
-        // one row, or up to four on narrow linears (measured, cold weights: 5120 x 17408 at 1 row 14.3 against 15.4 us for
+        // one or two rows, or up to four on narrow linears (measured, cold weights: 5120 x 17408 at 1 row 14.3 against 15.4 us for
         // the weight tiles with K splits, 5120 x 5120 at 1..4 rows 7.2-7.8 against 9.7-10.0; at k = 17408 the staging
         // costs more than the hand-off it saves: 17.0 against 15.8). gemv_strips 2 forces it wherever it fits.
         const bool strips_fit = k % 256 == 0 && (size_t)m * k * 2 <= 48 * 1024 && m <= 16;
-        const bool strips_pay = k <= 8192 && (m == 1 || (n <= 8192 && m <= 4));
+        const bool strips_pay = k <= 8192 && (m <= 2 || (n <= 8192 && m <= 4));  // (5120 x 17408 at 2 rows: 14.3 against 15.3 us; at 4: 16.5)
         if (kern->gemv_strips && strips_fit && (strips_pay || kern->gemv_strips == 2)) {
             const uint32_t strips = n / 16;
             uint32_t waves = 4;  // wavefronts of a workgroup: two or more a SIMD in all
